@@ -1,0 +1,76 @@
+// Operand splitting for TCEC on gfx950.
+//
+// An fp32 value v is represented by a short sum of 16-bit floats whose
+// pairwise products are exact in fp32:
+//   half        : v ~ hi + lo/2048,  hi = RN16(v), lo = RN16((v - hi) * 2048)
+//                 (reference: tcec/tcec.hpp:219-223 with tcec/detail/scale.hpp:8-20)
+//   bfloat16    : v ~ hi + lo            two bf16 terms, ~16 significand bits
+//   precision::tf32 : v ~ hi + mid + lo  three bf16 terms, ~24 significand bits
+// gfx950 has no xf32 MFMA; the reference's tf32 policy (two 11-bit terms,
+// ~22 bits, no scaling) is replaced by the three-term bf16 split, which keeps
+// fp32's exponent range and needs no scaling.
+#pragma once
+#include "../../detail/common.hpp"
+
+namespace mtk {
+namespace wmma {
+namespace tcec {
+namespace detail {
+
+template <class T> struct split_traits;
+
+template <> struct split_traits<mtk::wmma::half> {
+  using mma_tag = mtk::wmma::half; // element tag of the MFMA operand
+  using storage = _Float16;
+  static constexpr int num_terms = 2;
+  static constexpr float scale = 2048.f;
+  static WMMAE_HD void split(const float v, storage &t0, storage &t1,
+                             storage &) {
+    t0 = static_cast<storage>(v);
+    t1 = static_cast<storage>((v - static_cast<float>(t0)) * scale);
+  }
+};
+#ifdef WMMAE_HAS_HIP_FP16
+template <> struct split_traits<__half> : split_traits<mtk::wmma::half> {};
+#endif
+
+template <> struct split_traits<mtk::wmma::bfloat16> {
+  using mma_tag = mtk::wmma::bfloat16;
+  using storage = __bf16;
+  static constexpr int num_terms = 2;
+  static constexpr float scale = 1.f;
+  static WMMAE_HD void split(const float v, storage &t0, storage &t1,
+                             storage &) {
+    t0 = static_cast<storage>(v);
+    t1 = static_cast<storage>(v - static_cast<float>(t0));
+  }
+};
+
+template <> struct split_traits<mtk::wmma::precision::tf32> {
+  using mma_tag = mtk::wmma::bfloat16;
+  using storage = __bf16;
+  static constexpr int num_terms = 3;
+  static constexpr float scale = 1.f;
+  static WMMAE_HD void split(const float v, storage &t0, storage &t1,
+                             storage &t2) {
+    t0 = static_cast<storage>(v);
+    const float r1 = v - static_cast<float>(t0);
+    t1 = static_cast<storage>(r1);
+    const float r2 = r1 - static_cast<float>(t1);
+    t2 = static_cast<storage>(r2);
+  }
+};
+
+// Scale applied to the residual before rounding it (0) and removed when the
+// error accumulator is folded back (1) (reference: tcec/detail/scale.hpp:8-20).
+template <class T> WMMAE_HD float correction_scale_0(const float v) {
+  return v * split_traits<T>::scale;
+}
+template <class T> WMMAE_HD float correction_scale_1(const float v) {
+  return v / split_traits<T>::scale;
+}
+
+} // namespace detail
+} // namespace tcec
+} // namespace wmma
+} // namespace mtk

@@ -1,0 +1,594 @@
+// TCEC: error-corrected fp32 matrix multiply-accumulate on the gfx950 matrix
+// cores, with the device-side API of the reference's mtk::wmma::tcec
+// (reference: include/wmma_extension/tcec/tcec.hpp:13-927 for with_ec and
+// tcec/detail/no_cor.hpp:13-897 for without_ec; docs/mma_f32.md:59-135).
+//
+// A tcec::fragment<Use,m,n,k,T,Layout,Policy> covers an m x n x k problem with
+// a grid of MFMA sub-fragments of the policy's shape.  Sub-block (bm,bn) is
+// stored at index bm + num_sub_frag_m*bn.  matrix_a / matrix_b fragments hold
+// the split terms of their fp32 source (sub_frag = leading term, sub_d_frag =
+// residual term, sub_d2_frag = second residual of the three-term split);
+// accumulators hold an fp32 main part (sub_frag) and an fp32 error part
+// (sub_d_frag, scaled by split_traits<T>::scale).  Everything is
+// wave64-collective; `sync` arguments are accepted and ignored because a wave
+// runs in lock step.
+#pragma once
+#include "detail/policy.hpp"
+#include "detail/split.hpp"
+
+namespace mtk {
+namespace wmma {
+namespace tcec {
+
+namespace detail {
+using mtk::wmma::detail::common::select_value;
+
+template <class Layout, int a, int b> struct layout_switch;
+template <int a, int b> struct layout_switch<col_major, a, b> {
+  static constexpr int value = a;
+};
+template <int a, int b> struct layout_switch<row_major, a, b> {
+  static constexpr int value = b;
+};
+
+// Memory offset of element (i,j) of sub-block at (m_offset, n_offset)
+// (reference: tcec/detail/common.hpp:32-63).
+template <class Layout>
+WMMAE_HD unsigned mem_offset(const unsigned i, const unsigned j,
+                             const unsigned ldm, const unsigned m_offset,
+                             const unsigned n_offset) {
+  if constexpr (std::is_same<Layout, col_major>::value)
+    return (i + m_offset) + (j + n_offset) * ldm;
+  else
+    return (j + n_offset) + (i + m_offset) * ldm;
+}
+} // namespace detail
+
+template <class Use, int m, int n, int k, class T, class Layout = void,
+          class Policy_ = typename detail::default_policy<T>::type>
+struct fragment {
+  using Policy = Policy_;
+  using element_type = float;
+  using split = detail::split_traits<T>;
+  static constexpr int sub_frag_m = Policy::m;
+  static constexpr int sub_frag_n = Policy::n;
+  static constexpr int sub_frag_k = Policy::k;
+  static constexpr bool is_acc = std::is_same<Use, accumulator>::value;
+  static constexpr bool has_ec =
+      std::is_same<typename Policy::error_correction, with_ec>::value;
+
+  using sub_elem_t = typename std::conditional<is_acc, float,
+                                               typename split::mma_tag>::type;
+  using sub_frag_t =
+      typename detail::default_fragment<Use, sub_elem_t, Layout, Policy>::type;
+  using storage_t = typename sub_frag_t::storage_element_type;
+
+  static constexpr int num_sub_frag_m =
+      detail::select_value<Use, m, k, m>::value /
+      detail::select_value<Use, sub_frag_m, sub_frag_k, sub_frag_m>::value;
+  static constexpr int num_sub_frag_n =
+      detail::select_value<Use, k, n, n>::value /
+      detail::select_value<Use, sub_frag_k, sub_frag_n, sub_frag_n>::value;
+  static constexpr int num_sub_frags = num_sub_frag_m * num_sub_frag_n;
+  static_assert(num_sub_frag_m * detail::select_value<Use, sub_frag_m,
+                                                      sub_frag_k,
+                                                      sub_frag_m>::value ==
+                        detail::select_value<Use, m, k, m>::value &&
+                    num_sub_frag_n * detail::select_value<Use, sub_frag_k,
+                                                          sub_frag_n,
+                                                          sub_frag_n>::value ==
+                        detail::select_value<Use, k, n, n>::value,
+                "m, n, k must be multiples of the policy's instruction shape");
+  // number of stored parts: 1 without error correction; accumulators keep
+  // main + error; operands keep as many terms as the split produces.
+  static constexpr int num_terms =
+      !has_ec ? 1 : (is_acc ? 2 : split::num_terms);
+
+  sub_frag_t sub_frag[num_sub_frags];
+  sub_frag_t sub_d_frag[num_terms >= 2 ? num_sub_frags : 0];
+  sub_frag_t sub_d2_frag[num_terms >= 3 ? num_sub_frags : 0];
+
+  static constexpr unsigned num_elements =
+      num_sub_frags * sub_frag_t::num_elements;
+
+  WMMAE_D storage_t &x(const unsigned index) {
+    return sub_frag[index / sub_frag_t::num_elements]
+        .x[index % sub_frag_t::num_elements];
+  }
+  WMMAE_D storage_t x(const unsigned index) const {
+    return sub_frag[index / sub_frag_t::num_elements]
+        .x[index % sub_frag_t::num_elements];
+  }
+  WMMAE_D storage_t &dx(const unsigned index) {
+    return sub_d_frag[index / sub_frag_t::num_elements]
+        .x[index % sub_frag_t::num_elements];
+  }
+  WMMAE_D storage_t dx(const unsigned index) const {
+    return sub_d_frag[index / sub_frag_t::num_elements]
+        .x[index % sub_frag_t::num_elements];
+  }
+
+  // Fold the error part of an accumulator into its main part.
+  WMMAE_D void integrate() {
+    if constexpr (num_terms >= 2) {
+#pragma unroll
+      for (int f = 0; f < num_sub_frags; f++) {
+#pragma unroll
+        for (unsigned i = 0; i < sub_frag_t::num_elements; i++) {
+          sub_frag[f].x[i] += detail::correction_scale_1<T>(
+              static_cast<float>(sub_d_frag[f].x[i]));
+          sub_d_frag[f].x[i] = static_cast<storage_t>(0);
+        }
+      }
+    }
+  }
+};
+
+#define WMMAE_TCEC_TPARAMS                                                     \
+  int m, int n, int k, class T, class Op, class EC, int fm, int fn, int fk
+#define WMMAE_TCEC_FRAG(Use, Layout)                                           \
+  fragment<Use, m, n, k, T, Layout, Policy<Op, EC, fm, fn, fk>>
+
+namespace detail {
+// Write the split of v into every stored term of an operand fragment.
+template <class Frag>
+WMMAE_D void put_split(Frag &frag, const unsigned block,
+                       const unsigned frag_index, const float v) {
+  using split = typename Frag::split;
+  typename split::storage t0, t1, t2;
+  split::split(v, t0, t1, t2);
+  frag.sub_frag[block].x[frag_index] = t0;
+  if constexpr (Frag::num_terms >= 2)
+    frag.sub_d_frag[block].x[frag_index] = t1;
+  if constexpr (Frag::num_terms >= 3)
+    frag.sub_d2_frag[block].x[frag_index] = t2;
+}
+
+// Value an accumulator element stands for.
+template <class Frag>
+WMMAE_D float combined(const Frag &frag, const unsigned block,
+                       const unsigned frag_index) {
+  if constexpr (Frag::num_terms >= 2)
+    return frag.sub_frag[block].x[frag_index] +
+           frag.sub_d_frag[block].x[frag_index] / Frag::split::scale;
+  else
+    return frag.sub_frag[block].x[frag_index];
+}
+} // namespace detail
+
+// ------------------------------------------------------------ fill / neg
+template <class Use, WMMAE_TCEC_TPARAMS, class Layout, class V>
+WMMAE_D void fill_fragment(WMMAE_TCEC_FRAG(Use, Layout) & frag, const V v) {
+  using F = WMMAE_TCEC_FRAG(Use, Layout);
+#pragma unroll
+  for (int b = 0; b < F::num_sub_frags; b++) {
+    mtk::wmma::fill_fragment(frag.sub_frag[b], v);
+    if constexpr (F::num_terms >= 2)
+      mtk::wmma::fill_zero(frag.sub_d_frag[b]);
+    if constexpr (F::num_terms >= 3)
+      mtk::wmma::fill_zero(frag.sub_d2_frag[b]);
+  }
+}
+
+template <class Use, WMMAE_TCEC_TPARAMS, class Layout>
+WMMAE_D void fill_zero(WMMAE_TCEC_FRAG(Use, Layout) & frag) {
+  using F = WMMAE_TCEC_FRAG(Use, Layout);
+#pragma unroll
+  for (int b = 0; b < F::num_sub_frags; b++) {
+    mtk::wmma::fill_zero(frag.sub_frag[b]);
+    if constexpr (F::num_terms >= 2)
+      mtk::wmma::fill_zero(frag.sub_d_frag[b]);
+    if constexpr (F::num_terms >= 3)
+      mtk::wmma::fill_zero(frag.sub_d2_frag[b]);
+  }
+}
+
+template <class Use, WMMAE_TCEC_TPARAMS, class Layout>
+WMMAE_D WMMAE_TCEC_FRAG(Use, Layout)
+    neg(const WMMAE_TCEC_FRAG(Use, Layout) & frag) {
+  using F = WMMAE_TCEC_FRAG(Use, Layout);
+  F res;
+#pragma unroll
+  for (int b = 0; b < F::num_sub_frags; b++) {
+#pragma unroll
+    for (unsigned i = 0; i < F::sub_frag_t::num_elements; i++) {
+      res.sub_frag[b].x[i] = -frag.sub_frag[b].x[i];
+      if constexpr (F::num_terms >= 2)
+        res.sub_d_frag[b].x[i] = -frag.sub_d_frag[b].x[i];
+      if constexpr (F::num_terms >= 3)
+        res.sub_d2_frag[b].x[i] = -frag.sub_d2_frag[b].x[i];
+    }
+  }
+  return res;
+}
+
+// ------------------------------------------------------------ load matrix
+// MatrixLayout is the layout of the memory being read; it is independent of
+// the fragment's own Layout argument (docs/mma_f32.md:114-123).  Operands are
+// split while loading; accumulators are taken as fp32 with a zero error part.
+template <class MatrixLayout, class Use, WMMAE_TCEC_TPARAMS, class Layout,
+          class MEM_T>
+WMMAE_D void load_matrix_sync_with_mul(WMMAE_TCEC_FRAG(Use, Layout) & frag,
+                                       const MEM_T *const ptr,
+                                       const unsigned ldm, const MEM_T mul,
+                                       const bool = true) {
+  using F = WMMAE_TCEC_FRAG(Use, Layout);
+  constexpr unsigned bm_size =
+      detail::select_value<Use, fm, fk, fm>::value; // rows of one sub-block
+  constexpr unsigned bn_size = detail::select_value<Use, fk, fn, fn>::value;
+  mtk::wmma::foreach_ij<typename F::sub_frag_t>(
+      [&](const unsigned *list, const unsigned, const unsigned i,
+          const unsigned j) {
+#pragma unroll
+        for (unsigned bm = 0; bm < unsigned(F::num_sub_frag_m); bm++) {
+#pragma unroll
+          for (unsigned bn = 0; bn < unsigned(F::num_sub_frag_n); bn++) {
+            const unsigned off = detail::mem_offset<MatrixLayout>(
+                i, j, ldm, bm * bm_size, bn * bn_size);
+            const unsigned block = bm + F::num_sub_frag_m * bn;
+            const float v = static_cast<float>(ptr[off]) *
+                            static_cast<float>(mul);
+            if constexpr (F::is_acc) {
+              frag.sub_frag[block].x[list[0]] = v;
+              if constexpr (F::num_terms >= 2)
+                frag.sub_d_frag[block].x[list[0]] = 0.f;
+            } else {
+              detail::put_split(frag, block, list[0], v);
+            }
+          }
+        }
+      });
+}
+
+template <class MatrixLayout, class Use, WMMAE_TCEC_TPARAMS, class Layout,
+          class MEM_T>
+WMMAE_D void load_matrix_sync(WMMAE_TCEC_FRAG(Use, Layout) & frag,
+                              const MEM_T *const ptr, const unsigned ldm,
+                              const bool sync = true) {
+  load_matrix_sync_with_mul<MatrixLayout>(frag, ptr, ldm,
+                                          static_cast<MEM_T>(1), sync);
+}
+
+// Memory layout = the fragment's own Layout (operands only).
+template <class Use, WMMAE_TCEC_TPARAMS, class Layout, class MEM_T>
+WMMAE_D void load_matrix_sync(WMMAE_TCEC_FRAG(Use, Layout) & frag,
+                              const MEM_T *const ptr, const unsigned ldm,
+                              const bool sync = true) {
+  static_assert(!std::is_same<Use, accumulator>::value,
+                "accumulator loads need a layout");
+  load_matrix_sync<Layout>(frag, ptr, ldm, sync);
+}
+template <class Use, WMMAE_TCEC_TPARAMS, class Layout, class MEM_T>
+WMMAE_D void load_matrix_sync_with_mul(WMMAE_TCEC_FRAG(Use, Layout) & frag,
+                                       const MEM_T *const ptr,
+                                       const unsigned ldm, const MEM_T mul,
+                                       const bool sync = true) {
+  static_assert(!std::is_same<Use, accumulator>::value,
+                "accumulator loads need a layout");
+  load_matrix_sync_with_mul<Layout>(frag, ptr, ldm, mul, sync);
+}
+
+// Accumulators with a run-time layout.
+template <WMMAE_TCEC_TPARAMS, class MEM_T>
+WMMAE_D void load_matrix_sync(WMMAE_TCEC_FRAG(accumulator, void) & frag,
+                              const MEM_T *const ptr, const unsigned ldm,
+                              const layout_t layout, const bool sync = true) {
+  if (layout == mem_col_major)
+    load_matrix_sync<col_major>(frag, ptr, ldm, sync);
+  else
+    load_matrix_sync<row_major>(frag, ptr, ldm, sync);
+}
+template <WMMAE_TCEC_TPARAMS, class MEM_T>
+WMMAE_D void load_matrix_sync_with_mul(WMMAE_TCEC_FRAG(accumulator, void) &
+                                           frag,
+                                       const MEM_T *const ptr,
+                                       const unsigned ldm, const MEM_T mul,
+                                       const layout_t layout,
+                                       const bool sync = true) {
+  if (layout == mem_col_major)
+    load_matrix_sync_with_mul<col_major>(frag, ptr, ldm, mul, sync);
+  else
+    load_matrix_sync_with_mul<row_major>(frag, ptr, ldm, mul, sync);
+}
+
+// ----------------------------------------------------------- store matrix
+template <class Layout, WMMAE_TCEC_TPARAMS, class MEM_T>
+WMMAE_D void
+store_matrix_sync_with_mul(MEM_T *const ptr,
+                           const WMMAE_TCEC_FRAG(accumulator, void) & frag,
+                           const unsigned ldm, const MEM_T mul,
+                           const bool = true) {
+  using F = WMMAE_TCEC_FRAG(accumulator, void);
+  mtk::wmma::foreach_ij<typename F::sub_frag_t>(
+      [&](const unsigned *list, const unsigned, const unsigned i,
+          const unsigned j) {
+#pragma unroll
+        for (unsigned bm = 0; bm < unsigned(F::num_sub_frag_m); bm++) {
+#pragma unroll
+          for (unsigned bn = 0; bn < unsigned(F::num_sub_frag_n); bn++) {
+            const unsigned off =
+                detail::mem_offset<Layout>(i, j, ldm, bm * fm, bn * fn);
+            const unsigned block = bm + F::num_sub_frag_m * bn;
+            ptr[off] = static_cast<MEM_T>(
+                detail::combined(frag, block, list[0]) *
+                static_cast<float>(mul));
+          }
+        }
+      });
+}
+template <class Layout, WMMAE_TCEC_TPARAMS, class MEM_T>
+WMMAE_D void store_matrix_sync(MEM_T *const ptr,
+                               const WMMAE_TCEC_FRAG(accumulator, void) & frag,
+                               const unsigned ldm, const bool sync = true) {
+  store_matrix_sync_with_mul<Layout>(ptr, frag, ldm, static_cast<MEM_T>(1),
+                                     sync);
+}
+template <WMMAE_TCEC_TPARAMS, class MEM_T>
+WMMAE_D void store_matrix_sync(MEM_T *const ptr,
+                               const WMMAE_TCEC_FRAG(accumulator, void) & frag,
+                               const unsigned ldm, const layout_t layout,
+                               const bool sync = true) {
+  if (layout == mem_col_major)
+    store_matrix_sync<col_major>(ptr, frag, ldm, sync);
+  else
+    store_matrix_sync<row_major>(ptr, frag, ldm, sync);
+}
+template <WMMAE_TCEC_TPARAMS, class MEM_T>
+WMMAE_D void
+store_matrix_sync_with_mul(MEM_T *const ptr,
+                           const WMMAE_TCEC_FRAG(accumulator, void) & frag,
+                           const unsigned ldm, const MEM_T mul,
+                           const layout_t layout, const bool sync = true) {
+  if (layout == mem_col_major)
+    store_matrix_sync_with_mul<col_major>(ptr, frag, ldm, mul, sync);
+  else
+    store_matrix_sync_with_mul<row_major>(ptr, frag, ldm, mul, sync);
+}
+
+// ------------------------------------------------------------ load vector
+// Operands: the vector goes into the first column (col_major fragment) or
+// first row (row_major fragment) of the m x k / k x n tile; only the
+// sub-blocks on that edge are written, the caller zero-fills first
+// (reference: tcec/tcec.hpp:450-536; test/tcec/matvec.cu:41-42).
+template <class Use, WMMAE_TCEC_TPARAMS, class Layout, class MEM_T>
+WMMAE_D void load_vector(WMMAE_TCEC_FRAG(Use, Layout) & frag,
+                         const MEM_T *const ptr, const MEM_T mul) {
+  using F = WMMAE_TCEC_FRAG(Use, Layout);
+  static_assert(!F::is_acc, "accumulator load_vector needs a layout_t");
+  constexpr unsigned bm_size = detail::select_value<Use, fm, fk, fm>::value;
+  constexpr unsigned bn_size = detail::select_value<Use, fk, fn, fn>::value;
+  constexpr unsigned num_blocks =
+      detail::layout_switch<Layout, F::num_sub_frag_m,
+                            F::num_sub_frag_n>::value;
+  constexpr unsigned block_ld =
+      detail::layout_switch<Layout, 1, F::num_sub_frag_m>::value;
+  constexpr unsigned vec_per_block =
+      detail::layout_switch<Layout, bm_size, bn_size>::value;
+  mtk::wmma::foreach_v<typename F::sub_frag_t>(
+      [&](const unsigned *list, const unsigned, const unsigned mem_index) {
+#pragma unroll
+        for (unsigned b = 0; b < num_blocks; b++) {
+          const float v =
+              static_cast<float>(ptr[mem_index + b * vec_per_block]) *
+              static_cast<float>(mul);
+          detail::put_split(frag, b * block_ld, list[0], v);
+        }
+      });
+}
+template <class Use, WMMAE_TCEC_TPARAMS, class Layout, class MEM_T>
+WMMAE_D void load_vector(WMMAE_TCEC_FRAG(Use, Layout) & frag,
+                         const MEM_T *const ptr) {
+  load_vector(frag, ptr, static_cast<MEM_T>(1));
+}
+
+// Accumulators: first column (mem_col_major) or first row (mem_row_major).
+// The touched main sub-blocks are zeroed and then receive the vector; the
+// error part is left as it is (reference: tcec/tcec.hpp:421-448, which
+// forwards to the primitive load_vector with its default fill).
+template <WMMAE_TCEC_TPARAMS, class MEM_T>
+WMMAE_D void load_vector(WMMAE_TCEC_FRAG(accumulator, void) & frag,
+                         const MEM_T *const ptr, const layout_t layout) {
+  using F = WMMAE_TCEC_FRAG(accumulator, void);
+  if (layout == mem_col_major) {
+#pragma unroll
+    for (unsigned bm = 0; bm < unsigned(F::num_sub_frag_m); bm++)
+      mtk::wmma::load_vector(frag.sub_frag[bm], ptr + bm * fm, layout);
+  } else {
+#pragma unroll
+    for (unsigned bn = 0; bn < unsigned(F::num_sub_frag_n); bn++)
+      mtk::wmma::load_vector(frag.sub_frag[bn * F::num_sub_frag_m],
+                             ptr + bn * fn, layout);
+  }
+}
+
+// ----------------------------------------------------------- store vector
+template <WMMAE_TCEC_TPARAMS, class MEM_T>
+WMMAE_D void store_vector(MEM_T *const ptr,
+                          const WMMAE_TCEC_FRAG(accumulator, void) & frag,
+                          const MEM_T mul, const layout_t layout) {
+  using F = WMMAE_TCEC_FRAG(accumulator, void);
+  const bool col = layout == mem_col_major;
+  mtk::wmma::foreach_v<typename F::sub_frag_t>(
+      layout,
+      [&](const unsigned *list, const unsigned, const unsigned mem_index) {
+        if (col) {
+#pragma unroll
+          for (unsigned bm = 0; bm < unsigned(F::num_sub_frag_m); bm++)
+            ptr[bm * fm + mem_index] = static_cast<MEM_T>(
+                detail::combined(frag, bm, list[0]) * static_cast<float>(mul));
+        } else {
+#pragma unroll
+          for (unsigned bn = 0; bn < unsigned(F::num_sub_frag_n); bn++)
+            ptr[bn * fn + mem_index] = static_cast<MEM_T>(
+                detail::combined(frag, bn * F::num_sub_frag_m, list[0]) *
+                static_cast<float>(mul));
+        }
+      });
+}
+template <WMMAE_TCEC_TPARAMS, class MEM_T>
+WMMAE_D void store_vector(MEM_T *const ptr,
+                          const WMMAE_TCEC_FRAG(accumulator, void) & frag,
+                          const layout_t layout) {
+  store_vector(ptr, frag, static_cast<MEM_T>(1), layout);
+}
+
+// -------------------------------------------------------------------- mma
+// d = a*b + c over the sub-block grid.  With error correction the products
+//   main:  a0*b0
+//   error: a1*b0 + a0*b1                      (two-term splits)
+//          + a1*b1 + a2*b0 + a0*b2            (three-term split)
+// are issued as separate MFMAs; a1*b1 of the two-term split and the
+// higher-order products of the three-term split are below fp32 resolution
+// and dropped (reference: tcec/tcec.hpp:640-706).
+namespace detail {
+template <bool main_outside, bool use_c, WMMAE_TCEC_TPARAMS, class LA, class LB>
+WMMAE_D void mma_core(WMMAE_TCEC_FRAG(accumulator, void) & d,
+                      const WMMAE_TCEC_FRAG(matrix_a, LA) & a,
+                      const WMMAE_TCEC_FRAG(matrix_b, LB) & b,
+                      const WMMAE_TCEC_FRAG(accumulator, void) * c) {
+  using FD = WMMAE_TCEC_FRAG(accumulator, void);
+  using FA = WMMAE_TCEC_FRAG(matrix_a, LA);
+  constexpr unsigned nmb = FD::num_sub_frag_m;
+  constexpr unsigned nnb = FD::num_sub_frag_n;
+  constexpr unsigned nkb = FA::num_sub_frag_n;
+  constexpr int terms = FA::num_terms;
+#pragma unroll
+  for (unsigned bm = 0; bm < nmb; bm++) {
+#pragma unroll
+    for (unsigned bn = 0; bn < nnb; bn++) {
+      const unsigned cd = bm + bn * nmb;
+      typename FD::sub_frag_t main_acc, err_acc;
+      if constexpr (use_c) {
+        main_acc = c->sub_frag[cd];
+        if constexpr (terms >= 2)
+          err_acc = c->sub_d_frag[cd];
+      } else {
+        mtk::wmma::fill_zero(main_acc);
+        mtk::wmma::fill_zero(err_acc);
+      }
+#pragma unroll
+      for (unsigned bk = 0; bk < nkb; bk++) {
+        const unsigned ia = bm + bk * nmb;
+        const unsigned ib = bk + bn * nkb;
+        if constexpr (main_outside) {
+          // round-to-nearest variant: the main product starts from a zero
+          // accumulator and is added to the running sum with an fp32 add.
+          typename FD::sub_frag_t tmp;
+          mtk::wmma::fill_zero(tmp);
+          mtk::wmma::mma_sync(tmp, a.sub_frag[ia], b.sub_frag[ib], tmp);
+#pragma unroll
+          for (unsigned i = 0; i < tmp.num_elements; i++)
+            main_acc.x[i] += tmp.x[i];
+        } else {
+          mtk::wmma::mma_sync(main_acc, a.sub_frag[ia], b.sub_frag[ib],
+                              main_acc);
+        }
+        if constexpr (terms >= 3) {
+          mtk::wmma::mma_sync(err_acc, a.sub_d2_frag[ia], b.sub_frag[ib],
+                              err_acc);
+          mtk::wmma::mma_sync(err_acc, a.sub_frag[ia], b.sub_d2_frag[ib],
+                              err_acc);
+          mtk::wmma::mma_sync(err_acc, a.sub_d_frag[ia], b.sub_d_frag[ib],
+                              err_acc);
+        }
+        if constexpr (terms >= 2) {
+          mtk::wmma::mma_sync(err_acc, a.sub_d_frag[ia], b.sub_frag[ib],
+                              err_acc);
+          mtk::wmma::mma_sync(err_acc, a.sub_frag[ia], b.sub_d_frag[ib],
+                              err_acc);
+        }
+      }
+      d.sub_frag[cd] = main_acc;
+      if constexpr (terms >= 2)
+        d.sub_d_frag[cd] = err_acc;
+    }
+  }
+}
+} // namespace detail
+
+// mma_rn_sync: main term accumulated with fp32 adds outside the matrix core.
+template <WMMAE_TCEC_TPARAMS, class LA, class LB>
+WMMAE_D void mma_rn_sync(WMMAE_TCEC_FRAG(accumulator, void) & d,
+                         const WMMAE_TCEC_FRAG(matrix_a, LA) & a,
+                         const WMMAE_TCEC_FRAG(matrix_b, LB) & b,
+                         const WMMAE_TCEC_FRAG(accumulator, void) & c) {
+  detail::mma_core<true, true>(d, a, b, &c);
+}
+template <WMMAE_TCEC_TPARAMS, class LA, class LB>
+WMMAE_D void mma_rn_sync(WMMAE_TCEC_FRAG(accumulator, void) & d,
+                         const WMMAE_TCEC_FRAG(matrix_a, LA) & a,
+                         const WMMAE_TCEC_FRAG(matrix_b, LB) & b) {
+  detail::mma_core<true, false>(
+      d, a, b, static_cast<const WMMAE_TCEC_FRAG(accumulator, void) *>(nullptr));
+}
+// mma_rz_sync: main term chained through the matrix core's own accumulator
+// (named after the truncating accumulate of the reference's hardware).
+template <WMMAE_TCEC_TPARAMS, class LA, class LB>
+WMMAE_D void mma_rz_sync(WMMAE_TCEC_FRAG(accumulator, void) & d,
+                         const WMMAE_TCEC_FRAG(matrix_a, LA) & a,
+                         const WMMAE_TCEC_FRAG(matrix_b, LB) & b,
+                         const WMMAE_TCEC_FRAG(accumulator, void) & c) {
+  detail::mma_core<false, true>(d, a, b, &c);
+}
+template <WMMAE_TCEC_TPARAMS, class LA, class LB>
+WMMAE_D void mma_rz_sync(WMMAE_TCEC_FRAG(accumulator, void) & d,
+                         const WMMAE_TCEC_FRAG(matrix_a, LA) & a,
+                         const WMMAE_TCEC_FRAG(matrix_b, LB) & b) {
+  detail::mma_core<false, false>(
+      d, a, b, static_cast<const WMMAE_TCEC_FRAG(accumulator, void) *>(nullptr));
+}
+
+// Default: with_ec -> mma_rn_sync (tcec.hpp:896-927); without_ec ->
+// mma_rz_sync (no_cor.hpp:858-897, docs/mma_f32.md:131-135).
+template <WMMAE_TCEC_TPARAMS, class LA, class LB>
+WMMAE_D void mma_sync(WMMAE_TCEC_FRAG(accumulator, void) & d,
+                      const WMMAE_TCEC_FRAG(matrix_a, LA) & a,
+                      const WMMAE_TCEC_FRAG(matrix_b, LB) & b,
+                      const WMMAE_TCEC_FRAG(accumulator, void) & c) {
+  if constexpr (std::is_same<EC, with_ec>::value)
+    mma_rn_sync(d, a, b, c);
+  else
+    mma_rz_sync(d, a, b, c);
+}
+template <WMMAE_TCEC_TPARAMS, class LA, class LB>
+WMMAE_D void mma_sync(WMMAE_TCEC_FRAG(accumulator, void) & d,
+                      const WMMAE_TCEC_FRAG(matrix_a, LA) & a,
+                      const WMMAE_TCEC_FRAG(matrix_b, LB) & b) {
+  if constexpr (std::is_same<EC, with_ec>::value)
+    mma_rn_sync(d, a, b);
+  else
+    mma_rz_sync(d, a, b);
+}
+
+// ------------------------------------------------------------ debug print
+template <class Use, WMMAE_TCEC_TPARAMS, class Layout>
+__device__ inline void print_fragment(const WMMAE_TCEC_FRAG(Use, Layout) & frag,
+                                      const char *const name = "") {
+  using F = WMMAE_TCEC_FRAG(Use, Layout);
+  const unsigned lane = mtk::wmma::detail::common::get_lane_id();
+  if (lane == 0 && name[0] != '\0')
+    printf("%s = \n", name);
+  for (unsigned l = 0; l < wave_size; l++) {
+    if (l == lane) {
+      for (unsigned i = 0; i < F::num_elements; i++) {
+        if constexpr (F::num_terms >= 2)
+          printf("(%+.3e)+(%+.3e) ", static_cast<float>(frag.x(i)),
+                 detail::correction_scale_1<T>(static_cast<float>(frag.dx(i))));
+        else
+          printf("(%+.3e) ", static_cast<float>(frag.x(i)));
+      }
+      printf("\n");
+    }
+  }
+}
+
+#undef WMMAE_TCEC_TPARAMS
+#undef WMMAE_TCEC_FRAG
+
+} // namespace tcec
+
+// Historic name of the same API.
+namespace mma_f32 = tcec;
+
+} // namespace wmma
+} // namespace mtk

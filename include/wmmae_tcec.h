@@ -1,0 +1,190 @@
+/*
+ * C ABI of the gfx950 TCEC library (libwmmae_tcec.so).
+ *
+ * The reference (wmmae/wmma_extension) is a header-only device library; the
+ * only host-callable GEMM it contains is the launcher of its batched test
+ * kernel.  This header is the host boundary of the rebuilt hot path: a
+ * BLAS-style driver for the error-corrected SGEMM, the two stages it is made
+ * of, and entry points that run the reference's one-warp test kernels on the
+ * header-only device API (include/wmma_extension/...) so that host programs
+ * and ctypes/cgo/JNI bindings can exercise that API without a device compiler.
+ *
+ * Conventions
+ *   - every pointer named A, B, C, X, tiles, ... is a DEVICE pointer unless the
+ *     comment says host; alpha/beta are HOST pointers
+ *   - `stream` is a hipStream_t passed as void* (NULL = the default stream);
+ *     all work is asynchronous on that stream, nothing synchronises
+ *   - return value: WMMAE_STATUS_SUCCESS (0) or a negative wmmae_status
+ *   - no global state; calls may come from any thread
+ *   - matrices follow the column-major BLAS convention; the reference's layout
+ *     (A row-major m x k, B column-major k x n, C column-major m x n,
+ *     test/tcec/batch_gemm.cu:259-260, 542-543) is transa='T', transb='N',
+ *     exactly as in its cublasSgemmBatched comparator (batch_gemm.cu:619-621)
+ */
+#ifndef WMMAE_TCEC_H
+#define WMMAE_TCEC_H
+
+#include <stddef.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+typedef enum {
+  WMMAE_STATUS_SUCCESS = 0,
+  WMMAE_STATUS_INVALID_VALUE = -1,  /* bad size, flag or enum value */
+  WMMAE_STATUS_NULL_POINTER = -2,   /* a required pointer is NULL */
+  WMMAE_STATUS_BAD_LEADING_DIM = -3,/* lda/ldb/ldc smaller than the matrix */
+  WMMAE_STATUS_NOT_SUPPORTED = -4,  /* valid request this build cannot run */
+  WMMAE_STATUS_WORKSPACE_TOO_SMALL = -5,
+  WMMAE_STATUS_RUNTIME_ERROR = -6,  /* a HIP call failed */
+  WMMAE_STATUS_MISALIGNED = -7      /* packed buffer not 16-byte aligned */
+} wmmae_status;
+
+/*
+ * Arithmetic policies.  They mirror the reference's
+ * Policy<Op, ErrorCorrection, ...> / default_policy<T, EC> choices
+ * (tcec/detail/policy.hpp:50-99):
+ *   F16_EC     T = half,  with_ec     v ~ hi + lo/2048, 3 MFMAs per product
+ *   F16_NOEC   T = half,  without_ec  1 MFMA
+ *   BF16X3_EC  T = tf32,  with_ec     gfx950 has no tf32 matrix op; the policy
+ *              is carried by a three-term bf16 split (6 MFMAs), fp32 range
+ *   BF16X2_EC  T = bfloat16, with_ec  two-term bf16 split (3 MFMAs, ~16 bits)
+ *   BF16_NOEC  T = bfloat16, without_ec
+ */
+typedef enum {
+  WMMAE_POLICY_F16_EC = 0,
+  WMMAE_POLICY_F16_NOEC = 1,
+  WMMAE_POLICY_BF16X3_EC = 2,
+  WMMAE_POLICY_BF16X2_EC = 3,
+  WMMAE_POLICY_BF16_NOEC = 4
+} wmmae_policy;
+
+/* flags for the GEMM entry points */
+#define WMMAE_FLAG_RN_MAIN 1 /* accumulate the leading product with fp32 adds
+                                outside the matrix core (the reference's
+                                mma_rn_sync, tcec/tcec.hpp:640-706) */
+
+const char *wmmae_status_string(int status);
+
+/* what: 0 = library version (major*10000 + minor*100 + patch),
+ *       1 = compute units of the current device,
+ *       2 = max engine clock in kHz,
+ *       3 = number of policies */
+int wmmae_query(int what, long long *out);
+
+/* ------------------------------------------------------------------ GEMM
+ * C = alpha * op(A) * op(B) + beta * C with TCEC arithmetic.
+ * Replaces: launch_bgemm + bgemm_kernel of the reference's GEMM harness
+ * (test/tcec/batch_gemm.cu:261-386, 433-443) and stands where that harness
+ * calls cublasSgemmBatched (batch_gemm.cu:619-621).
+ *
+ * workspace holds the split operands; size from wmmae_tcec_sgemm_workspace_bytes.
+ * workspace == NULL lets the library take it from the stream-ordered allocator
+ * (hipMallocAsync / hipFreeAsync on `stream`). */
+int wmmae_tcec_sgemm_workspace_bytes(int m, int n, int k, int batch, int policy,
+                                     size_t *bytes);
+
+int wmmae_tcec_sgemm(char transa, char transb, int m, int n, int k,
+                     const float *alpha, const float *A, int lda,
+                     const float *B, int ldb, const float *beta, float *C,
+                     int ldc, int policy, int flags, void *workspace,
+                     size_t workspace_bytes, void *stream);
+
+int wmmae_tcec_sgemm_strided_batched(char transa, char transb, int m, int n,
+                                     int k, const float *alpha, const float *A,
+                                     int lda, long long stride_a,
+                                     const float *B, int ldb,
+                                     long long stride_b, const float *beta,
+                                     float *C, int ldc, long long stride_c,
+                                     int batch, int policy, int flags,
+                                     void *workspace, size_t workspace_bytes,
+                                     void *stream);
+
+/* The two stages, for callers that keep an operand split across many
+ * products.  A packed operand is `rows` x k (rows = m for op(A), n for op(B))
+ * with element (r, l) read from X[r*row_stride + l*k_stride]; the packed form
+ * is opaque, 16-byte aligned, and only meaningful with the same policy.
+ * Replaces: the per-warp split inside tcec::load_matrix_sync
+ * (tcec/tcec.hpp:194-236), done once per element instead. */
+int wmmae_tcec_pack_bytes(int rows, int k, int batch, int policy,
+                          size_t *bytes);
+int wmmae_tcec_pack(int policy, int rows, int k, const float *X,
+                    long long row_stride, long long k_stride,
+                    long long batch_stride, int batch, void *packed,
+                    size_t packed_bytes, void *stream);
+int wmmae_tcec_gemm_packed(int policy, int m, int n, int k, const float *alpha,
+                           const void *packed_a, const void *packed_b,
+                           const float *beta, float *C, int ldc,
+                           long long stride_c, int batch, int flags,
+                           void *stream);
+
+/* ------------------------------------------- device-API harness kernels
+ * Each runs one of the reference's test kernels, rebuilt on the gfx950
+ * headers, on caller-provided device buffers. */
+
+/* Fragment primitives over num_tiles 16x16 fp32 tiles (256 floats each).
+ * Outputs per tile: a_row, a_col, b_row, b_col: 64 lanes x 4 fp16 registers of
+ * a 16x16x16 fragment filled through foreach_ij; acc_out: 256 floats (tile
+ * read row-major through foreach, stored column-major); vec_out: 32 floats
+ * (load_vector/store_vector round trip of tile[0..15] and tile[16..31]).
+ * Replaces: test/primitive/foreach_ij.cu:20-92, wmma.load_vector.cu:44-72,
+ * wmma.store_vector.cu:36-42. */
+int wmmae_primitive_tiles(const float *tiles, long long num_tiles, void *a_row,
+                          void *a_col, void *b_row, void *b_col,
+                          float *acc_out, float *vec_out, void *stream);
+
+/* Integer layout tables of fragment<use, m, n, k> (use: 0 matrix_a, 1
+ * matrix_b, 2 accumulator; elem: 0 half, 1 bfloat16, 2 float accumulator is
+ * implied by use == 2).  col != 0 selects col_major / mem_col_major.
+ *   ij[(lane*R + reg)*2 + {0,1}], mem_index[lane*R + reg], v_index[lane*R + reg]
+ *   (-1 = not visited by foreach_v), map_tid/map_fid[i*cols + j]
+ * Replaces: test/primitive/map.cu:11-58 and research/fragment_analysis. */
+int wmmae_layout_dump(int use, int m, int n, int k, int col, int *ij,
+                      int *mem_index, int *v_index, int *map_tid, int *map_fid,
+                      void *stream);
+
+/* One-wave TCEC product D = A*B (+C), every operand in one tcec::fragment.
+ * shape: 0 -> m=n=k=32, 1 -> (m,n,k) = (16,48,64) [(32,64,32) for inst 2];
+ * type: 0 half, 1 bfloat16, 2 tf32; ec: 1 with_ec, 0 without_ec;
+ * inst: 0 -> 16x16x32, 1 -> 16x16x16, 2 -> 32x32x16; *_col: memory layouts
+ * (1 = column major, dense leading dimension); c may be NULL;
+ * rounding: 0 mma_sync, 1 mma_rn_sync, 2 mma_rz_sync.
+ * Replaces: mma_kernel_abcd / mma_kernel_abd, test/tcec/mma.cu:23-100. */
+int wmmae_tcec_mma_tile(int shape, int type, int ec, int inst, float *d,
+                        const float *a, const float *b, const float *c,
+                        int a_col, int b_col, int c_col, int d_col,
+                        int rounding, void *stream);
+
+/* Same with m=n=k=32, 16x16x32, operands loaded through the load_matrix_sync
+ * overload that takes the memory layout from the fragment's Layout argument. */
+int wmmae_tcec_mma_tile_native(int type, int ec, int a_frag_col,
+                               int b_frag_col, float *d, const float *a,
+                               const float *b, int d_col, void *stream);
+
+/* y = A*x (left_vector == 0) or y^T = x^T*A (left_vector != 0), N = 32, through
+ * tcec::load_vector / store_vector.  Replaces: test/tcec/matvec.cu:21-50. */
+int wmmae_tcec_matvec(int type, int ec, float *y, const float *a,
+                      const float *x, int a_col, int left_vector,
+                      void *stream);
+
+/* 16-bit split terms held by a 32x32x32 operand fragment (use 0/1) after
+ * load_matrix_sync (from_vector == 0) or load_vector (from_vector != 0):
+ * terms[(term*E + e)*64 + lane], E = fragment num_elements, e = index of x(e).
+ * Replaces: test/tcec/vector.cu:15-61 and test/tcec/elementwise.cu:7-26. */
+int wmmae_tcec_frag_dump(int use, int type, int ec, int frag_col,
+                         unsigned short *terms, const float *src,
+                         int from_vector, int mem_col, void *stream);
+
+/* One raw MFMA D = A*B + C on 16-bit patterns (type 0 half, 1 bfloat16);
+ * (m,n,k) one of (16,16,16), (16,16,32), (32,32,8), (32,32,16); a: m x k,
+ * b: k x n, c/d: m x n, all row-major.
+ * Replaces: test/primitive/mma.cu:11-45 (mma::mma_sync on one tile). */
+int wmmae_mfma_probe(int type, int m, int n, int k, float *d,
+                     const unsigned short *a, const unsigned short *b,
+                     const float *c, void *stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* WMMAE_TCEC_H */

@@ -1,0 +1,424 @@
+/*
+ * CPU oracle for the TCEC SGEMM path.  TEST INFRASTRUCTURE ONLY.
+ *
+ * This file restates, in plain C, the algorithm of the reference
+ * (wmmae/wmma_extension) for the error-corrected fp32 GEMM emulation and the
+ * layout model of the gfx950 MFMA fragments.  It is the checker the GPU code
+ * is compared with.  Only tests/, __graft_entry__.smoke() and the
+ * cpu_baseline leg of bench.py may load it; nothing the library ships calls
+ * into it.
+ *
+ * What pins each function (tests/test_oracle_*.py):
+ *   orc_f32_to_f16 / bf16      numpy's independent float16 conversion over
+ *                              structured + random bit patterns; bf16 against
+ *                              the integer round-to-nearest-even formula and
+ *                              torch.bfloat16
+ *   orc_split_*                closed forms: hi + lo/scale reproduces v to
+ *                              <= 2^-21|v| (fp16), 2^-15 (bf16x2), 2^-23
+ *                              (bf16x3); lo == 0 for representable v
+ *   orc_frag_*                 bijection of (lane,reg)->(i,j), map o foreach_ij
+ *                              = identity, the known-answer inputs of the
+ *                              reference's primitive tests, and on the GPU the
+ *                              multiply-and-compare test against a real MFMA
+ *   orc_tcec_mma / _gemm       identity-B, power-of-two and fp16-representable
+ *                              special cases (exact), reference thresholds
+ *                              1e-5 / 1e-2 (test/tcec/mma.cu:5-21)
+ *   orc_gemm_f64 / _f32        numpy float64 / float32 matmul
+ * PARITY UNPINNED: the bit-level result of the reference's hardware MMA
+ * (CUDA <mma.h> / PTX mma.sync; summation order and rounding inside the tensor
+ * core are not specified and not reproducible on MFMA).  orc_mma_block models
+ * one matrix instruction as an exactly-summed dot product rounded once to
+ * fp32; agreement with either vendor's hardware is to tolerance only.
+ */
+#include <math.h>
+#ifdef _OPENMP
+#include <omp.h>
+#endif
+#include <stdint.h>
+#include <stdlib.h>
+#include <string.h>
+
+/* ------------------------------------------------------------ conversions */
+static inline uint32_t f2u(float f) {
+  uint32_t u;
+  memcpy(&u, &f, 4);
+  return u;
+}
+static inline float u2f(uint32_t u) {
+  float f;
+  memcpy(&f, &u, 4);
+  return f;
+}
+
+/* IEEE binary32 -> binary16, round to nearest even, subnormals kept.
+ * (reference: detail/common.hpp:25-27 cast<half>, a static_cast to half) */
+uint16_t orc_f32_to_f16(float f) {
+  const uint32_t u = f2u(f);
+  const uint32_t sign = (u >> 16) & 0x8000u;
+  const uint32_t absu = u & 0x7fffffffu;
+  if (absu >= 0x7f800000u) { /* inf / nan */
+    if (absu == 0x7f800000u)
+      return (uint16_t)(sign | 0x7c00u);
+    return (uint16_t)(sign | 0x7e00u | ((absu >> 13) & 0x3ffu));
+  }
+  const int32_t exp = (int32_t)(absu >> 23) - 127;
+  uint32_t man = absu & 0x7fffffu;
+  if (exp > 15)
+    return (uint16_t)(sign | 0x7c00u); /* overflow (also after rounding below) */
+  if (exp >= -14) { /* normal range */
+    uint32_t h = ((uint32_t)(exp + 15) << 10) | (man >> 13);
+    const uint32_t rem = man & 0x1fffu;
+    if (rem > 0x1000u || (rem == 0x1000u && (h & 1u)))
+      h++; /* may carry into the exponent, up to inf: correct */
+    return (uint16_t)(sign | h);
+  }
+  if (exp < -25)
+    return (uint16_t)sign; /* below half of the smallest subnormal */
+  /* subnormal result: value = man24 * 2^(exp-23), unit 2^-24 */
+  man |= 0x800000u;
+  const int shift = -exp - 1; /* 14..24 */
+  uint32_t h = man >> shift;
+  const uint32_t rem = man & ((1u << shift) - 1u);
+  const uint32_t half = 1u << (shift - 1);
+  if (rem > half || (rem == half && (h & 1u)))
+    h++;
+  return (uint16_t)(sign | h);
+}
+
+float orc_f16_to_f32(uint16_t h) {
+  const uint32_t sign = ((uint32_t)h & 0x8000u) << 16;
+  const uint32_t exp = (h >> 10) & 0x1fu;
+  uint32_t man = h & 0x3ffu;
+  if (exp == 0x1fu)
+    return u2f(sign | 0x7f800000u | (man << 13));
+  if (exp == 0) {
+    if (man == 0)
+      return u2f(sign);
+    const float v = (float)man * 0x1p-24f;
+    return sign ? -v : v;
+  }
+  return u2f(sign | ((exp + 112u) << 23) | (man << 13));
+}
+
+/* IEEE binary32 -> bfloat16, round to nearest even. */
+uint16_t orc_f32_to_bf16(float f) {
+  uint32_t u = f2u(f);
+  if ((u & 0x7fffffffu) > 0x7f800000u)
+    return (uint16_t)((u >> 16) | 0x0040u); /* quiet nan */
+  u += 0x7fffu + ((u >> 16) & 1u);
+  return (uint16_t)(u >> 16);
+}
+float orc_bf16_to_f32(uint16_t h) { return u2f((uint32_t)h << 16); }
+
+/* ------------------------------------------------------------------ split
+ * kind 0: fp16  two terms, residual scaled by 2048
+ *         (reference: tcec/tcec.hpp:219-223, tcec/detail/scale.hpp:8-20)
+ * kind 1: bf16  two terms, no scaling
+ * kind 2: bf16  three terms, no scaling (stands in for the reference's tf32
+ *         policy, which gfx950 cannot run)
+ * terms[] receives the 16-bit patterns; returns the number of terms. */
+enum { ORC_SPLIT_F16 = 0, ORC_SPLIT_BF16X2 = 1, ORC_SPLIT_BF16X3 = 2 };
+
+int orc_split_terms(int kind) { return kind == ORC_SPLIT_BF16X3 ? 3 : 2; }
+float orc_split_scale(int kind) { return kind == ORC_SPLIT_F16 ? 2048.f : 1.f; }
+
+int orc_split(int kind, float v, uint16_t terms[3]) {
+  if (kind == ORC_SPLIT_F16) {
+    const uint16_t hi = orc_f32_to_f16(v);
+    const float r = (v - orc_f16_to_f32(hi)) * 2048.f;
+    terms[0] = hi;
+    terms[1] = orc_f32_to_f16(r);
+    terms[2] = 0;
+    return 2;
+  }
+  const uint16_t hi = orc_f32_to_bf16(v);
+  const float r1 = v - orc_bf16_to_f32(hi);
+  terms[0] = hi;
+  terms[1] = orc_f32_to_bf16(r1);
+  terms[2] = 0;
+  if (kind == ORC_SPLIT_BF16X2)
+    return 2;
+  const float r2 = r1 - orc_bf16_to_f32(terms[1]);
+  terms[2] = orc_f32_to_bf16(r2);
+  return 3;
+}
+
+float orc_term_to_f32(int kind, uint16_t t) {
+  return kind == ORC_SPLIT_F16 ? orc_f16_to_f32(t) : orc_bf16_to_f32(t);
+}
+
+void orc_split_array(int kind, const float *v, long long n, uint16_t *t0,
+                     uint16_t *t1, uint16_t *t2) {
+#pragma omp parallel for
+  for (long long i = 0; i < n; i++) {
+    uint16_t t[3];
+    orc_split(kind, v[i], t);
+    t0[i] = t[0];
+    if (t1)
+      t1[i] = t[1];
+    if (t2)
+      t2[i] = t[2];
+  }
+}
+
+/* ------------------------------------------------ gfx950 fragment layout
+ * use: 0 = matrix_a (M x K), 1 = matrix_b (K x N), 2 = accumulator (M x N).
+ * Lane l of a wave64, register x:
+ *   A: (i,j) = (l % M, P*(l / M) + x),  P = K*M/64
+ *   B: (i,j) = (P*(l / N) + x, l % N),  P = K*N/64
+ *   C: (i,j) = ((256/N)*(x/4) + 4*(l / N) + x % 4, l % N)
+ * Constants as in ck_tile's warp_gemm_attribute_mfma_impl.hpp (kAMLane,
+ * kABKLane, kABKPerLane, kCMLane, kCNLane, kCM0PerLane, kCM1PerLane); these
+ * replace the NVIDIA tables of the reference (detail/sm_80.hpp:9-402). */
+enum { ORC_USE_A = 0, ORC_USE_B = 1, ORC_USE_ACC = 2 };
+
+int orc_frag_rows(int use, int M, int N, int K) {
+  (void)N;
+  return use == ORC_USE_B ? K : M;
+}
+int orc_frag_cols(int use, int M, int N, int K) {
+  (void)M;
+  return use == ORC_USE_A ? K : N;
+}
+int orc_frag_num_elements(int use, int M, int N, int K) {
+  return orc_frag_rows(use, M, N, K) * orc_frag_cols(use, M, N, K) / 64;
+}
+
+void orc_frag_ij(int use, int M, int N, int K, int lane, int reg, int *i,
+                 int *j) {
+  if (use == ORC_USE_A) {
+    const int P = K * M / 64;
+    *i = lane % M;
+    *j = P * (lane / M) + reg;
+  } else if (use == ORC_USE_B) {
+    const int P = K * N / 64;
+    *i = P * (lane / N) + reg;
+    *j = lane % N;
+  } else {
+    const int groups = 64 / N;
+    *i = 4 * groups * (reg / 4) + 4 * (lane / N) + reg % 4;
+    *j = lane % N;
+  }
+}
+
+/* Inverse: (i,j) -> (lane, reg) (reference: wmma_extension.hpp:115-123). */
+void orc_frag_map(int use, int M, int N, int K, int i, int j, int *tid,
+                  int *fid) {
+  if (use == ORC_USE_A) {
+    const int P = K * M / 64;
+    *tid = i + M * (j / P);
+    *fid = j % P;
+  } else if (use == ORC_USE_B) {
+    const int P = K * N / 64;
+    *tid = j + N * (i / P);
+    *fid = i % P;
+  } else {
+    const int block_rows = 4 * (64 / N);
+    *tid = j + N * ((i % block_rows) / 4);
+    *fid = 4 * (i / block_rows) + i % 4;
+  }
+}
+
+/* mem_index handed to the foreach callback: position in a dense tile
+ * (reference: wmma_extension.hpp:27-55; i + j*rows or i*cols + j). */
+int orc_foreach_mem_index(int use, int M, int N, int K, int col, int lane,
+                          int reg) {
+  int i, j;
+  orc_frag_ij(use, M, N, K, lane, reg, &i, &j);
+  return col ? i + j * orc_frag_rows(use, M, N, K)
+             : i * orc_frag_cols(use, M, N, K) + j;
+}
+
+/* foreach_v: registers holding the first column (col) or first row (!col);
+ * returns the position in the vector, or -1 when the register is skipped
+ * (reference: wmma_extension.hpp:89-112, detail/sm_80.hpp:178-315). */
+int orc_foreach_v_index(int use, int M, int N, int K, int col, int lane,
+                        int reg) {
+  int i, j;
+  orc_frag_ij(use, M, N, K, lane, reg, &i, &j);
+  if (col)
+    return j == 0 ? i : -1;
+  return i == 0 ? j : -1;
+}
+
+/* ----------------------------------------------------------- TCEC model */
+/* One matrix instruction on an fm x fn x fk block: d = sum_k a*b + c with
+ * exact products, an (effectively) exact sum and ONE rounding to fp32.
+ * a points at row i (stride 1 over k), b at column j (stride 1 over k). */
+static inline float orc_mma_block(const float *a, const float *b, int fk,
+                                  float c) {
+  double s = (double)c;
+  for (int l = 0; l < fk; l++)
+    s += (double)a[l] * (double)b[l];
+  return (float)s;
+}
+
+/* Whole-matrix TCEC product following the reference's mma_rn_sync /
+ * mma_rz_sync over k blocks of fk (tcec/tcec.hpp:640-706, 773-831) and its
+ * recombination hi + lo/scale on store (tcec.hpp:332-336).
+ *
+ *   A: m x k, element (i,l) at A[i*lda_r + l*lda_c]
+ *   B: k x n, element (l,j) at B[l*ldb_r + j*ldb_c]
+ *   C/D: m x n, element (i,j) at [i*ld_r + j*ld_c]; C may be NULL
+ *   kind: split kind; ec: 1 = with error correction, 0 = leading term only
+ *   main_outside: 1 = mma_rn_sync (main product rounded alone, then added with
+ *                 an fp32 add), 0 = mma_rz_sync (chained through the accumulator)
+ * D = alpha * (main + err/scale) + beta * C_in is NOT done here; D receives
+ * main + err/scale with C added into main first, as tcec::mma_sync does. */
+void orc_tcec_matmul(int m, int n, int k, int fk, const float *A,
+                     long long lda_r, long long lda_c, const float *B,
+                     long long ldb_r, long long ldb_c, const float *C,
+                     float *D, long long ld_r, long long ld_c, int kind,
+                     int ec, int main_outside) {
+  const int terms = ec ? orc_split_terms(kind) : 1;
+  const float inv_scale = 1.f / orc_split_scale(kind);
+  /* split terms as fp32, K contiguous for both operands */
+  float *At = (float *)malloc(sizeof(float) * 3 * (size_t)m * k);
+  float *Bt = (float *)malloc(sizeof(float) * 3 * (size_t)n * k);
+#pragma omp parallel for
+  for (int i = 0; i < m; i++)
+    for (int l = 0; l < k; l++) {
+      uint16_t t[3];
+      orc_split(kind, A[i * lda_r + l * lda_c], t);
+      for (int p = 0; p < 3; p++)
+        At[((size_t)p * m + i) * k + l] = orc_term_to_f32(kind, t[p]);
+    }
+#pragma omp parallel for
+  for (int j = 0; j < n; j++)
+    for (int l = 0; l < k; l++) {
+      uint16_t t[3];
+      orc_split(kind, B[l * ldb_r + j * ldb_c], t);
+      for (int p = 0; p < 3; p++)
+        Bt[((size_t)p * n + j) * k + l] = orc_term_to_f32(kind, t[p]);
+    }
+#pragma omp parallel for collapse(2)
+  for (int i = 0; i < m; i++) {
+    for (int j = 0; j < n; j++) {
+      const float *a0 = At + ((size_t)0 * m + i) * k;
+      const float *a1 = At + ((size_t)1 * m + i) * k;
+      const float *a2 = At + ((size_t)2 * m + i) * k;
+      const float *b0 = Bt + ((size_t)0 * n + j) * k;
+      const float *b1 = Bt + ((size_t)1 * n + j) * k;
+      const float *b2 = Bt + ((size_t)2 * n + j) * k;
+      float mainv = C ? C[i * ld_r + j * ld_c] : 0.f;
+      float err = 0.f;
+      for (int l0 = 0; l0 < k; l0 += fk) {
+        const int kb = (k - l0 < fk) ? (k - l0) : fk;
+        if (main_outside) {
+          const float tmp = orc_mma_block(a0 + l0, b0 + l0, kb, 0.f);
+          mainv = mainv + tmp;
+        } else {
+          mainv = orc_mma_block(a0 + l0, b0 + l0, kb, mainv);
+        }
+        if (terms >= 3) {
+          err = orc_mma_block(a2 + l0, b0 + l0, kb, err);
+          err = orc_mma_block(a0 + l0, b2 + l0, kb, err);
+          err = orc_mma_block(a1 + l0, b1 + l0, kb, err);
+        }
+        if (terms >= 2) {
+          err = orc_mma_block(a1 + l0, b0 + l0, kb, err);
+          err = orc_mma_block(a0 + l0, b1 + l0, kb, err);
+        }
+      }
+      D[i * ld_r + j * ld_c] = mainv + err * inv_scale;
+    }
+  }
+  free(At);
+  free(Bt);
+}
+
+/* ------------------------------------------------------- reference GEMMs
+ * FP64-accumulate loop of the reference's check
+ * (test/tcec/batch_gemm.cu:559-575; test/tcec/mma.cu:131-152). */
+void orc_gemm_f64(int m, int n, int k, const float *A, long long lda_r,
+                  long long lda_c, const float *B, long long ldb_r,
+                  long long ldb_c, double *D, long long ld_r, long long ld_c) {
+#pragma omp parallel for collapse(2)
+  for (int i = 0; i < m; i++) {
+    for (int j = 0; j < n; j++) {
+      double c = 0.;
+      for (int l = 0; l < k; l++)
+        c += (double)A[i * lda_r + l * lda_c] * (double)B[l * ldb_r + j * ldb_c];
+      D[i * ld_r + j * ld_c] = c;
+    }
+  }
+}
+
+/* Same loop nest with a float accumulator: the plain fp32 SGEMM used as the
+ * accuracy comparator and as the timed CPU baseline.  The product and the add
+ * are rounded separately (no fused multiply-add). */
+void orc_gemm_f32(int m, int n, int k, const float *A, long long lda_r,
+                  long long lda_c, const float *B, long long ldb_r,
+                  long long ldb_c, float *D, long long ld_r, long long ld_c) {
+#pragma omp parallel for collapse(2)
+  for (int i = 0; i < m; i++) {
+    for (int j = 0; j < n; j++) {
+      float c = 0.f;
+      for (int l = 0; l < k; l++) {
+        const float p = A[i * lda_r + l * lda_c] * B[l * ldb_r + j * ldb_c];
+        c += p; /* built with -ffp-contract=off: two roundings */
+      }
+      D[i * ld_r + j * ld_c] = c;
+    }
+  }
+}
+
+/* Fast variant of the same fp32 loop for timing: both operands K-contiguous,
+ * the compiler is free to vectorise the reduction. */
+void orc_gemm_f32_tn(int m, int n, int k, const float *A, int lda,
+                     const float *B, int ldb, float *D, int ldd) {
+#pragma omp parallel for collapse(2)
+  for (int i = 0; i < m; i++) {
+    for (int j = 0; j < n; j++) {
+      const float *a = A + (size_t)i * lda;
+      const float *b = B + (size_t)j * ldb;
+      float c = 0.f;
+      for (int l = 0; l < k; l++)
+        c += a[l] * b[l];
+      D[i + (size_t)j * ldd] = c;
+    }
+  }
+}
+
+/* ---------------------------------------------------------- error metrics */
+/* max|x - ref| / max|ref| (reference: test/primitive/common.hpp:54-103) */
+double orc_max_rel_err(const float *x, const double *ref, long long n) {
+  double md = 0., mr = 0.;
+  for (long long i = 0; i < n; i++) {
+    const double d = fabs((double)x[i] - ref[i]);
+    const double r = fabs(ref[i]);
+    if (d > md)
+      md = d;
+    if (r > mr)
+      mr = r;
+  }
+  return mr > 0. ? md / mr : md;
+}
+/* max|x - ref| (reference: test/tcec/mma.cu:131-152) */
+double orc_max_abs_err(const float *x, const double *ref, long long n) {
+  double md = 0.;
+  for (long long i = 0; i < n; i++) {
+    const double d = fabs((double)x[i] - ref[i]);
+    if (d > md)
+      md = d;
+  }
+  return md;
+}
+/* sqrt(sum (x-ref)^2 / sum ref^2) (reference: test/tcec/batch_gemm.cu:559-605) */
+double orc_frobenius_residual(const float *x, const double *ref, long long n) {
+  double dn = 0., bn = 0.;
+  for (long long i = 0; i < n; i++) {
+    const double d = (double)x[i] - ref[i];
+    dn += d * d;
+    bn += ref[i] * ref[i];
+  }
+  return bn > 0. ? sqrt(dn / bn) : sqrt(dn);
+}
+
+int orc_num_threads(void) {
+#ifdef _OPENMP
+  return omp_get_max_threads();
+#else
+  return 1;
+#endif
+}

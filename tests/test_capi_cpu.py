@@ -1,0 +1,117 @@
+"""Host-side checks of the C-ABI that need no GPU: the library loads, exports
+every declared symbol, and rejects bad arguments before touching a device."""
+import ctypes
+import os
+import re
+
+import pytest
+
+from wmma_extension_amd import _lib
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+
+
+@pytest.fixture(scope="module")
+def h():
+    if not os.path.exists(_lib.LIB_PATH):
+        _lib.build()
+    return _lib.lib()
+
+
+def test_header_and_library_agree(h):
+    text = open(os.path.join(ROOT, "include", "wmmae_tcec.h")).read()
+    declared = set(re.findall(r"\b(wmmae_[a-z0-9_]+)\s*\(", text))
+    assert declared == set(_lib.EXPORTS)
+    for name in declared:
+        assert getattr(h, name) is not None
+
+
+def test_status_strings(h):
+    assert h.wmmae_status_string(0) == b"success"
+    for code in range(-7, 0):
+        assert h.wmmae_status_string(code) not in (b"success", b"unknown status")
+    assert h.wmmae_status_string(-99) == b"unknown status"
+
+
+def test_sizes_are_host_only(h):
+    out = ctypes.c_size_t(0)
+    assert h.wmmae_tcec_pack_bytes(16, 32, 1, 0, ctypes.byref(out)) == 0
+    assert out.value == 2 * 2 * 1024            # k tiles padded to 2, two terms
+    assert h.wmmae_tcec_pack_bytes(4096, 4096, 1, 0, ctypes.byref(out)) == 0
+    assert out.value == 4096 * 4096 * 4          # hi + lo = 4 bytes per element
+    assert h.wmmae_tcec_pack_bytes(4096, 4096, 1, 2, ctypes.byref(out)) == 0
+    assert out.value == 4096 * 4096 * 6
+    assert h.wmmae_tcec_pack_bytes(17, 33, 3, 1, ctypes.byref(out)) == 0
+    assert out.value == 3 * 2 * 2 * 1024
+    assert h.wmmae_tcec_sgemm_workspace_bytes(4096, 4096, 4096, 1, 0, ctypes.byref(out)) == 0
+    assert out.value == 2 * 4096 * 4096 * 4
+    assert h.wmmae_tcec_pack_bytes(16, 32, 1, 9, ctypes.byref(out)) == -1
+    assert h.wmmae_tcec_pack_bytes(-1, 32, 1, 0, ctypes.byref(out)) == -1
+    assert h.wmmae_tcec_pack_bytes(16, 32, 1, 0, None) == -2
+
+
+def _sgemm(h, ta=b"T", tb=b"N", m=64, n=64, k=64, alpha=True, A=1, lda=64, B=1, ldb=64,
+           beta=True, C=1, ldc=64, policy=0, flags=0):
+    one = ctypes.c_float(1.0)
+    return h.wmmae_tcec_sgemm(ta, tb, m, n, k, ctypes.byref(one) if alpha else None,
+                              ctypes.c_void_p(A), lda, ctypes.c_void_p(B), ldb,
+                              ctypes.byref(one) if beta else None, ctypes.c_void_p(C), ldc,
+                              policy, flags, None, 0, None)
+
+
+def test_sgemm_argument_validation(h):
+    # all of these return before any device access (the pointers are fake)
+    assert _sgemm(h, ta=b"X") == -1
+    assert _sgemm(h, tb=b"?") == -1
+    assert _sgemm(h, m=-1) == -1
+    assert _sgemm(h, k=-5) == -1
+    assert _sgemm(h, policy=7) == -1
+    assert _sgemm(h, flags=4) == -1
+    assert _sgemm(h, alpha=False) == -2
+    assert _sgemm(h, beta=False) == -2
+    assert _sgemm(h, A=0) == -2
+    assert _sgemm(h, B=0) == -2
+    assert _sgemm(h, C=0) == -2
+    assert _sgemm(h, lda=63) == -3              # 'T': lda >= k
+    assert _sgemm(h, ldb=10) == -3
+    assert _sgemm(h, ldc=63) == -3
+    assert _sgemm(h, ta=b"N", m=128, lda=64) == -3   # 'N': lda >= m
+    # empty problems succeed without touching anything
+    assert _sgemm(h, m=0, A=0, B=0, C=0) == 0
+    assert _sgemm(h, n=0, A=0, B=0, C=0) == 0
+
+
+def test_other_entry_points_validate(h):
+    one = ctypes.c_float(1.0)
+    p = ctypes.c_void_p
+    assert h.wmmae_tcec_pack(0, 16, 32, p(0), 32, 1, 0, 1, p(16), 4096, None) == -2
+    assert h.wmmae_tcec_pack(0, 16, 32, p(16), 32, 2, 0, 1, p(16), 4096, None) == -3
+    assert h.wmmae_tcec_pack(0, 16, 32, p(16), 32, 1, 0, 1, p(24), 4096, None) == -7
+    assert h.wmmae_tcec_pack(0, 16, 32, p(16), 32, 1, 0, 1, p(32), 100, None) == -5
+    assert h.wmmae_tcec_gemm_packed(0, 16, 16, 32, ctypes.byref(one), p(16), p(16),
+                                    ctypes.byref(one), p(0), 16, 0, 1, 0, None) == -2
+    assert h.wmmae_tcec_gemm_packed(0, 16, 16, 32, ctypes.byref(one), p(16), p(16),
+                                    ctypes.byref(one), p(16), 8, 0, 1, 0, None) == -3
+    assert h.wmmae_tcec_gemm_packed(0, 16, 16, 32, ctypes.byref(one), p(8), p(16),
+                                    ctypes.byref(one), p(16), 16, 0, 1, 0, None) == -7
+    assert h.wmmae_primitive_tiles(p(0), 4, p(0), p(0), p(0), p(0), p(0), p(0), None) == -2
+    assert h.wmmae_primitive_tiles(p(0), -1, p(0), p(0), p(0), p(0), p(0), p(0), None) == -1
+    assert h.wmmae_layout_dump(0, 16, 16, 16, 0, p(0), p(0), p(0), p(0), p(0), None) == -2
+    assert h.wmmae_layout_dump(0, 8, 8, 4, 0, p(8), p(8), p(8), p(8), p(8), None) == -4
+    assert h.wmmae_tcec_mma_tile(0, 0, 1, 0, p(0), p(8), p(8), p(0), 0, 0, 0, 0, 0, None) == -2
+    assert h.wmmae_tcec_mma_tile(3, 0, 1, 0, p(8), p(8), p(8), p(0), 0, 0, 0, 0, 0, None) == -1
+    assert h.wmmae_tcec_mma_tile(0, 5, 1, 0, p(8), p(8), p(8), p(0), 0, 0, 0, 0, 0, None) == -1
+    assert h.wmmae_mfma_probe(0, 8, 8, 8, p(8), p(8), p(8), p(8), None) == -4
+    assert h.wmmae_mfma_probe(2, 16, 16, 16, p(8), p(8), p(8), p(8), None) == -1
+    out = ctypes.c_longlong(0)
+    assert h.wmmae_query(0, ctypes.byref(out)) == 0 and out.value == 100
+    assert h.wmmae_query(3, ctypes.byref(out)) == 0 and out.value == 5
+    assert h.wmmae_query(0, None) == -2
+    assert h.wmmae_query(42, ctypes.byref(out)) == -1
+
+
+def test_missing_library_fails_loudly(monkeypatch):
+    monkeypatch.setattr(_lib, "_LIB", None)
+    monkeypatch.setattr(_lib, "LIB_PATH", "/nonexistent/libwmmae_tcec.so")
+    with pytest.raises(RuntimeError, match="no CPU fallback"):
+        _lib.lib()

@@ -1,0 +1,115 @@
+"""Loader and builder of libwmmae_tcec.so (the C-ABI declared in include/wmmae_tcec.h).
+
+The library is built in-tree with hipcc for gfx950 and loaded with ctypes.
+There is no fallback: if the shared object is missing, `lib()` raises.
+"""
+import ctypes
+import os
+import subprocess
+
+_PKG = os.path.dirname(os.path.abspath(__file__))
+ROOT = os.path.dirname(_PKG)
+INCLUDE_DIR = os.path.join(ROOT, "include")
+CSRC_DIR = os.path.join(_PKG, "csrc")
+LIB_DIR = os.path.join(_PKG, "lib")
+LIB_PATH = os.path.join(LIB_DIR, "libwmmae_tcec.so")
+
+HIPCC_FLAGS = [
+    "--offload-arch=gfx950",
+    "-O3",
+    "-std=c++17",
+    "-fPIC",
+    "-shared",
+    # keep the compiler from forming packed-fp32 VALU ops
+    "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
+]
+
+# every symbol include/wmmae_tcec.h declares
+EXPORTS = [
+    "wmmae_status_string",
+    "wmmae_query",
+    "wmmae_tcec_sgemm_workspace_bytes",
+    "wmmae_tcec_sgemm",
+    "wmmae_tcec_sgemm_strided_batched",
+    "wmmae_tcec_pack_bytes",
+    "wmmae_tcec_pack",
+    "wmmae_tcec_gemm_packed",
+    "wmmae_primitive_tiles",
+    "wmmae_layout_dump",
+    "wmmae_tcec_mma_tile",
+    "wmmae_tcec_mma_tile_native",
+    "wmmae_tcec_matvec",
+    "wmmae_tcec_frag_dump",
+    "wmmae_mfma_probe",
+]
+
+
+def build(verbose=False):
+    """Compile the HIP sources into LIB_PATH (always recompiles)."""
+    os.makedirs(LIB_DIR, exist_ok=True)
+    hipcc = os.environ.get("HIPCC", "/opt/rocm/bin/hipcc")
+    cmd = [hipcc, *HIPCC_FLAGS, "-I" + INCLUDE_DIR,
+           os.path.join(CSRC_DIR, "capi.hip"), "-o", LIB_PATH]
+    res = subprocess.run(cmd, stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True)
+    if verbose or res.returncode != 0:
+        print(res.stdout)
+    if res.returncode != 0:
+        raise RuntimeError("hipcc failed building libwmmae_tcec.so:\n" + res.stdout[-4000:])
+    return LIB_PATH
+
+
+_LIB = None
+
+_c = ctypes
+_vp, _i, _ll, _sz = _c.c_void_p, _c.c_int, _c.c_longlong, _c.c_size_t
+_fp = _c.POINTER(_c.c_float)
+
+_SIGNATURES = {
+    "wmmae_status_string": (_c.c_char_p, [_i]),
+    "wmmae_query": (_i, [_i, _c.POINTER(_ll)]),
+    "wmmae_tcec_sgemm_workspace_bytes": (_i, [_i, _i, _i, _i, _i, _c.POINTER(_sz)]),
+    "wmmae_tcec_sgemm": (_i, [_c.c_char, _c.c_char, _i, _i, _i, _fp, _vp, _i, _vp, _i, _fp,
+                              _vp, _i, _i, _i, _vp, _sz, _vp]),
+    "wmmae_tcec_sgemm_strided_batched": (_i, [_c.c_char, _c.c_char, _i, _i, _i, _fp, _vp, _i, _ll,
+                                              _vp, _i, _ll, _fp, _vp, _i, _ll, _i, _i, _i,
+                                              _vp, _sz, _vp]),
+    "wmmae_tcec_pack_bytes": (_i, [_i, _i, _i, _i, _c.POINTER(_sz)]),
+    "wmmae_tcec_pack": (_i, [_i, _i, _i, _vp, _ll, _ll, _ll, _i, _vp, _sz, _vp]),
+    "wmmae_tcec_gemm_packed": (_i, [_i, _i, _i, _i, _fp, _vp, _vp, _fp, _vp, _i, _ll, _i, _i, _vp]),
+    "wmmae_primitive_tiles": (_i, [_vp, _ll, _vp, _vp, _vp, _vp, _vp, _vp, _vp]),
+    "wmmae_layout_dump": (_i, [_i, _i, _i, _i, _i, _vp, _vp, _vp, _vp, _vp, _vp]),
+    "wmmae_tcec_mma_tile": (_i, [_i, _i, _i, _i, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _vp]),
+    "wmmae_tcec_mma_tile_native": (_i, [_i, _i, _i, _i, _vp, _vp, _vp, _i, _vp]),
+    "wmmae_tcec_matvec": (_i, [_i, _i, _vp, _vp, _vp, _i, _i, _vp]),
+    "wmmae_tcec_frag_dump": (_i, [_i, _i, _i, _i, _vp, _vp, _i, _i, _vp]),
+    "wmmae_mfma_probe": (_i, [_i, _i, _i, _i, _vp, _vp, _vp, _vp, _vp]),
+}
+
+
+def lib():
+    """Return the loaded C-ABI library; raise if it has not been built."""
+    global _LIB
+    if _LIB is None:
+        if not os.path.exists(LIB_PATH):
+            raise RuntimeError(
+                f"{LIB_PATH} is missing: build it with __graft_entry__.build() "
+                "(hipcc --offload-arch=gfx950); there is no CPU fallback")
+        handle = ctypes.CDLL(LIB_PATH)
+        for name, (restype, argtypes) in _SIGNATURES.items():
+            fn = getattr(handle, name)
+            fn.restype = restype
+            fn.argtypes = argtypes
+        _LIB = handle
+    return _LIB
+
+
+class WmmaeError(RuntimeError):
+    def __init__(self, status, where):
+        self.status = status
+        msg = lib().wmmae_status_string(status).decode()
+        super().__init__(f"{where}: {msg} (status {status})")
+
+
+def check(status, where):
+    if status != 0:
+        raise WmmaeError(status, where)

@@ -1,0 +1,708 @@
+// extern "C" boundary of libwmmae_tcec.so: argument validation, kernel
+// selection and launches.  Declarations and per-entry documentation live in
+// include/wmmae_tcec.h.
+#include "harness_kernels.hpp"
+#include "tcec_gemm_kernels.hpp"
+#include <wmmae_tcec.h>
+
+#include <hip/hip_runtime.h>
+
+namespace {
+namespace w = mtk::wmma;
+namespace tcec = mtk::wmma::tcec;
+using wmmae_gemm::u32x4;
+
+#define WMMAE_HIP_TRY(expr)                                                    \
+  do {                                                                         \
+    if ((expr) != hipSuccess)                                                  \
+      return WMMAE_STATUS_RUNTIME_ERROR;                                       \
+  } while (0)
+
+inline int launch_status() {
+  return hipGetLastError() == hipSuccess ? WMMAE_STATUS_SUCCESS
+                                         : WMMAE_STATUS_RUNTIME_ERROR;
+}
+
+template <class T> struct tag {
+  using type = T;
+};
+
+// ------------------------------------------------------------ policy table
+struct PolicyInfo {
+  int terms;       // stored terms per operand
+  bool bf16;       // MFMA element type
+  float inv_scale; // factor applied to the error accumulator
+};
+inline bool policy_info(const int policy, PolicyInfo &p) {
+  switch (policy) {
+  case WMMAE_POLICY_F16_EC:
+    p = {2, false, 1.f / 2048.f};
+    return true;
+  case WMMAE_POLICY_F16_NOEC:
+    p = {1, false, 1.f};
+    return true;
+  case WMMAE_POLICY_BF16X3_EC:
+    p = {3, true, 1.f};
+    return true;
+  case WMMAE_POLICY_BF16X2_EC:
+    p = {2, true, 1.f};
+    return true;
+  case WMMAE_POLICY_BF16_NOEC:
+    p = {1, true, 1.f};
+    return true;
+  default:
+    return false;
+  }
+}
+
+constexpr int kKtPad = 2; // packed k tiles are padded to a multiple of this
+
+inline long long ceil_div(const long long a, const long long b) {
+  return (a + b - 1) / b;
+}
+inline long long packed_row_blocks(const int rows) { return ceil_div(rows, 16); }
+inline int packed_k_tiles(const int k) {
+  return static_cast<int>(ceil_div(ceil_div(k, 32), kKtPad) * kKtPad);
+}
+// u32x4 elements of one packed matrix
+inline long long packed_elems(const int rows, const int k, const int terms) {
+  return packed_row_blocks(rows) * packed_k_tiles(k) * terms * 64;
+}
+
+// ------------------------------------------------------------------ pack
+template <class T, int TERMS>
+int launch_pack(const int rows, const int k, const float *X,
+                const long long row_stride, const long long k_stride,
+                const long long batch_stride, const int batch, void *packed,
+                hipStream_t stream) {
+  const int KT = packed_k_tiles(k);
+  const long long chunks = packed_row_blocks(rows) * KT;
+  const long long blocks = ceil_div(chunks * 64, 256);
+  if (blocks > 0x7fffffffLL || batch > 65535)
+    return WMMAE_STATUS_NOT_SUPPORTED;
+  hipLaunchKernelGGL((wmmae_gemm::split_pack_kernel<T, TERMS>),
+                     dim3(static_cast<unsigned>(blocks), batch), dim3(256), 0,
+                     stream, X, row_stride, k_stride, rows, k, KT, chunks,
+                     batch_stride, static_cast<u32x4 *>(packed),
+                     chunks * TERMS * 64);
+  return launch_status();
+}
+
+int pack_dispatch(const int policy, const int rows, const int k, const float *X,
+                  const long long row_stride, const long long k_stride,
+                  const long long batch_stride, const int batch, void *packed,
+                  hipStream_t stream) {
+#define WMMAE_PACK_ARGS                                                        \
+  rows, k, X, row_stride, k_stride, batch_stride, batch, packed, stream
+  switch (policy) {
+  case WMMAE_POLICY_F16_EC:
+    return launch_pack<w::half, 2>(WMMAE_PACK_ARGS);
+  case WMMAE_POLICY_F16_NOEC:
+    return launch_pack<w::half, 1>(WMMAE_PACK_ARGS);
+  case WMMAE_POLICY_BF16X3_EC:
+    return launch_pack<w::precision::tf32, 3>(WMMAE_PACK_ARGS);
+  case WMMAE_POLICY_BF16X2_EC:
+    return launch_pack<w::bfloat16, 2>(WMMAE_PACK_ARGS);
+  case WMMAE_POLICY_BF16_NOEC:
+    return launch_pack<w::bfloat16, 1>(WMMAE_PACK_ARGS);
+  default:
+    return WMMAE_STATUS_INVALID_VALUE;
+  }
+#undef WMMAE_PACK_ARGS
+}
+
+// ------------------------------------------------------------------ gemm
+struct GemmArgs {
+  const u32x4 *a, *b;
+  float *c;
+  int m, n, k;
+  long long ldc, stride_c;
+  float alpha, beta, inv_scale;
+  int batch, terms;
+  hipStream_t stream;
+};
+
+template <class MT, int TERMS, int BM, int BN, int WGM, int WGN, int KS,
+          bool RN>
+int launch_gemm(const GemmArgs &g) {
+  using Cfg = wmmae_gemm::GemmConfig<MT, TERMS, BM, BN, WGM, WGN, KS, RN>;
+  static_assert(kKtPad % KS == 0, "packed K padding must cover KS");
+  auto kernel = wmmae_gemm::tcec_gemm_kernel<MT, TERMS, BM, BN, WGM, WGN, KS, RN>;
+  WMMAE_HIP_TRY(hipFuncSetAttribute(reinterpret_cast<const void *>(kernel),
+                                    hipFuncAttributeMaxDynamicSharedMemorySize,
+                                    Cfg::LDS_BYTES));
+  const int tiles_m = static_cast<int>(ceil_div(g.m, BM));
+  const int tiles_n = static_cast<int>(ceil_div(g.n, BN));
+  const int KT = packed_k_tiles(g.k);
+  const int rb_a = static_cast<int>(packed_row_blocks(g.m));
+  const int rb_b = static_cast<int>(packed_row_blocks(g.n));
+  const int vec_store =
+      (g.ldc % 4 == 0) && (reinterpret_cast<uintptr_t>(g.c) % 16 == 0) &&
+      (g.stride_c % 4 == 0);
+  hipLaunchKernelGGL(kernel, dim3(tiles_m * tiles_n, g.batch),
+                     dim3(Cfg::NTHREADS), Cfg::LDS_BYTES, g.stream, g.a, g.b,
+                     g.c, g.m, g.n, KT, rb_a, rb_b, g.ldc, g.alpha, g.beta,
+                     g.inv_scale, tiles_m, tiles_n, vec_store,
+                     static_cast<long long>(rb_a) * KT * TERMS * 64,
+                     static_cast<long long>(rb_b) * KT * TERMS * 64,
+                     g.stride_c);
+  return launch_status();
+}
+
+// Tile choice: the large tile when it still gives every compute unit work,
+// otherwise smaller tiles so that more blocks exist.
+template <class MT, int TERMS, bool RN> int gemm_by_size(const GemmArgs &g) {
+  int cus = 256;
+  {
+    int dev = 0;
+    hipDeviceProp_t prop;
+    if (hipGetDevice(&dev) == hipSuccess &&
+        hipGetDeviceProperties(&prop, dev) == hipSuccess &&
+        prop.multiProcessorCount > 0)
+      cus = prop.multiProcessorCount;
+  }
+  const long long big =
+      ceil_div(g.m, 256) * ceil_div(g.n, 128) * static_cast<long long>(g.batch);
+  const long long mid =
+      ceil_div(g.m, 128) * ceil_div(g.n, 128) * static_cast<long long>(g.batch);
+  if constexpr (TERMS <= 2) {
+    if (big >= cus)
+      return launch_gemm<MT, TERMS, 256, 128, 2, 2, 1, RN>(g);
+  }
+  if (mid >= cus || (g.m > 64 && g.n > 64))
+    return launch_gemm<MT, TERMS, 128, 128, 2, 2, TERMS == 3 ? 1 : 2, RN>(g);
+  return launch_gemm<MT, TERMS, 64, 64, 2, 2, 2, RN>(g);
+}
+
+int gemm_dispatch(const int policy, const int flags, const GemmArgs &g) {
+  const bool rn = (flags & WMMAE_FLAG_RN_MAIN) != 0;
+  switch (policy) {
+  case WMMAE_POLICY_F16_EC:
+    return rn ? gemm_by_size<_Float16, 2, true>(g)
+              : gemm_by_size<_Float16, 2, false>(g);
+  case WMMAE_POLICY_F16_NOEC:
+    return rn ? WMMAE_STATUS_NOT_SUPPORTED
+              : gemm_by_size<_Float16, 1, false>(g);
+  case WMMAE_POLICY_BF16X3_EC:
+    return rn ? gemm_by_size<__bf16, 3, true>(g)
+              : gemm_by_size<__bf16, 3, false>(g);
+  case WMMAE_POLICY_BF16X2_EC:
+    return rn ? WMMAE_STATUS_NOT_SUPPORTED
+              : gemm_by_size<__bf16, 2, false>(g);
+  case WMMAE_POLICY_BF16_NOEC:
+    return rn ? WMMAE_STATUS_NOT_SUPPORTED : gemm_by_size<__bf16, 1, false>(g);
+  default:
+    return WMMAE_STATUS_INVALID_VALUE;
+  }
+}
+
+inline bool is_n(const char t) { return t == 'N' || t == 'n'; }
+inline bool is_t(const char t) {
+  return t == 'T' || t == 't' || t == 'C' || t == 'c';
+}
+
+} // namespace
+
+// ===========================================================================
+extern "C" {
+
+const char *wmmae_status_string(const int status) {
+  switch (status) {
+  case WMMAE_STATUS_SUCCESS:
+    return "success";
+  case WMMAE_STATUS_INVALID_VALUE:
+    return "invalid value";
+  case WMMAE_STATUS_NULL_POINTER:
+    return "null pointer";
+  case WMMAE_STATUS_BAD_LEADING_DIM:
+    return "leading dimension too small";
+  case WMMAE_STATUS_NOT_SUPPORTED:
+    return "not supported";
+  case WMMAE_STATUS_WORKSPACE_TOO_SMALL:
+    return "workspace too small";
+  case WMMAE_STATUS_RUNTIME_ERROR:
+    return "HIP runtime error";
+  case WMMAE_STATUS_MISALIGNED:
+    return "buffer not 16-byte aligned";
+  default:
+    return "unknown status";
+  }
+}
+
+int wmmae_query(const int what, long long *const out) {
+  if (out == nullptr)
+    return WMMAE_STATUS_NULL_POINTER;
+  if (what == 0) {
+    *out = 100; // 0.1.0
+    return WMMAE_STATUS_SUCCESS;
+  }
+  if (what == 3) {
+    *out = 5;
+    return WMMAE_STATUS_SUCCESS;
+  }
+  if (what == 1 || what == 2) {
+    int dev = 0;
+    hipDeviceProp_t prop;
+    WMMAE_HIP_TRY(hipGetDevice(&dev));
+    WMMAE_HIP_TRY(hipGetDeviceProperties(&prop, dev));
+    *out = what == 1 ? prop.multiProcessorCount : prop.clockRate;
+    return WMMAE_STATUS_SUCCESS;
+  }
+  return WMMAE_STATUS_INVALID_VALUE;
+}
+
+// ------------------------------------------------------------- pack / gemm
+int wmmae_tcec_pack_bytes(const int rows, const int k, const int batch,
+                          const int policy, size_t *const bytes) {
+  PolicyInfo p;
+  if (bytes == nullptr)
+    return WMMAE_STATUS_NULL_POINTER;
+  if (!policy_info(policy, p) || rows < 0 || k < 0 || batch < 0)
+    return WMMAE_STATUS_INVALID_VALUE;
+  *bytes = static_cast<size_t>(packed_elems(rows, k, p.terms)) * 16u *
+           static_cast<size_t>(batch);
+  return WMMAE_STATUS_SUCCESS;
+}
+
+int wmmae_tcec_pack(const int policy, const int rows, const int k,
+                    const float *const X, const long long row_stride,
+                    const long long k_stride, const long long batch_stride,
+                    const int batch, void *const packed,
+                    const size_t packed_bytes, void *const stream) {
+  PolicyInfo p;
+  if (!policy_info(policy, p) || rows < 0 || k < 0 || batch < 0)
+    return WMMAE_STATUS_INVALID_VALUE;
+  if (rows == 0 || k == 0 || batch == 0)
+    return WMMAE_STATUS_SUCCESS;
+  if (X == nullptr || packed == nullptr)
+    return WMMAE_STATUS_NULL_POINTER;
+  if (row_stride < 1 || k_stride < 1 || (row_stride != 1 && k_stride != 1))
+    return WMMAE_STATUS_BAD_LEADING_DIM;
+  if (reinterpret_cast<uintptr_t>(packed) % 16 != 0)
+    return WMMAE_STATUS_MISALIGNED;
+  size_t need = 0;
+  wmmae_tcec_pack_bytes(rows, k, batch, policy, &need);
+  if (packed_bytes < need)
+    return WMMAE_STATUS_WORKSPACE_TOO_SMALL;
+  return pack_dispatch(policy, rows, k, X, row_stride, k_stride, batch_stride,
+                       batch, packed, static_cast<hipStream_t>(stream));
+}
+
+int wmmae_tcec_gemm_packed(const int policy, const int m, const int n,
+                           const int k, const float *const alpha,
+                           const void *const packed_a,
+                           const void *const packed_b, const float *const beta,
+                           float *const C, const int ldc,
+                           const long long stride_c, const int batch,
+                           const int flags, void *const stream) {
+  PolicyInfo p;
+  if (!policy_info(policy, p) || m < 0 || n < 0 || k < 0 || batch < 0 ||
+      (flags & ~WMMAE_FLAG_RN_MAIN) != 0)
+    return WMMAE_STATUS_INVALID_VALUE;
+  if (alpha == nullptr || beta == nullptr)
+    return WMMAE_STATUS_NULL_POINTER;
+  if (m == 0 || n == 0 || batch == 0)
+    return WMMAE_STATUS_SUCCESS;
+  if (C == nullptr || (k > 0 && (packed_a == nullptr || packed_b == nullptr)))
+    return WMMAE_STATUS_NULL_POINTER;
+  if (ldc < m)
+    return WMMAE_STATUS_BAD_LEADING_DIM;
+  if (batch > 65535)
+    return WMMAE_STATUS_NOT_SUPPORTED;
+  if (k > 0 && (reinterpret_cast<uintptr_t>(packed_a) % 16 != 0 ||
+                reinterpret_cast<uintptr_t>(packed_b) % 16 != 0))
+    return WMMAE_STATUS_MISALIGNED;
+  if (k == 0) {
+    const long long blocks = ceil_div(static_cast<long long>(m) * n, 256);
+    if (blocks > 0x7fffffffLL)
+      return WMMAE_STATUS_NOT_SUPPORTED;
+    hipLaunchKernelGGL(wmmae_gemm::scale_c_kernel,
+                       dim3(static_cast<unsigned>(blocks), batch), dim3(256), 0,
+                       static_cast<hipStream_t>(stream), C, m, n,
+                       static_cast<long long>(ldc), stride_c, *beta);
+    return launch_status();
+  }
+  GemmArgs g;
+  g.a = static_cast<const u32x4 *>(packed_a);
+  g.b = static_cast<const u32x4 *>(packed_b);
+  g.c = C;
+  g.m = m;
+  g.n = n;
+  g.k = k;
+  g.ldc = ldc;
+  g.stride_c = stride_c;
+  g.alpha = *alpha;
+  g.beta = *beta;
+  g.inv_scale = p.inv_scale;
+  g.batch = batch;
+  g.terms = p.terms;
+  g.stream = static_cast<hipStream_t>(stream);
+  return gemm_dispatch(policy, flags, g);
+}
+
+int wmmae_tcec_sgemm_workspace_bytes(const int m, const int n, const int k,
+                                     const int batch, const int policy,
+                                     size_t *const bytes) {
+  size_t a = 0, b = 0;
+  if (bytes == nullptr)
+    return WMMAE_STATUS_NULL_POINTER;
+  if (m < 0 || n < 0)
+    return WMMAE_STATUS_INVALID_VALUE;
+  int s = wmmae_tcec_pack_bytes(m, k, batch, policy, &a);
+  if (s != WMMAE_STATUS_SUCCESS)
+    return s;
+  s = wmmae_tcec_pack_bytes(n, k, batch, policy, &b);
+  if (s != WMMAE_STATUS_SUCCESS)
+    return s;
+  *bytes = a + b;
+  return WMMAE_STATUS_SUCCESS;
+}
+
+int wmmae_tcec_sgemm_strided_batched(
+    const char transa, const char transb, const int m, const int n, const int k,
+    const float *const alpha, const float *const A, const int lda,
+    const long long stride_a, const float *const B, const int ldb,
+    const long long stride_b, const float *const beta, float *const C,
+    const int ldc, const long long stride_c, const int batch, const int policy,
+    const int flags, void *workspace, const size_t workspace_bytes,
+    void *const stream) {
+  PolicyInfo p;
+  if ((!is_n(transa) && !is_t(transa)) || (!is_n(transb) && !is_t(transb)) ||
+      m < 0 || n < 0 || k < 0 || batch < 0 || !policy_info(policy, p) ||
+      (flags & ~WMMAE_FLAG_RN_MAIN) != 0)
+    return WMMAE_STATUS_INVALID_VALUE;
+  if (alpha == nullptr || beta == nullptr)
+    return WMMAE_STATUS_NULL_POINTER;
+  if (m == 0 || n == 0 || batch == 0)
+    return WMMAE_STATUS_SUCCESS;
+  if (C == nullptr || (k > 0 && (A == nullptr || B == nullptr)))
+    return WMMAE_STATUS_NULL_POINTER;
+  const int a_rows = is_n(transa) ? m : k; // rows of A as stored (column major)
+  const int b_rows = is_n(transb) ? k : n;
+  if (lda < (a_rows > 1 ? a_rows : 1) || ldb < (b_rows > 1 ? b_rows : 1) ||
+      ldc < m)
+    return WMMAE_STATUS_BAD_LEADING_DIM;
+
+  size_t bytes_a = 0, bytes_b = 0;
+  wmmae_tcec_pack_bytes(m, k, batch, policy, &bytes_a);
+  wmmae_tcec_pack_bytes(n, k, batch, policy, &bytes_b);
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  bool own = false;
+  if (workspace == nullptr) {
+    if (bytes_a + bytes_b > 0) {
+      WMMAE_HIP_TRY(hipMallocAsync(&workspace, bytes_a + bytes_b, s));
+      own = true;
+    }
+  } else {
+    if (reinterpret_cast<uintptr_t>(workspace) % 16 != 0)
+      return WMMAE_STATUS_MISALIGNED;
+    if (workspace_bytes < bytes_a + bytes_b)
+      return WMMAE_STATUS_WORKSPACE_TOO_SMALL;
+  }
+  void *const pa = workspace;
+  void *const pb = static_cast<char *>(workspace) + bytes_a;
+
+  int st = WMMAE_STATUS_SUCCESS;
+  if (k > 0) {
+    // op(A)(i,l): 'N' -> A[i + l*lda], 'T' -> A[l + i*lda]
+    st = wmmae_tcec_pack(policy, m, k, A, is_n(transa) ? 1 : lda,
+                         is_n(transa) ? lda : 1, stride_a, batch, pa, bytes_a,
+                         stream);
+    // op(B)(l,j): 'N' -> B[l + j*ldb], 'T' -> B[j + l*ldb]; packed rows = j
+    if (st == WMMAE_STATUS_SUCCESS)
+      st = wmmae_tcec_pack(policy, n, k, B, is_n(transb) ? ldb : 1,
+                           is_n(transb) ? 1 : ldb, stride_b, batch, pb, bytes_b,
+                           stream);
+  }
+  if (st == WMMAE_STATUS_SUCCESS)
+    st = wmmae_tcec_gemm_packed(policy, m, n, k, alpha, pa, pb, beta, C, ldc,
+                                stride_c, batch, flags, stream);
+  if (own) {
+    if (hipFreeAsync(workspace, s) != hipSuccess &&
+        st == WMMAE_STATUS_SUCCESS)
+      st = WMMAE_STATUS_RUNTIME_ERROR;
+  }
+  return st;
+}
+
+int wmmae_tcec_sgemm(const char transa, const char transb, const int m,
+                     const int n, const int k, const float *const alpha,
+                     const float *const A, const int lda, const float *const B,
+                     const int ldb, const float *const beta, float *const C,
+                     const int ldc, const int policy, const int flags,
+                     void *const workspace, const size_t workspace_bytes,
+                     void *const stream) {
+  return wmmae_tcec_sgemm_strided_batched(transa, transb, m, n, k, alpha, A,
+                                          lda, 0, B, ldb, 0, beta, C, ldc, 0, 1,
+                                          policy, flags, workspace,
+                                          workspace_bytes, stream);
+}
+
+// ------------------------------------------------------------ harness
+int wmmae_primitive_tiles(const float *const tiles, const long long num_tiles,
+                          void *const a_row, void *const a_col,
+                          void *const b_row, void *const b_col,
+                          float *const acc_out, float *const vec_out,
+                          void *const stream) {
+  if (num_tiles < 0)
+    return WMMAE_STATUS_INVALID_VALUE;
+  if (num_tiles == 0)
+    return WMMAE_STATUS_SUCCESS;
+  if (!tiles || !a_row || !a_col || !b_row || !b_col || !acc_out || !vec_out)
+    return WMMAE_STATUS_NULL_POINTER;
+  long long blocks = (num_tiles + 3) / 4; // 4 waves per block, one tile per wave
+  if (blocks > 256 * 32)
+    blocks = 256 * 32; // grid-stride beyond this
+  hipLaunchKernelGGL(wmmae_harness::primitive_tiles_kernel,
+                     dim3(static_cast<unsigned>(blocks)), dim3(256), 0,
+                     static_cast<hipStream_t>(stream), tiles, num_tiles,
+                     static_cast<w::half *>(a_row), static_cast<w::half *>(a_col),
+                     static_cast<w::half *>(b_row), static_cast<w::half *>(b_col),
+                     acc_out, vec_out);
+  return launch_status();
+}
+
+} // extern "C"
+
+namespace {
+template <class Frag>
+int launch_layout_dump(const int col, int *ij, int *mem_index, int *v_index,
+                       int *map_tid, int *map_fid, hipStream_t s) {
+  hipLaunchKernelGGL((wmmae_harness::layout_dump_kernel<Frag>), dim3(1),
+                     dim3(64), 0, s, col, ij, mem_index, v_index, map_tid,
+                     map_fid);
+  return launch_status();
+}
+template <int M, int N, int K>
+int layout_dump_shape(const int use, const int col, int *ij, int *mem_index,
+                      int *v_index, int *map_tid, int *map_fid,
+                      hipStream_t s) {
+  if (use == 0) {
+    return col ? launch_layout_dump<
+                     w::fragment<w::matrix_a, M, N, K, w::half, w::col_major>>(
+                     col, ij, mem_index, v_index, map_tid, map_fid, s)
+               : launch_layout_dump<
+                     w::fragment<w::matrix_a, M, N, K, w::half, w::row_major>>(
+                     col, ij, mem_index, v_index, map_tid, map_fid, s);
+  }
+  if (use == 1) {
+    return col ? launch_layout_dump<
+                     w::fragment<w::matrix_b, M, N, K, w::half, w::col_major>>(
+                     col, ij, mem_index, v_index, map_tid, map_fid, s)
+               : launch_layout_dump<
+                     w::fragment<w::matrix_b, M, N, K, w::half, w::row_major>>(
+                     col, ij, mem_index, v_index, map_tid, map_fid, s);
+  }
+  if (use == 2)
+    return launch_layout_dump<w::fragment<w::accumulator, M, N, K, float>>(
+        col, ij, mem_index, v_index, map_tid, map_fid, s);
+  return WMMAE_STATUS_INVALID_VALUE;
+}
+} // namespace
+
+extern "C" {
+
+int wmmae_layout_dump(const int use, const int m, const int n, const int k,
+                      const int col, int *const ij, int *const mem_index,
+                      int *const v_index, int *const map_tid,
+                      int *const map_fid, void *const stream) {
+  if (!ij || !mem_index || !v_index || !map_tid || !map_fid)
+    return WMMAE_STATUS_NULL_POINTER;
+  hipStream_t s = static_cast<hipStream_t>(stream);
+#define WMMAE_SHAPE(M_, N_, K_)                                                \
+  if (m == M_ && n == N_ && k == K_)                                           \
+    return layout_dump_shape<M_, N_, K_>(use, col, ij, mem_index, v_index,     \
+                                         map_tid, map_fid, s);
+  WMMAE_SHAPE(16, 16, 16)
+  WMMAE_SHAPE(16, 16, 32)
+  WMMAE_SHAPE(32, 32, 8)
+  WMMAE_SHAPE(32, 32, 16)
+#undef WMMAE_SHAPE
+  return WMMAE_STATUS_NOT_SUPPORTED;
+}
+
+} // extern "C"
+
+namespace {
+template <class F> int with_type(const int type, F f) {
+  switch (type) {
+  case 0:
+    return f(tag<w::half>{});
+  case 1:
+    return f(tag<w::bfloat16>{});
+  case 2:
+    return f(tag<w::precision::tf32>{});
+  default:
+    return WMMAE_STATUS_INVALID_VALUE;
+  }
+}
+template <class F> int with_ec(const int ec, F f) {
+  if (ec)
+    return f(tag<tcec::with_ec>{});
+  return f(tag<tcec::without_ec>{});
+}
+template <class F> int with_layout(const int col, F f) {
+  if (col)
+    return f(tag<w::col_major>{});
+  return f(tag<w::row_major>{});
+}
+} // namespace
+
+extern "C" {
+
+int wmmae_tcec_mma_tile(const int shape, const int type, const int ec,
+                        const int inst, float *const d, const float *const a,
+                        const float *const b, const float *const c,
+                        const int a_col, const int b_col, const int c_col,
+                        const int d_col, const int rounding,
+                        void *const stream) {
+  if (!d || !a || !b)
+    return WMMAE_STATUS_NULL_POINTER;
+  if (shape < 0 || shape > 1 || inst < 0 || inst > 2 || rounding < 0 ||
+      rounding > 2)
+    return WMMAE_STATUS_INVALID_VALUE;
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  return with_type(type, [&](auto tt) {
+    using T = typename decltype(tt)::type;
+    return with_ec(ec, [&](auto te) {
+      using EC = typename decltype(te)::type;
+      auto go = [&](auto kernel) {
+        hipLaunchKernelGGL(kernel, dim3(1), dim3(64), 0, s, d, a, b, c, a_col,
+                           b_col, c_col, d_col, rounding);
+        return launch_status();
+      };
+      using R = w::row_major;
+      using Cm = w::col_major;
+      if (inst == 0) {
+        using P = tcec::Policy<tcec::op_mfma, EC, 16, 16, 32>;
+        return shape == 0
+                   ? go(wmmae_harness::tcec_mma_tile_kernel<32, 32, 32, T, P, R,
+                                                            Cm>)
+                   : go(wmmae_harness::tcec_mma_tile_kernel<16, 48, 64, T, P, R,
+                                                            Cm>);
+      }
+      if (inst == 1) {
+        using P = tcec::Policy<tcec::op_mfma, EC, 16, 16, 16>;
+        return shape == 0
+                   ? go(wmmae_harness::tcec_mma_tile_kernel<32, 32, 32, T, P, R,
+                                                            Cm>)
+                   : go(wmmae_harness::tcec_mma_tile_kernel<16, 48, 64, T, P, R,
+                                                            Cm>);
+      }
+      using P = tcec::Policy<tcec::op_mfma, EC, 32, 32, 16>;
+      return shape == 0
+                 ? go(wmmae_harness::tcec_mma_tile_kernel<32, 32, 32, T, P, R,
+                                                          Cm>)
+                 : go(wmmae_harness::tcec_mma_tile_kernel<32, 64, 32, T, P, R,
+                                                          Cm>);
+    });
+  });
+}
+
+int wmmae_tcec_mma_tile_native(const int type, const int ec,
+                               const int a_frag_col, const int b_frag_col,
+                               float *const d, const float *const a,
+                               const float *const b, const int d_col,
+                               void *const stream) {
+  if (!d || !a || !b)
+    return WMMAE_STATUS_NULL_POINTER;
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  return with_type(type, [&](auto tt) {
+    using T = typename decltype(tt)::type;
+    return with_ec(ec, [&](auto te) {
+      using EC = typename decltype(te)::type;
+      using P = tcec::Policy<tcec::op_mfma, EC, 16, 16, 32>;
+      return with_layout(a_frag_col, [&](auto la) {
+        using AL = typename decltype(la)::type;
+        return with_layout(b_frag_col, [&](auto lb) {
+          using BL = typename decltype(lb)::type;
+          hipLaunchKernelGGL(
+              (wmmae_harness::tcec_mma_tile_native_kernel<32, 32, 32, T, P, AL,
+                                                          BL>),
+              dim3(1), dim3(64), 0, s, d, a, b, d_col);
+          return launch_status();
+        });
+      });
+    });
+  });
+}
+
+int wmmae_tcec_matvec(const int type, const int ec, float *const y,
+                      const float *const a, const float *const x,
+                      const int a_col, const int left_vector,
+                      void *const stream) {
+  if (!y || !a || !x)
+    return WMMAE_STATUS_NULL_POINTER;
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  return with_type(type, [&](auto tt) {
+    using T = typename decltype(tt)::type;
+    return with_ec(ec, [&](auto te) {
+      using EC = typename decltype(te)::type;
+      using P = tcec::Policy<tcec::op_mfma, EC, 16, 16, 32>;
+      hipLaunchKernelGGL((wmmae_harness::tcec_matvec_kernel<32, T, P>), dim3(1),
+                         dim3(64), 0, s, y, a, x, a_col, left_vector);
+      return launch_status();
+    });
+  });
+}
+
+int wmmae_tcec_frag_dump(const int use, const int type, const int ec,
+                         const int frag_col, unsigned short *const terms,
+                         const float *const src, const int from_vector,
+                         const int mem_col, void *const stream) {
+  if (!terms || !src)
+    return WMMAE_STATUS_NULL_POINTER;
+  if (use < 0 || use > 1)
+    return WMMAE_STATUS_INVALID_VALUE;
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  return with_type(type, [&](auto tt) {
+    using T = typename decltype(tt)::type;
+    return with_ec(ec, [&](auto te) {
+      using EC = typename decltype(te)::type;
+      using P = tcec::Policy<tcec::op_mfma, EC, 16, 16, 32>;
+      return with_layout(frag_col, [&](auto ll) {
+        using L = typename decltype(ll)::type;
+        if (use == 0)
+          hipLaunchKernelGGL(
+              (wmmae_harness::tcec_frag_dump_kernel<w::matrix_a, 32, T, P, L>),
+              dim3(1), dim3(64), 0, s, terms, src, from_vector, mem_col);
+        else
+          hipLaunchKernelGGL(
+              (wmmae_harness::tcec_frag_dump_kernel<w::matrix_b, 32, T, P, L>),
+              dim3(1), dim3(64), 0, s, terms, src, from_vector, mem_col);
+        return launch_status();
+      });
+    });
+  });
+}
+
+int wmmae_mfma_probe(const int type, const int m, const int n, const int k,
+                     float *const d, const unsigned short *const a,
+                     const unsigned short *const b, const float *const c,
+                     void *const stream) {
+  if (!d || !a || !b || !c)
+    return WMMAE_STATUS_NULL_POINTER;
+  if (type < 0 || type > 1)
+    return WMMAE_STATUS_INVALID_VALUE;
+  hipStream_t s = static_cast<hipStream_t>(stream);
+#define WMMAE_PROBE(M_, N_, K_)                                                \
+  if (m == M_ && n == N_ && k == K_) {                                         \
+    if (type == 0)                                                             \
+      hipLaunchKernelGGL(                                                      \
+          (wmmae_harness::mfma_probe_kernel<w::half, M_, N_, K_>), dim3(1),    \
+          dim3(64), 0, s, d, a, b, c);                                         \
+    else                                                                       \
+      hipLaunchKernelGGL(                                                      \
+          (wmmae_harness::mfma_probe_kernel<w::bfloat16, M_, N_, K_>),         \
+          dim3(1), dim3(64), 0, s, d, a, b, c);                                \
+    return launch_status();                                                    \
+  }
+  WMMAE_PROBE(16, 16, 16)
+  WMMAE_PROBE(16, 16, 32)
+  WMMAE_PROBE(32, 32, 8)
+  WMMAE_PROBE(32, 32, 16)
+#undef WMMAE_PROBE
+  return WMMAE_STATUS_NOT_SUPPORTED;
+}
+
+} // extern "C"

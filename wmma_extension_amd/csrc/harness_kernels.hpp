@@ -1,0 +1,338 @@
+// One-wave and tile-stream kernels that exercise the public device API the
+// way the reference's own test programs do.  They are compiled into the C-ABI
+// library so that host tests can drive the header-only API without a
+// compiler on the test machine.
+//
+//   primitive_tiles_kernel  : foreach / foreach_ij / load_vector / store_vector
+//                             over a stream of 16x16 tiles
+//                             (reference: test/primitive/foreach_ij.cu:20-92,
+//                             wmma.load_vector.cu:44-72, wmma.store_vector.cu:36-42)
+//   layout_dump_kernel      : integer tables of foreach_ij / foreach / foreach_v / map
+//                             (reference: test/primitive/map.cu:11-58)
+//   tcec_mma_tile_kernel    : one-wave D = A*B (+C) through tcec::load_matrix_sync /
+//                             mma_sync / store_matrix_sync
+//                             (reference: test/tcec/mma.cu:23-100)
+//   tcec_matvec_kernel      : y = A*x through tcec::load_vector / store_vector
+//                             (reference: test/tcec/matvec.cu:21-50)
+//   tcec_frag_dump_kernel   : split terms held by an operand fragment after
+//                             load_matrix_sync or load_vector
+//                             (reference: test/tcec/vector.cu:15-61)
+//   mfma_probe_kernel       : one raw MFMA on caller-supplied bit patterns
+#pragma once
+#include <wmma_extension/tcec/tcec.hpp>
+#include <wmma_extension/wmma_mma.hpp>
+
+namespace wmmae_harness {
+namespace w = mtk::wmma;
+namespace tcec = mtk::wmma::tcec;
+
+// --------------------------------------------------------------------------
+// Fragment primitives over a stream of tiles.  One wave per tile, grid-stride.
+// Per tile (256 fp32 in):
+//   a_row/a_col/b_row/b_col : (lane,reg) dump of a 16x16x16 half fragment filled
+//                             through foreach_ij from the tile read in that layout
+//   acc_out                 : tile read as a row-major accumulator through
+//                             foreach(mem_row_major), written with
+//                             store_matrix_sync(mem_col_major)  (a transpose)
+//   vec_out[0]              : tile[0..15] -> load_vector(acc, col) -> store_vector(col)
+//   vec_out[1]              : tile[16..31] -> load_vector(acc, row) -> store_vector(row)
+// --------------------------------------------------------------------------
+__global__ void __launch_bounds__(256)
+    primitive_tiles_kernel(const float *__restrict__ tiles,
+                           const long long num_tiles,
+                           w::half *__restrict__ a_row,
+                           w::half *__restrict__ a_col,
+                           w::half *__restrict__ b_row,
+                           w::half *__restrict__ b_col,
+                           float *__restrict__ acc_out,
+                           float *__restrict__ vec_out) {
+  const unsigned lane = w::detail::common::get_lane_id();
+  const long long wave = (static_cast<long long>(blockIdx.x) * blockDim.x +
+                          threadIdx.x) /
+                         w::wave_size;
+  const long long num_waves =
+      static_cast<long long>(gridDim.x) * blockDim.x / w::wave_size;
+  using FA_R = w::fragment<w::matrix_a, 16, 16, 16, w::half, w::row_major>;
+  using FA_C = w::fragment<w::matrix_a, 16, 16, 16, w::half, w::col_major>;
+  using FB_R = w::fragment<w::matrix_b, 16, 16, 16, w::half, w::row_major>;
+  using FB_C = w::fragment<w::matrix_b, 16, 16, 16, w::half, w::col_major>;
+  using FC = w::fragment<w::accumulator, 16, 16, 16, float>;
+
+  for (long long t = wave; t < num_tiles; t += num_waves) {
+    const float *const tile = tiles + t * 256;
+    {
+      FA_R f;
+      w::foreach_ij<FA_R>([&](const unsigned *list, const unsigned count,
+                              const unsigned i, const unsigned j) {
+        for (unsigned c = 0; c < count; c++)
+          f.x[list[c]] = w::detail::common::cast<w::half>(tile[i * 16 + j]);
+      });
+      for (unsigned x = 0; x < f.num_elements; x++)
+        a_row[(t * 64 + lane) * f.num_elements + x] = f.x[x];
+    }
+    {
+      FA_C f;
+      w::foreach_ij<FA_C>([&](const unsigned *list, const unsigned count,
+                              const unsigned i, const unsigned j) {
+        for (unsigned c = 0; c < count; c++)
+          f.x[list[c]] = w::detail::common::cast<w::half>(tile[i + j * 16]);
+      });
+      for (unsigned x = 0; x < f.num_elements; x++)
+        a_col[(t * 64 + lane) * f.num_elements + x] = f.x[x];
+    }
+    {
+      FB_R f;
+      w::foreach_ij<FB_R>([&](const unsigned *list, const unsigned count,
+                              const unsigned i, const unsigned j) {
+        for (unsigned c = 0; c < count; c++)
+          f.x[list[c]] = w::detail::common::cast<w::half>(tile[i * 16 + j]);
+      });
+      for (unsigned x = 0; x < f.num_elements; x++)
+        b_row[(t * 64 + lane) * f.num_elements + x] = f.x[x];
+    }
+    {
+      FB_C f;
+      w::foreach_ij<FB_C>([&](const unsigned *list, const unsigned count,
+                              const unsigned i, const unsigned j) {
+        for (unsigned c = 0; c < count; c++)
+          f.x[list[c]] = w::detail::common::cast<w::half>(tile[i + j * 16]);
+      });
+      for (unsigned x = 0; x < f.num_elements; x++)
+        b_col[(t * 64 + lane) * f.num_elements + x] = f.x[x];
+    }
+    {
+      FC f;
+      w::foreach<FC>(w::mem_row_major,
+                     [&](const unsigned *list, const unsigned count,
+                         const unsigned mem_index) {
+                       for (unsigned c = 0; c < count; c++)
+                         f.x[list[c]] = tile[mem_index];
+                     });
+      w::store_matrix_sync(acc_out + t * 256, f, 16, w::mem_col_major);
+    }
+    {
+      FC f;
+      w::load_vector(f, tile, w::mem_col_major);
+      w::store_vector(vec_out + t * 32, f, w::mem_col_major);
+      w::load_vector(f, tile + 16, w::mem_row_major);
+      w::store_vector(vec_out + t * 32 + 16, f, w::mem_row_major);
+    }
+  }
+}
+
+// --------------------------------------------------------------------------
+// Integer layout tables of one fragment type, one wave.
+//   ij[(lane*R + reg)*2 + {0,1}]      = (i, j) from foreach_ij
+//   mem_index[lane*R + reg]           = mem_index from foreach
+//   v_index[lane*R + reg]             = mem_index from foreach_v, or -1 if the
+//                                       register is not visited
+//   map_tid/map_fid[i*cols + j]       = map(i, j)
+// R = num_elements.  col selects col_major / mem_col_major.
+// --------------------------------------------------------------------------
+template <class Frag>
+__global__ void __launch_bounds__(64)
+    layout_dump_kernel(const int col, int *__restrict__ ij,
+                       int *__restrict__ mem_index, int *__restrict__ v_index,
+                       int *__restrict__ map_tid, int *__restrict__ map_fid) {
+  constexpr bool is_acc = std::is_same<typename Frag::use, w::accumulator>::value;
+  constexpr unsigned R = Frag::num_elements;
+  const unsigned lane = w::detail::common::get_lane_id();
+  for (unsigned x = 0; x < R; x++)
+    v_index[lane * R + x] = -1;
+  w::foreach_ij<Frag>([&](const unsigned *list, const unsigned count,
+                          const unsigned i, const unsigned j) {
+    for (unsigned c = 0; c < count; c++) {
+      ij[(lane * R + list[c]) * 2 + 0] = i;
+      ij[(lane * R + list[c]) * 2 + 1] = j;
+    }
+  });
+  auto put_mem = [&](const unsigned *list, const unsigned count,
+                     const unsigned idx) {
+    for (unsigned c = 0; c < count; c++)
+      mem_index[lane * R + list[c]] = idx;
+  };
+  auto put_v = [&](const unsigned *list, const unsigned count,
+                   const unsigned idx) {
+    for (unsigned c = 0; c < count; c++)
+      v_index[lane * R + list[c]] = idx;
+  };
+  if constexpr (is_acc) {
+    const w::layout_t l = col ? w::mem_col_major : w::mem_row_major;
+    w::foreach<Frag>(l, put_mem);
+    w::foreach_v<Frag>(l, put_v);
+  } else {
+    w::foreach<Frag>(put_mem);
+    w::foreach_v<Frag>(put_v);
+  }
+  using L = typename Frag::layout_model;
+  for (unsigned e = lane; e < L::rows * L::cols; e += w::wave_size) {
+    unsigned tid[2], fid[2], n;
+    w::map<Frag>(tid, fid, n, e / L::cols, e % L::cols);
+    map_tid[e] = n == 1 ? int(tid[0]) : -1;
+    map_fid[e] = n == 1 ? int(fid[0]) : -1;
+  }
+}
+
+// --------------------------------------------------------------------------
+// One-wave TCEC matrix product, m x n x k in one tcec::fragment each.
+// A is m x k, B is k x n, C/D are m x n; memory layouts are run-time flags
+// (1 = column major) and the leading dimensions are the dense ones.
+// rounding: 0 = mma_sync (policy default), 1 = mma_rn_sync, 2 = mma_rz_sync.
+// --------------------------------------------------------------------------
+template <int m, int n, int k, class T, class Policy, class AL, class BL>
+__global__ void __launch_bounds__(64)
+    tcec_mma_tile_kernel(float *const d, const float *const a,
+                         const float *const b, const float *const c,
+                         const int a_col, const int b_col, const int c_col,
+                         const int d_col, const int rounding) {
+  tcec::fragment<w::matrix_a, m, n, k, T, AL, Policy> fa;
+  tcec::fragment<w::matrix_b, m, n, k, T, BL, Policy> fb;
+  tcec::fragment<w::accumulator, m, n, k, T, void, Policy> fc, fd;
+
+  if (a_col)
+    tcec::load_matrix_sync<w::col_major>(fa, a, m);
+  else
+    tcec::load_matrix_sync<w::row_major>(fa, a, k);
+  if (b_col)
+    tcec::load_matrix_sync<w::col_major>(fb, b, k);
+  else
+    tcec::load_matrix_sync<w::row_major>(fb, b, n);
+
+  if (c != nullptr) {
+    tcec::load_matrix_sync(fc, c, c_col ? m : n,
+                           c_col ? w::mem_col_major : w::mem_row_major);
+    if (rounding == 1)
+      tcec::mma_rn_sync(fd, fa, fb, fc);
+    else if (rounding == 2)
+      tcec::mma_rz_sync(fd, fa, fb, fc);
+    else
+      tcec::mma_sync(fd, fa, fb, fc);
+  } else {
+    if (rounding == 1)
+      tcec::mma_rn_sync(fd, fa, fb);
+    else if (rounding == 2)
+      tcec::mma_rz_sync(fd, fa, fb);
+    else
+      tcec::mma_sync(fd, fa, fb);
+  }
+  tcec::store_matrix_sync(d, fd, d_col ? m : n,
+                          d_col ? w::mem_col_major : w::mem_row_major);
+}
+
+// Same product with the operand memory layout taken from the fragment Layout
+// (the load_matrix_sync overload without a MatrixLayout argument).
+template <int m, int n, int k, class T, class Policy, class AL, class BL>
+__global__ void __launch_bounds__(64)
+    tcec_mma_tile_native_kernel(float *const d, const float *const a,
+                                const float *const b, const int d_col) {
+  tcec::fragment<w::matrix_a, m, n, k, T, AL, Policy> fa;
+  tcec::fragment<w::matrix_b, m, n, k, T, BL, Policy> fb;
+  tcec::fragment<w::accumulator, m, n, k, T, void, Policy> fd;
+  tcec::load_matrix_sync(fa, a, std::is_same<AL, w::col_major>::value ? m : k);
+  tcec::load_matrix_sync(fb, b, std::is_same<BL, w::col_major>::value ? k : n);
+  tcec::mma_sync(fd, fa, fb);
+  tcec::store_matrix_sync(d, fd, d_col ? m : n,
+                          d_col ? w::mem_col_major : w::mem_row_major);
+}
+
+// --------------------------------------------------------------------------
+// y = A * x with x loaded by tcec::load_vector into the first column of a
+// matrix_b fragment and y read back with tcec::store_vector (col), or
+// y^T = x^T * A with x in the first row of a matrix_a fragment (row).
+// A is N x N; a_col gives its memory layout.
+// --------------------------------------------------------------------------
+template <int N, class T, class Policy>
+__global__ void __launch_bounds__(64)
+    tcec_matvec_kernel(float *const y, const float *const a,
+                       const float *const x, const int a_col,
+                       const int left_vector) {
+  tcec::fragment<w::accumulator, N, N, N, T, void, Policy> fc;
+  tcec::fill_zero(fc);
+  if (!left_vector) {
+    tcec::fragment<w::matrix_a, N, N, N, T, w::row_major, Policy> fa;
+    tcec::fragment<w::matrix_b, N, N, N, T, w::col_major, Policy> fx;
+    tcec::fill_zero(fx);
+    if (a_col)
+      tcec::load_matrix_sync<w::col_major>(fa, a, N);
+    else
+      tcec::load_matrix_sync<w::row_major>(fa, a, N);
+    tcec::load_vector(fx, x);
+    tcec::mma_sync(fc, fa, fx, fc);
+    tcec::store_vector(y, fc, w::mem_col_major);
+  } else {
+    tcec::fragment<w::matrix_a, N, N, N, T, w::row_major, Policy> fx;
+    tcec::fragment<w::matrix_b, N, N, N, T, w::col_major, Policy> fa;
+    tcec::fill_zero(fx);
+    if (a_col)
+      tcec::load_matrix_sync<w::col_major>(fa, a, N);
+    else
+      tcec::load_matrix_sync<w::row_major>(fa, a, N);
+    tcec::load_vector(fx, x);
+    tcec::mma_sync(fc, fx, fa, fc);
+    tcec::store_vector(y, fc, w::mem_row_major);
+  }
+}
+
+// --------------------------------------------------------------------------
+// Raw split terms of an operand fragment.  src is a dense N x N fp32 matrix
+// (or an N vector when from_vector != 0).  Output, 16-bit patterns:
+//   terms[(term*num_elements + e)*64 + lane],  e = flat element index x(e)
+// --------------------------------------------------------------------------
+template <class Use, int N, class T, class Policy, class Layout>
+__global__ void __launch_bounds__(64)
+    tcec_frag_dump_kernel(unsigned short *const terms, const float *const src,
+                          const int from_vector, const int mem_col) {
+  using F = tcec::fragment<Use, N, N, N, T, Layout, Policy>;
+  F f;
+  tcec::fill_zero(f);
+  if (from_vector) {
+    tcec::load_vector(f, src);
+  } else {
+    if (mem_col)
+      tcec::load_matrix_sync<w::col_major>(f, src, N);
+    else
+      tcec::load_matrix_sync<w::row_major>(f, src, N);
+  }
+  const unsigned lane = w::detail::common::get_lane_id();
+  for (unsigned e = 0; e < F::num_elements; e++) {
+    const unsigned b = e / F::sub_frag_t::num_elements;
+    const unsigned r = e % F::sub_frag_t::num_elements;
+    terms[(0 * F::num_elements + e) * 64 + lane] =
+        __builtin_bit_cast(unsigned short, f.sub_frag[b].x[r]);
+    if constexpr (F::num_terms >= 2)
+      terms[(1 * F::num_elements + e) * 64 + lane] =
+          __builtin_bit_cast(unsigned short, f.sub_d_frag[b].x[r]);
+    if constexpr (F::num_terms >= 3)
+      terms[(2 * F::num_elements + e) * 64 + lane] =
+          __builtin_bit_cast(unsigned short, f.sub_d2_frag[b].x[r]);
+  }
+}
+
+// --------------------------------------------------------------------------
+// One MFMA on caller-supplied bit patterns: D = A*B + C.
+// a: M x K row-major 16-bit patterns, b: K x N row-major, c/d: M x N row-major fp32.
+// Used to measure the matrix core's accumulate rounding and subnormal handling
+// and to check the layout model against silicon.
+// --------------------------------------------------------------------------
+template <class T, int M, int N, int K>
+__global__ void __launch_bounds__(64)
+    mfma_probe_kernel(float *const d, const unsigned short *const a,
+                      const unsigned short *const b, const float *const c) {
+  using S = typename w::detail::common::storage_t<T>::type;
+  w::fragment<w::matrix_a, M, N, K, T, w::row_major> fa;
+  w::fragment<w::matrix_b, M, N, K, T, w::row_major> fb;
+  w::fragment<w::accumulator, M, N, K, float> fc;
+  w::foreach_ij<decltype(fa)>([&](const unsigned *list, const unsigned,
+                                  const unsigned i, const unsigned j) {
+    fa.x[list[0]] = __builtin_bit_cast(S, a[i * K + j]);
+  });
+  w::foreach_ij<decltype(fb)>([&](const unsigned *list, const unsigned,
+                                  const unsigned i, const unsigned j) {
+    fb.x[list[0]] = __builtin_bit_cast(S, b[i * N + j]);
+  });
+  w::load_matrix_sync(fc, c, N, w::mem_row_major);
+  w::mma_sync(fc, fa, fb, fc);
+  w::store_matrix_sync(d, fc, N, w::mem_row_major);
+}
+
+} // namespace wmmae_harness

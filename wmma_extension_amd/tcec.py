@@ -1,0 +1,204 @@
+"""Host-side calls into the gfx950 TCEC library, on torch CUDA tensors.
+
+torch is used for device memory and streams only; all arithmetic happens in
+the HIP kernels behind the C-ABI (include/wmmae_tcec.h).  The functions keep
+the argument meaning of the reference's GEMM harness
+(test/tcec/batch_gemm.cu:433-443: m, n, k, alpha, A, lda, B, ldb, beta, C, ldc,
+batch) and of its one-warp test kernels.
+"""
+import ctypes
+import enum
+
+import torch
+
+from . import _lib
+
+
+class Policy(enum.IntEnum):
+    """Arithmetic policies (reference: tcec/detail/policy.hpp:50-99)."""
+    F16_EC = 0      # half, with_ec
+    F16_NOEC = 1    # half, without_ec
+    BF16X3_EC = 2   # tf32 policy carried by a three-term bf16 split
+    BF16X2_EC = 3   # bfloat16, with_ec (two terms)
+    BF16_NOEC = 4   # bfloat16, without_ec
+
+
+FLAG_RN_MAIN = 1
+
+TYPE_HALF, TYPE_BF16, TYPE_TF32 = 0, 1, 2
+USE_A, USE_B, USE_ACC = 0, 1, 2
+
+
+def _stream():
+    return ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
+
+
+def _ptr(t):
+    return ctypes.c_void_p(t.data_ptr()) if t is not None else ctypes.c_void_p(0)
+
+
+def _f(v):
+    return ctypes.byref(ctypes.c_float(float(v)))
+
+
+def _need_cuda(*tensors):
+    for t in tensors:
+        if t is not None and not t.is_cuda:
+            raise ValueError("device tensors required")
+
+
+def query(what):
+    out = ctypes.c_longlong(0)
+    _lib.check(_lib.lib().wmmae_query(int(what), ctypes.byref(out)), "wmmae_query")
+    return out.value
+
+
+def workspace_bytes(m, n, k, batch=1, policy=Policy.F16_EC):
+    out = ctypes.c_size_t(0)
+    _lib.check(_lib.lib().wmmae_tcec_sgemm_workspace_bytes(m, n, k, batch, int(policy),
+                                                           ctypes.byref(out)),
+               "wmmae_tcec_sgemm_workspace_bytes")
+    return out.value
+
+
+def pack_bytes(rows, k, batch=1, policy=Policy.F16_EC):
+    out = ctypes.c_size_t(0)
+    _lib.check(_lib.lib().wmmae_tcec_pack_bytes(rows, k, batch, int(policy), ctypes.byref(out)),
+               "wmmae_tcec_pack_bytes")
+    return out.value
+
+
+def sgemm(transa, transb, m, n, k, alpha, A, lda, B, ldb, beta, C, ldc,
+          policy=Policy.F16_EC, flags=0, workspace=None):
+    """C = alpha*op(A)*op(B) + beta*C, column-major BLAS convention."""
+    _need_cuda(A, B, C, workspace)
+    ws_bytes = workspace.numel() * workspace.element_size() if workspace is not None else 0
+    st = _lib.lib().wmmae_tcec_sgemm(transa.encode(), transb.encode(), m, n, k, _f(alpha),
+                                     _ptr(A), lda, _ptr(B), ldb, _f(beta), _ptr(C), ldc,
+                                     int(policy), flags, _ptr(workspace), ws_bytes, _stream())
+    _lib.check(st, "wmmae_tcec_sgemm")
+
+
+def sgemm_strided_batched(transa, transb, m, n, k, alpha, A, lda, stride_a, B, ldb, stride_b,
+                          beta, C, ldc, stride_c, batch, policy=Policy.F16_EC, flags=0,
+                          workspace=None):
+    _need_cuda(A, B, C, workspace)
+    ws_bytes = workspace.numel() * workspace.element_size() if workspace is not None else 0
+    st = _lib.lib().wmmae_tcec_sgemm_strided_batched(
+        transa.encode(), transb.encode(), m, n, k, _f(alpha), _ptr(A), lda, stride_a,
+        _ptr(B), ldb, stride_b, _f(beta), _ptr(C), ldc, stride_c, batch, int(policy), flags,
+        _ptr(workspace), ws_bytes, _stream())
+    _lib.check(st, "wmmae_tcec_sgemm_strided_batched")
+
+
+def pack(policy, rows, k, X, row_stride, k_stride, packed, batch=1, batch_stride=0):
+    _need_cuda(X, packed)
+    st = _lib.lib().wmmae_tcec_pack(int(policy), rows, k, _ptr(X), row_stride, k_stride,
+                                    batch_stride, batch, _ptr(packed),
+                                    packed.numel() * packed.element_size(), _stream())
+    _lib.check(st, "wmmae_tcec_pack")
+
+
+def gemm_packed(policy, m, n, k, alpha, packed_a, packed_b, beta, C, ldc, batch=1,
+                stride_c=0, flags=0):
+    _need_cuda(packed_a, packed_b, C)
+    st = _lib.lib().wmmae_tcec_gemm_packed(int(policy), m, n, k, _f(alpha), _ptr(packed_a),
+                                           _ptr(packed_b), _f(beta), _ptr(C), ldc, stride_c,
+                                           batch, flags, _stream())
+    _lib.check(st, "wmmae_tcec_gemm_packed")
+
+
+def matmul_tn(A, B, policy=Policy.F16_EC, flags=0, workspace=None, out=None):
+    """The reference harness layout: A is (m,k) row-major, B is given as (n,k)
+    row-major (= k x n column-major), result (n,m) row-major (= m x n column-major,
+    ldc = m).  Returns the tensor holding C column-major, i.e. C^T as a torch view."""
+    m, k = A.shape
+    n, k2 = B.shape
+    assert k == k2 and A.is_contiguous() and B.is_contiguous()
+    if out is None:
+        out = torch.empty((n, m), dtype=torch.float32, device=A.device)
+    sgemm("T", "N", m, n, k, 1.0, A, k, B, k, 0.0, out, m, policy, flags, workspace)
+    return out
+
+
+# --------------------------------------------------------------- harness
+def primitive_tiles(tiles):
+    """tiles: (T,256) fp32.  Returns dict of the per-tile outputs."""
+    _need_cuda(tiles)
+    T = tiles.shape[0]
+    dev = tiles.device
+    out = {
+        "a_row": torch.empty((T, 64, 4), dtype=torch.float16, device=dev),
+        "a_col": torch.empty((T, 64, 4), dtype=torch.float16, device=dev),
+        "b_row": torch.empty((T, 64, 4), dtype=torch.float16, device=dev),
+        "b_col": torch.empty((T, 64, 4), dtype=torch.float16, device=dev),
+        "acc": torch.empty((T, 256), dtype=torch.float32, device=dev),
+        "vec": torch.empty((T, 32), dtype=torch.float32, device=dev),
+    }
+    st = _lib.lib().wmmae_primitive_tiles(_ptr(tiles), T, _ptr(out["a_row"]), _ptr(out["a_col"]),
+                                          _ptr(out["b_row"]), _ptr(out["b_col"]),
+                                          _ptr(out["acc"]), _ptr(out["vec"]), _stream())
+    _lib.check(st, "wmmae_primitive_tiles")
+    return out
+
+
+def layout_dump(use, m, n, k, col, device="cuda"):
+    rows = k if use == USE_B else m
+    cols = k if use == USE_A else n
+    R = rows * cols // 64
+    ij = torch.full((64, R, 2), -7, dtype=torch.int32, device=device)
+    mem = torch.full((64, R), -7, dtype=torch.int32, device=device)
+    vidx = torch.full((64, R), -7, dtype=torch.int32, device=device)
+    tid = torch.full((rows, cols), -7, dtype=torch.int32, device=device)
+    fid = torch.full((rows, cols), -7, dtype=torch.int32, device=device)
+    st = _lib.lib().wmmae_layout_dump(use, m, n, k, int(col), _ptr(ij), _ptr(mem), _ptr(vidx),
+                                      _ptr(tid), _ptr(fid), _stream())
+    _lib.check(st, "wmmae_layout_dump")
+    return ij, mem, vidx, tid, fid
+
+
+def mma_tile(shape, type_, ec, inst, a, b, c, a_col, b_col, c_col, d_col, rounding, d):
+    _need_cuda(a, b, c, d)
+    st = _lib.lib().wmmae_tcec_mma_tile(shape, type_, int(ec), inst, _ptr(d), _ptr(a), _ptr(b),
+                                        _ptr(c), int(a_col), int(b_col), int(c_col), int(d_col),
+                                        rounding, _stream())
+    _lib.check(st, "wmmae_tcec_mma_tile")
+    return d
+
+
+def mma_tile_native(type_, ec, a_frag_col, b_frag_col, a, b, d_col, d):
+    _need_cuda(a, b, d)
+    st = _lib.lib().wmmae_tcec_mma_tile_native(type_, int(ec), int(a_frag_col), int(b_frag_col),
+                                               _ptr(d), _ptr(a), _ptr(b), int(d_col), _stream())
+    _lib.check(st, "wmmae_tcec_mma_tile_native")
+    return d
+
+
+def matvec(type_, ec, a, x, a_col, left_vector):
+    _need_cuda(a, x)
+    y = torch.empty(32, dtype=torch.float32, device=a.device)
+    st = _lib.lib().wmmae_tcec_matvec(type_, int(ec), _ptr(y), _ptr(a), _ptr(x), int(a_col),
+                                      int(left_vector), _stream())
+    _lib.check(st, "wmmae_tcec_matvec")
+    return y
+
+
+def frag_dump(use, type_, ec, frag_col, src, from_vector, mem_col):
+    _need_cuda(src)
+    terms = 1 if not ec else (3 if type_ == TYPE_TF32 else 2)
+    E = 32 * 32 // 64
+    out = torch.zeros((terms, E, 64), dtype=torch.int16, device=src.device)
+    st = _lib.lib().wmmae_tcec_frag_dump(use, type_, int(ec), int(frag_col), _ptr(out), _ptr(src),
+                                         int(from_vector), int(mem_col), _stream())
+    _lib.check(st, "wmmae_tcec_frag_dump")
+    return out
+
+
+def mfma_probe(type_, m, n, k, a_bits, b_bits, c):
+    """a_bits (m,k) / b_bits (k,n): int16 tensors of raw 16-bit patterns; c (m,n) fp32."""
+    _need_cuda(a_bits, b_bits, c)
+    d = torch.empty((m, n), dtype=torch.float32, device=c.device)
+    st = _lib.lib().wmmae_mfma_probe(type_, m, n, k, _ptr(d), _ptr(a_bits), _ptr(b_bits), _ptr(c),
+                                     _stream())
+    _lib.check(st, "wmmae_mfma_probe")
+    return d
