@@ -1,0 +1,199 @@
+#!/usr/bin/env python3
+"""Benchmark of the TCEC SGEMM hot path on one MI355X.
+
+One "step" = one full product C = A*B on synthetic seeded fp32 inputs that are
+already resident in HBM: split+pack of A, split+pack of B, MFMA GEMM (the
+workspace for the packed operands is allocated once, outside the timed region).
+
+Prints ONE JSON line: effective fp32 TFLOPS (2*M*N*K*batch / t), the MFMA
+roofline of the GEMM kernel measured with HIP events inside the timed region,
+the accuracy against an FP64 reference on a row sample, and the CPU oracle's
+plain fp32 GEMM timed on the host cores.
+"""
+import argparse
+import json
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, ROOT)
+
+WORKLOADS = {
+    # name: (M, N, K, batch, policy name, distribution, MFMA flop multiplier)
+    "c3": dict(m=4096, n=4096, k=4096, batch=1, policy="F16_EC", dist="uniform", mult=3,
+               desc="TCEC SGEMM fp16 hi+lo with EC, M=N=K=4096, A row-major, B col-major"),
+    "c4": dict(m=16384, n=16384, k=16384, batch=1, policy="BF16X3_EC", dist="exp", mult=6,
+               desc="TCEC SGEMM bf16 three-term split (tf32-policy replacement), M=N=K=16384"),
+    "c4f16": dict(m=16384, n=16384, k=16384, batch=1, policy="F16_EC", dist="uniform", mult=3,
+                  desc="TCEC SGEMM fp16 hi+lo with EC, M=N=K=16384"),
+    "c5a": dict(m=256, n=256, k=256, batch=1024, policy="F16_EC", dist="normal", mult=3,
+                desc="strided-batched TCEC SGEMM, 1024 x 256^3"),
+    "c5b": dict(m=1024, n=1024, k=262144, batch=1, policy="F16_EC", dist="normal", mult=3,
+                desc="K-heavy TCEC SGEMM, M=N=1024, K=262144"),
+}
+PEAK_MFMA_TFLOPS = 2500.0      # dense fp16 / bf16 MFMA, MI355X
+PEAK_HBM_GBS = 8000.0
+
+
+def make_inputs(torch, w, dev, seed):
+    g = torch.Generator(device=dev)
+    g.manual_seed(seed)
+    shape_a = (w["batch"], w["m"], w["k"])
+    shape_b = (w["batch"], w["n"], w["k"])
+
+    def draw(shape):
+        if w["dist"] == "uniform":
+            return torch.rand(shape, generator=g, device=dev, dtype=torch.float32) * 2 - 1
+        if w["dist"] == "normal":
+            return torch.randn(shape, generator=g, device=dev, dtype=torch.float32)
+        # +-x * 2^e, x ~ U[1,2), e ~ U{-15..15}
+        x = torch.rand(shape, generator=g, device=dev, dtype=torch.float32) + 1
+        e = torch.randint(-15, 16, shape, generator=g, device=dev).to(torch.float32)
+        s = torch.randint(0, 2, shape, generator=g, device=dev).to(torch.float32) * 2 - 1
+        return s * x * torch.exp2(e)
+    return draw(shape_a), draw(shape_b)
+
+
+def accuracy_sample(torch, orc, A, Bt, Ct, rows):
+    """max|C - C64| / max|C64| on `rows` full rows of batch 0, for TCEC and for
+    the plain fp32 loop on the same inputs."""
+    import numpy as np
+    m = A.shape[1]
+    g = torch.Generator().manual_seed(1234)
+    idx = torch.randperm(m, generator=g)[:rows].sort().values
+    a = A[0][idx.to(A.device)].cpu().numpy()
+    bt = Bt[0].cpu().numpy()
+    c = Ct[0][:, idx.to(Ct.device)].cpu().numpy().T          # (rows, n)
+    ref = orc.gemm_f64(a, bt.T)
+    c32 = orc.gemm_f32_tn(a, bt).T
+    return orc.max_rel_err(np.ascontiguousarray(c), ref), orc.max_rel_err(np.ascontiguousarray(c32), ref)
+
+
+def cpu_baseline(orc, w, target_s=15.0):
+    """Plain fp32 GEMM loop of the oracle on the host cores, on a sample of the
+    workload sized for about target_s seconds (full K, a square block of C)."""
+    import numpy as np
+    rng = np.random.default_rng(1)
+    k = min(w["k"], 16384)
+    probe = 256
+    a = rng.uniform(-1, 1, (probe, k)).astype(np.float32)
+    b = rng.uniform(-1, 1, (probe, k)).astype(np.float32)
+    t0 = time.perf_counter()
+    orc.gemm_f32_tn(a, b)
+    dt = time.perf_counter() - t0
+    rate = 2.0 * probe * probe * k / dt
+    side = int((rate * target_s / (2.0 * k)) ** 0.5)
+    side = max(256, min(side, w["m"], w["n"], 8192) // 64 * 64)
+    a = rng.uniform(-1, 1, (side, k)).astype(np.float32)
+    b = rng.uniform(-1, 1, (side, k)).astype(np.float32)
+    best = None
+    for _ in range(2):
+        t0 = time.perf_counter()
+        orc.gemm_f32_tn(a, b)
+        dt = time.perf_counter() - t0
+        best = dt if best is None else min(best, dt)
+    return {"value": 2.0 * side * side * k / best / 1e12, "unit": "TFLOPS", "cores": orc.num_threads(),
+            "kind": "port",
+            "sample": f"fp32 triple loop (OpenMP collapse(2), float accumulator) on a {side}x{side}x{k} "
+                      f"block of the workload, best of 2, {best:.2f} s"}
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=10)
+    ap.add_argument("--warmup", type=int, default=2)
+    ap.add_argument("--workload", default="c4", choices=sorted(WORKLOADS))
+    ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
+    ap.add_argument("--no-accuracy", action="store_true")
+    ap.add_argument("--flags", type=int, default=0)
+    args = ap.parse_args()
+    if args.gpus != 1:
+        print("bench.py: this build measures one GPU only; --gpus must be 1 "
+              "(the path shards by C blocks / batch with no exchange, see DESIGN.md)", file=sys.stderr)
+        sys.exit(2)
+
+    import torch
+    from wmma_extension_amd import _lib, tcec
+    _lib.lib()
+    dev = torch.device("cuda:0")
+    torch.cuda.set_device(dev)
+    w = WORKLOADS[args.workload]
+    policy = tcec.Policy[w["policy"]]
+    m, n, k, batch = w["m"], w["n"], w["k"], w["batch"]
+
+    A, Bt = make_inputs(torch, w, dev, 0x5EED + 3)
+    Ct = torch.empty((batch, n, m), dtype=torch.float32, device=dev)
+    pa = torch.empty(tcec.pack_bytes(m, k, batch, policy), dtype=torch.uint8, device=dev)
+    pb = torch.empty(tcec.pack_bytes(n, k, batch, policy), dtype=torch.uint8, device=dev)
+
+    def step(ev=None):
+        tcec.pack(policy, m, k, A, k, 1, pa, batch, m * k)
+        tcec.pack(policy, n, k, Bt, k, 1, pb, batch, n * k)
+        if ev is not None:
+            ev[0].record()
+        tcec.gemm_packed(policy, m, n, k, 1.0, pa, pb, 0.0, Ct, m, batch, n * m, args.flags)
+        if ev is not None:
+            ev[1].record()
+
+    for _ in range(args.warmup):
+        step()
+    torch.cuda.synchronize()
+    events = [(torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True))
+              for _ in range(args.steps)]
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for i in range(args.steps):
+        step(events[i])
+    torch.cuda.synchronize()
+    elapsed = time.perf_counter() - t0
+
+    flops = 2.0 * m * n * k * batch
+    ms_per_step = elapsed / args.steps * 1e3
+    value = flops / (elapsed / args.steps) / 1e12
+    gemm_ms = sum(e0.elapsed_time(e1) for e0, e1 in events) / args.steps
+    achieved = flops * w["mult"] / (gemm_ms * 1e-3) / 1e12
+    bytes_min = 4.0 * (m * k + k * n + m * n) * batch
+
+    out = {
+        "metric": "TCEC SGEMM effective fp32 TFLOPS",
+        "value": round(value, 3),
+        "unit": "TFLOPS",
+        "n_gpus": 1,
+        "steps": args.steps,
+        "warmup": args.warmup,
+        "ms_per_step": round(ms_per_step, 4),
+        "higher_is_better": True,
+        "scaling": "weak",
+        "vs_baseline": None,
+        "dtype": "bf16" if "BF16" in w["policy"] else "f16",
+        "data": "synthetic",
+        "config": {"workload": f"{args.workload}: {w['desc']}", "m": m, "n": n, "k": k, "batch": batch,
+                   "policy": w["policy"], "distribution": w["dist"], "flags": args.flags,
+                   "step": "split+pack A, split+pack B, MFMA GEMM; inputs and workspace resident in HBM"},
+        "roofline": {"bound": "mfma", "achieved": round(achieved, 2), "peak": PEAK_MFMA_TFLOPS,
+                     "unit": "TFLOP/s", "frac": round(achieved / PEAK_MFMA_TFLOPS, 4), "traffic": None,
+                     "kernel": "tcec_gemm_kernel", "kernel_ms": round(gemm_ms, 4),
+                     "issued_flop_multiplier": w["mult"],
+                     "hbm_frac_of_min_traffic": round(bytes_min / (gemm_ms * 1e-3) / 1e9 / PEAK_HBM_GBS, 4)},
+        "gemm_only_effective_tflops": round(flops / (gemm_ms * 1e-3) / 1e12, 3),
+        "fp32_vector_peak_tflops": 157.3,
+    }
+    if not args.no_accuracy:
+        from oracle import oracle as orc
+        rows = 64 if k >= 8192 else 256
+        err, err32 = accuracy_sample(torch, orc, A, Bt, Ct, min(rows, m))
+        out["max_rel_err_vs_fp64"] = float(f"{err:.4e}")
+        out["plain_fp32_max_rel_err_vs_fp64"] = float(f"{err32:.4e}")
+        out["accuracy_sample"] = f"{min(rows, m)} seeded full rows of C (batch 0), FP64 host loop"
+    if not args.no_cpu:
+        from oracle import oracle as orc
+        out["cpu_baseline"] = cpu_baseline(orc, w)
+    else:
+        out["cpu_baseline"] = None
+    print(json.dumps(out))
+
+
+if __name__ == "__main__":
+    main()

@@ -1,0 +1,194 @@
+"""The TCEC SGEMM driver (C-ABI) against the CPU oracle: FP64 loop, TCEC
+emulator, plain fp32 comparator, and size-independent properties."""
+import numpy as np
+import pytest
+import torch
+
+pytestmark = pytest.mark.gpu
+
+POL_KIND = {0: (0, True), 1: (0, False), 2: (2, True), 3: (1, True), 4: (1, False)}
+
+
+def _gemm(tc, dev, A, B, policy, alpha=1.0, beta=0.0, C=None, ta="T", tb="N", flags=0,
+          workspace=None, ld_pad=0):
+    """A (m,k), B (k,n) numpy -> C (m,n) numpy, through wmmae_tcec_sgemm.
+    ta/tb choose how the operands are laid out in device memory (BLAS, column major)."""
+    m, k = A.shape
+    n = B.shape[1]
+    # column-major storage of op(A): 'N' -> m x k col-major (= A.T C-order), 'T' -> k x m col-major (= A C-order)
+    a_store = A.T if ta == "N" else A
+    b_store = B.T if tb == "N" else B
+    lda = a_store.shape[1] + ld_pad
+    ldb = b_store.shape[1] + ld_pad
+    ldc = m + ld_pad
+
+    def dev_padded(x, ld):
+        buf = torch.zeros((x.shape[0], ld), dtype=torch.float32, device=dev)
+        buf[:, :x.shape[1]] = torch.from_numpy(np.ascontiguousarray(x)).to(dev)
+        return buf
+    dA, dB = dev_padded(a_store, lda), dev_padded(b_store, ldb)
+    dC = torch.full((n, ldc), 777.0, dtype=torch.float32, device=dev)
+    if C is not None:
+        dC[:, :m] = torch.from_numpy(np.ascontiguousarray(C.T)).to(dev)
+    tc.sgemm(ta, tb, m, n, k, alpha, dA, lda, dB, ldb, beta, dC, ldc, policy, flags, workspace)
+    torch.cuda.synchronize()
+    out = dC.cpu().numpy()
+    if ld_pad:
+        assert (out[:, m:] == 777.0).all()          # padding untouched
+    return out[:, :m].T.copy()
+
+
+def _check(orc, D, A, B, policy, ref=None, C=None, alpha=1.0, beta=0.0):
+    kind, ec = POL_KIND[policy]
+    ref = (alpha * orc.gemm_f64(A, B) + (beta * C if C is not None else 0)) if ref is None else ref
+    err = orc.max_rel_err(D, ref)
+    e32 = orc.max_rel_err((alpha * orc.gemm_f32(A, B) + (beta * C if C is not None else 0))
+                          .astype(np.float32), ref)
+    k = A.shape[1]
+    if ec and kind != 1:
+        # gate: no worse than 2x plain fp32 SGEMM on the same inputs.  For short
+        # sums fp32 itself is nearly exact and the split's own resolution
+        # (2^-22 per product) is what is left, so that floor is allowed there.
+        assert err <= 2 * e32 + (0.0 if k >= 256 else 2.0**-21), (err, e32)
+    elif ec:
+        assert err <= 2.0**-14
+    else:
+        assert err <= (2.0**-9 if kind == 0 else 2.0**-6)
+    return err, e32
+
+
+@pytest.mark.parametrize("policy", [0, 1, 2, 3, 4])
+@pytest.mark.parametrize("mnk", [(128, 128, 128), (256, 128, 64), (64, 64, 32), (512, 256, 160)])
+def test_sgemm_aligned_shapes(tc, orc, dev, policy, mnk):
+    m, n, k = mnk
+    rng = np.random.default_rng(m + n + k + policy)
+    A = rng.uniform(-1, 1, (m, k)).astype(np.float32)
+    B = rng.uniform(-1, 1, (k, n)).astype(np.float32)
+    D = _gemm(tc, dev, A, B, policy)
+    _check(orc, D, A, B, policy)
+    kind, ec = POL_KIND[policy]
+    emu = orc.tcec_matmul(A, B, kind=kind, ec=ec, fk=32, main_outside=False)
+    assert np.abs(D - emu).max() <= 32 * 2.0**-24 * np.abs(emu).max()
+
+
+@pytest.mark.parametrize("policy", [0, 2])
+@pytest.mark.parametrize("mnk", [(1, 1, 1), (17, 5, 3), (100, 37, 77), (129, 255, 33), (300, 200, 100),
+                                 (16, 16, 1000), (1000, 3, 8)])
+def test_sgemm_ragged_shapes(tc, orc, dev, policy, mnk):
+    m, n, k = mnk
+    rng = np.random.default_rng(m * 7 + n * 3 + k + policy)
+    A = rng.uniform(-1, 1, (m, k)).astype(np.float32)
+    B = rng.uniform(-1, 1, (k, n)).astype(np.float32)
+    for ld_pad in (0, 3):
+        D = _gemm(tc, dev, A, B, policy, ld_pad=ld_pad)
+        _check(orc, D, A, B, policy)
+
+
+@pytest.mark.parametrize("policy", [0, 2])
+@pytest.mark.parametrize("trans", ["NN", "NT", "TN", "TT"])
+def test_sgemm_transposes_alpha_beta(tc, orc, dev, policy, trans):
+    m, n, k = 96, 80, 72
+    rng = np.random.default_rng(ord(trans[0]) + 2 * ord(trans[1]) + policy)
+    A = rng.uniform(-1, 1, (m, k)).astype(np.float32)
+    B = rng.uniform(-1, 1, (k, n)).astype(np.float32)
+    C = rng.uniform(-1, 1, (m, n)).astype(np.float32)
+    base = _gemm(tc, dev, A, B, policy, ta="T", tb="N")
+    D = _gemm(tc, dev, A, B, policy, ta=trans[0], tb=trans[1])
+    assert np.array_equal(D, base)               # the layout of the inputs does not change a bit
+    D = _gemm(tc, dev, A, B, policy, alpha=-1.5, beta=0.75, C=C, ta=trans[0], tb=trans[1], ld_pad=4)
+    expect = (np.float32(-1.5) * base + np.float32(0.75) * C).astype(np.float32)
+    assert np.abs(D - expect).max() <= 2.0**-22 * np.abs(expect).max()
+    # beta == 0 must not read C (NaN in C stays out)
+    D = _gemm(tc, dev, A, B, policy, alpha=1.0, beta=0.0, C=np.full((m, n), np.nan, np.float32),
+              ta=trans[0], tb=trans[1])
+    assert np.array_equal(D, base)
+
+
+def test_sgemm_k_zero_and_workspace(tc, orc, dev):
+    m, n = 20, 12
+    C = np.arange(m * n, dtype=np.float32).reshape(m, n)
+    D = _gemm(tc, dev, np.zeros((m, 0), np.float32), np.zeros((0, n), np.float32), 0,
+              alpha=1.0, beta=2.0, C=C)
+    assert np.array_equal(D, 2 * C)
+    rng = np.random.default_rng(3)
+    A = rng.uniform(-1, 1, (64, 64)).astype(np.float32)
+    B = rng.uniform(-1, 1, (64, 64)).astype(np.float32)
+    ws = torch.empty(tc.workspace_bytes(64, 64, 64), dtype=torch.uint8, device=dev)
+    assert np.array_equal(_gemm(tc, dev, A, B, 0, workspace=ws), _gemm(tc, dev, A, B, 0))
+    small = torch.empty(16, dtype=torch.uint8, device=dev)
+    from wmma_extension_amd._lib import WmmaeError
+    with pytest.raises(WmmaeError) as e:
+        _gemm(tc, dev, A, B, 0, workspace=small)
+    assert e.value.status == -5
+
+
+@pytest.mark.parametrize("policy", [0, 2])
+def test_sgemm_exact_inputs_bit_exact(tc, orc, dev, policy):
+    """Small dyadic inputs: all partial sums exact -> result equals the exact product
+    whatever the tiling, for every tile configuration the dispatcher can choose."""
+    rng = np.random.default_rng(8)
+    for m, n, k in ((64, 64, 64), (256, 256, 96), (2048, 4096, 64)):
+        A = (rng.integers(-8, 9, (m, k)) * 0.25).astype(np.float32)
+        B = (rng.integers(-8, 9, (k, n)) * 0.5).astype(np.float32)
+        D = _gemm(tc, dev, A, B, policy)
+        assert np.array_equal(D, (A.astype(np.float64) @ B.astype(np.float64)).astype(np.float32))
+
+
+@pytest.mark.parametrize("policy", [0, 2])
+def test_sgemm_identity_and_scaling_properties(tc, orc, dev, policy):
+    """B = I reproduces A to the split's resolution; scaling an operand by a power
+    of two scales the result exactly (size independent properties)."""
+    rng = np.random.default_rng(12)
+    n = 512
+    A = rng.uniform(-1, 1, (n, n)).astype(np.float32)
+    I = np.eye(n, dtype=np.float32)
+    D = _gemm(tc, dev, A, I, policy)
+    kind, _ = POL_KIND[policy]
+    assert np.array_equal(D, orc.tcec_matmul(A, I, kind=kind, ec=True))
+    assert np.abs(D - A).max() <= 2.0**-21
+    B = rng.uniform(-1, 1, (n, n)).astype(np.float32)
+    D1 = _gemm(tc, dev, A, B, policy)
+    D2 = _gemm(tc, dev, (A * np.float32(4)).astype(np.float32), (B * np.float32(0.5)).astype(np.float32), policy)
+    assert np.array_equal(D2, D1 * np.float32(2))
+
+
+def test_strided_batched(tc, orc, dev):
+    """Independent 64^3 products, N(0,1) entries, reference layout (T,N)."""
+    batch, m, n, k = 5, 64, 48, 80
+    rng = np.random.default_rng(33)
+    A = rng.standard_normal((batch, m, k)).astype(np.float32)
+    Bt = rng.standard_normal((batch, n, k)).astype(np.float32)
+    dA, dB = torch.from_numpy(A).to(dev), torch.from_numpy(Bt).to(dev)
+    dC = torch.zeros((batch, n, m), dtype=torch.float32, device=dev)
+    for policy in (0, 2):
+        tc.sgemm_strided_batched("T", "N", m, n, k, 1.0, dA, k, m * k, dB, k, n * k, 0.0,
+                                 dC, m, n * m, batch, policy)
+        torch.cuda.synchronize()
+        out = dC.cpu().numpy()
+        for b in range(batch):
+            _check(orc, out[b].T, A[b], Bt[b].T, policy)
+
+
+def test_pack_then_gemm_reuses_operands(tc, orc, dev):
+    m, n, k = 128, 64, 96
+    rng = np.random.default_rng(44)
+    A = rng.uniform(-1, 1, (m, k)).astype(np.float32)
+    Bt = rng.uniform(-1, 1, (n, k)).astype(np.float32)
+    dA, dB = torch.from_numpy(A).to(dev), torch.from_numpy(Bt).to(dev)
+    pa = torch.empty(tc.pack_bytes(m, k), dtype=torch.uint8, device=dev)
+    pb = torch.empty(tc.pack_bytes(n, k), dtype=torch.uint8, device=dev)
+    tc.pack(0, m, k, dA, k, 1, pa)
+    tc.pack(0, n, k, dB, k, 1, pb)
+    dC = torch.zeros((n, m), dtype=torch.float32, device=dev)
+    tc.gemm_packed(0, m, n, k, 1.0, pa, pb, 0.0, dC, m)
+    torch.cuda.synchronize()
+    assert np.array_equal(dC.cpu().numpy().T, _gemm(tc, dev, A, Bt.T, 0))
+    # packed operand bytes: lane l of chunk (rb,kt,term) holds row 16*rb + l%16, k 32*kt+8*(l/16)..+7
+    terms = orc.split(0, A)
+    raw = pa.cpu().numpy().view(np.uint16).reshape(m // 16, -1, 2, 64, 8)
+    KT = raw.shape[1]
+    for rb, kt, t, lane in ((0, 0, 0, 0), (3, 1, 1, 37), (7, 2, 0, 63)):
+        r, k0 = 16 * rb + lane % 16, 32 * kt + 8 * (lane // 16)
+        assert np.array_equal(raw[rb, kt, t, lane], terms[t][r, k0:k0 + 8])
+    assert KT == 4                                   # 96/32 = 3 tiles padded to a multiple of 2
+    assert (raw[:, 3] == 0).all()

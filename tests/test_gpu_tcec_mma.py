@@ -1,0 +1,176 @@
+"""One-wave TCEC kernels on the GPU (device API of include/wmma_extension/tcec)
+against the CPU emulator, the FP64 loop and the reference's thresholds."""
+import itertools
+import os
+
+import numpy as np
+import pytest
+import torch
+
+pytestmark = pytest.mark.gpu
+KAT = np.load(os.path.join(os.path.dirname(__file__), "golden", "primitive_kat.npz"))
+TH_EC = float(KAT["threshold_with_ec"])
+TH_NOEC = float(KAT["threshold_without_ec"])
+KIND_OF_TYPE = {0: 0, 1: 1, 2: 2}           # half -> f16 split, bf16 -> bf16x2, tf32 -> bf16x3
+INST_K = {0: 32, 1: 16, 2: 16}
+
+
+def _dims(shape, inst):
+    if shape == 0:
+        return 32, 32, 32
+    return (32, 64, 32) if inst == 2 else (16, 48, 64)
+
+
+def _mem(x, col):
+    """Dense memory image of matrix x in row- or column-major order."""
+    return np.ascontiguousarray(x.T if col else x).reshape(-1)
+
+
+def _run(tc, dev, shape, type_, ec, inst, A, B, C, a_col, b_col, c_col, d_col, rounding):
+    m, n = A.shape[0], B.shape[1]
+    d = torch.full((m * n,), float("nan"), dtype=torch.float32, device=dev)
+    tc.mma_tile(shape, type_, ec, inst, torch.from_numpy(_mem(A, a_col)).to(dev),
+                torch.from_numpy(_mem(B, b_col)).to(dev),
+                None if C is None else torch.from_numpy(_mem(C, c_col)).to(dev),
+                a_col, b_col, c_col, d_col, rounding, d)
+    torch.cuda.synchronize()
+    out = d.cpu().numpy()
+    return out.reshape(n, m).T if d_col else out.reshape(m, n)
+
+
+@pytest.mark.parametrize("type_", [0, 1, 2])
+@pytest.mark.parametrize("ec", [1, 0])
+@pytest.mark.parametrize("inst", [0, 1, 2])
+@pytest.mark.parametrize("shape", [0, 1])
+def test_mma_tile_all_layouts(tc, orc, dev, type_, ec, inst, shape):
+    """Every memory-layout combination of A, B, C, D, with and without C
+    (the matrix of test/tcec/mma.cu:186-3526), seeded uniform[-1,1]."""
+    m, n, k = _dims(shape, inst)
+    rng = np.random.default_rng(1000 * type_ + 100 * ec + 10 * inst + shape)
+    kind = KIND_OF_TYPE[type_]
+    for a_col, b_col, c_col, d_col, with_c in itertools.product((0, 1), repeat=5):
+        A = rng.uniform(-1, 1, (m, k)).astype(np.float32)
+        B = rng.uniform(-1, 1, (k, n)).astype(np.float32)
+        C = rng.uniform(-1, 1, (m, n)).astype(np.float32) if with_c else None
+        D = _run(tc, dev, shape, type_, ec, inst, A, B, C, a_col, b_col, c_col, d_col, 0)
+        ref = orc.gemm_f64(A, B) + (C if with_c else 0)
+        err = orc.max_abs_err(D, ref)
+        emu = orc.tcec_matmul(A, B, C, kind=kind, ec=bool(ec), fk=INST_K[inst],
+                              main_outside=bool(ec))
+        # the emulator sums each instruction exactly; the matrix core may round
+        # inside an instruction, so agreement is to a few fp32 ulps of the result
+        assert np.abs(D - emu).max() <= 16 * 2.0**-24 * max(1.0, np.abs(ref).max()), \
+            (a_col, b_col, c_col, d_col, with_c)
+        if ec and type_ != 1:
+            assert err < TH_EC                       # test/tcec/mma.cu:7-13
+        elif ec:
+            assert err < 1e-3                        # two bf16 terms: ~16 bits
+        else:
+            assert err < (TH_NOEC if type_ == 0 else 8 * TH_NOEC)   # bf16 has 3 fewer bits
+
+
+@pytest.mark.parametrize("type_", [0, 1, 2])
+@pytest.mark.parametrize("ec", [1, 0])
+def test_mma_tile_exact_cases(tc, orc, dev, type_, ec):
+    """Inputs whose partial sums are all exact: bit-exact against the exact product
+    for mma_sync, mma_rn_sync and mma_rz_sync alike."""
+    rng = np.random.default_rng(77)
+    A = (rng.integers(-8, 9, (32, 32)) * 0.25).astype(np.float32)
+    B = (rng.integers(-8, 9, (32, 32)) * 0.5).astype(np.float32)
+    C = rng.integers(-100, 100, (32, 32)).astype(np.float32)
+    exact = (A.astype(np.float64) @ B.astype(np.float64) + C).astype(np.float32)
+    for inst in (0, 1, 2):
+        for rounding in (0, 1, 2):
+            D = _run(tc, dev, 0, type_, ec, inst, A, B, C, 0, 1, 1, 1, rounding)
+            assert np.array_equal(D, exact), (inst, rounding)
+    # identity B returns the recombined split of A
+    eye = np.eye(32, dtype=np.float32)
+    A = rng.uniform(-1, 1, (32, 32)).astype(np.float32)
+    D = _run(tc, dev, 0, type_, ec, 0, A, eye, None, 0, 0, 0, 0, 0)
+    assert np.array_equal(D, orc.tcec_matmul(A, eye, kind=KIND_OF_TYPE[type_], ec=bool(ec)))
+
+
+@pytest.mark.parametrize("type_", [0, 2])
+def test_mma_tile_native_layout_overload(tc, orc, dev, type_):
+    rng = np.random.default_rng(5)
+    for ec, a_fc, b_fc, d_col in itertools.product((1, 0), (0, 1), (0, 1), (0, 1)):
+        A = rng.uniform(-1, 1, (32, 32)).astype(np.float32)
+        B = rng.uniform(-1, 1, (32, 32)).astype(np.float32)
+        d = torch.empty(32 * 32, dtype=torch.float32, device=dev)
+        tc.mma_tile_native(type_, ec, a_fc, b_fc, torch.from_numpy(_mem(A, a_fc)).to(dev),
+                           torch.from_numpy(_mem(B, b_fc)).to(dev), d_col, d)
+        out = d.cpu().numpy()
+        D = out.reshape(32, 32).T if d_col else out.reshape(32, 32)
+        err = orc.max_abs_err(D, orc.gemm_f64(A, B))
+        assert err < (TH_EC if ec else (TH_NOEC if type_ == 0 else 8 * TH_NOEC))
+
+
+@pytest.mark.parametrize("type_", [0, 1, 2])
+@pytest.mark.parametrize("ec", [1, 0])
+def test_matvec(tc, orc, dev, type_, ec):
+    """y = A x and y^T = x^T A through load_vector / store_vector
+    (test/tcec/matvec.cu:21-50; its with_ec gate is 1e-5 as for mma)."""
+    rng = np.random.default_rng(9)
+    for a_col, left in itertools.product((0, 1), (0, 1)):
+        A = rng.uniform(-1, 1, (32, 32)).astype(np.float32)
+        x = rng.uniform(-1, 1, 32).astype(np.float32)
+        y = tc.matvec(type_, ec, torch.from_numpy(_mem(A, a_col)).to(dev),
+                      torch.from_numpy(x).to(dev), a_col, left).cpu().numpy()
+        ref = (x.astype(np.float64) @ A.astype(np.float64)) if left else \
+            (A.astype(np.float64) @ x.astype(np.float64))
+        err = np.abs(y - ref).max()
+        if ec and type_ != 1:
+            assert err < TH_EC
+        elif ec:
+            assert err < 1e-3
+        else:
+            assert err < (TH_NOEC if type_ == 0 else 8 * TH_NOEC)
+
+
+@pytest.mark.parametrize("type_", [0, 1, 2])
+@pytest.mark.parametrize("use", [0, 1])
+def test_fragment_terms_bit_exact(tc, orc, dev, type_, use):
+    """The 16-bit terms a fragment holds after load_matrix_sync equal the oracle's
+    split of the element the layout model assigns to that register, bit for bit;
+    load_vector fills exactly the first column / row (test/tcec/vector.cu:109-199)."""
+    rng = np.random.default_rng(21)
+    kind = KIND_OF_TYPE[type_]
+    N = 32
+    fm = (16, 16, 32)
+    ij = orc.frag_ij_table(use, *fm)             # (64, R, 2) for one sub-fragment
+    R = ij.shape[1]
+    sub_rows, sub_cols = (16, 32) if use == 0 else (32, 16)
+    nbm, nbn = N // sub_rows, N // sub_cols
+    for ec, frag_col, mem_col in itertools.product((1, 0), (0, 1), (0, 1)):
+        X = rng.uniform(-1, 1, (N, N)).astype(np.float32)
+        X[0, 0], X[1, 1], X[2, 3] = 0.0, 2.0**-16, 1.0
+        got = tc.frag_dump(use, type_, ec, frag_col, torch.from_numpy(_mem(X, mem_col)).to(dev),
+                           0, mem_col).cpu().numpy().view(np.uint16)
+        terms = orc.split(kind, X)
+        nterms = got.shape[0]
+        for e in range(nbm * nbn * R):
+            block, reg = divmod(e, R)
+            bm, bn = block % nbm, block // nbm
+            for lane in range(64):
+                i = ij[lane, reg, 0] + bm * sub_rows
+                j = ij[lane, reg, 1] + bn * sub_cols
+                for t in range(nterms):
+                    assert got[t, e, lane] == terms[t][i, j], (ec, frag_col, mem_col, e, lane, t)
+        # load_vector: first column (col_major fragment) or first row (row_major)
+        v = rng.uniform(-1, 1, N).astype(np.float32)
+        gotv = tc.frag_dump(use, type_, ec, frag_col, torch.from_numpy(v).to(dev), 1, 0)
+        gotv = gotv.cpu().numpy().view(np.uint16)
+        dense = np.zeros((N, N), dtype=np.float32)
+        if frag_col:
+            dense[:, 0] = v
+        else:
+            dense[0, :] = v
+        tv = orc.split(kind, dense)
+        for e in range(nbm * nbn * R):
+            block, reg = divmod(e, R)
+            bm, bn = block % nbm, block // nbm
+            for lane in range(64):
+                i = ij[lane, reg, 0] + bm * sub_rows
+                j = ij[lane, reg, 1] + bn * sub_cols
+                for t in range(nterms):
+                    assert gotv[t, e, lane] == tv[t][i, j]
