@@ -36,13 +36,13 @@ def test_status_strings(h):
 def test_sizes_are_host_only(h):
     out = ctypes.c_size_t(0)
     assert h.wmmae_tcec_pack_bytes(16, 32, 1, 0, ctypes.byref(out)) == 0
-    assert out.value == 2 * 2 * 1024            # k tiles padded to 2, two terms
+    assert out.value == 2 * 1024                # one chunk, two terms
     assert h.wmmae_tcec_pack_bytes(4096, 4096, 1, 0, ctypes.byref(out)) == 0
     assert out.value == 4096 * 4096 * 4          # hi + lo = 4 bytes per element
     assert h.wmmae_tcec_pack_bytes(4096, 4096, 1, 2, ctypes.byref(out)) == 0
     assert out.value == 4096 * 4096 * 6
     assert h.wmmae_tcec_pack_bytes(17, 33, 3, 1, ctypes.byref(out)) == 0
-    assert out.value == 3 * 2 * 2 * 1024
+    assert out.value == 3 * 2 * 2 * 1024         # batch 3, 2 row blocks x 2 k tiles, one term
     assert h.wmmae_tcec_sgemm_workspace_bytes(4096, 4096, 4096, 1, 0, ctypes.byref(out)) == 0
     assert out.value == 2 * 4096 * 4096 * 4
     assert h.wmmae_tcec_pack_bytes(16, 32, 1, 9, ctypes.byref(out)) == -1

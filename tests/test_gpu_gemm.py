@@ -18,8 +18,8 @@ def _gemm(tc, dev, A, B, policy, alpha=1.0, beta=0.0, C=None, ta="T", tb="N", fl
     # column-major storage of op(A): 'N' -> m x k col-major (= A.T C-order), 'T' -> k x m col-major (= A C-order)
     a_store = A.T if ta == "N" else A
     b_store = B.T if tb == "N" else B
-    lda = a_store.shape[1] + ld_pad
-    ldb = b_store.shape[1] + ld_pad
+    lda = max(1, a_store.shape[1]) + ld_pad
+    ldb = max(1, b_store.shape[1]) + ld_pad
     ldc = m + ld_pad
 
     def dev_padded(x, ld):
@@ -146,7 +146,10 @@ def test_sgemm_identity_and_scaling_properties(tc, orc, dev, policy):
     kind, _ = POL_KIND[policy]
     assert np.array_equal(D, orc.tcec_matmul(A, I, kind=kind, ec=True))
     assert np.abs(D - A).max() <= 2.0**-21
-    B = rng.uniform(-1, 1, (n, n)).astype(np.float32)
+    # magnitudes in [2^-4, 1): scaling by 4 and 0.5 keeps every fp16 term normal,
+    # so the split commutes with the scaling and the result scales exactly
+    A = (rng.uniform(2.0**-4, 1, (n, n)) * rng.choice([-1, 1], (n, n))).astype(np.float32)
+    B = (rng.uniform(2.0**-4, 1, (n, n)) * rng.choice([-1, 1], (n, n))).astype(np.float32)
     D1 = _gemm(tc, dev, A, B, policy)
     D2 = _gemm(tc, dev, (A * np.float32(4)).astype(np.float32), (B * np.float32(0.5)).astype(np.float32), policy)
     assert np.array_equal(D2, D1 * np.float32(2))
@@ -190,5 +193,18 @@ def test_pack_then_gemm_reuses_operands(tc, orc, dev):
     for rb, kt, t, lane in ((0, 0, 0, 0), (3, 1, 1, 37), (7, 2, 0, 63)):
         r, k0 = 16 * rb + lane % 16, 32 * kt + 8 * (lane // 16)
         assert np.array_equal(raw[rb, kt, t, lane], terms[t][r, k0:k0 + 8])
-    assert KT == 4                                   # 96/32 = 3 tiles padded to a multiple of 2
-    assert (raw[:, 3] == 0).all()
+    assert KT == 3
+    # rows and k beyond the matrix are zero filled
+    m2, k2 = 20, 40
+    p2 = torch.full((tc.pack_bytes(m2, k2),), 0xFF, dtype=torch.uint8, device=dev)
+    tc.pack(0, m2, k2, dA, k, 1, p2)
+    raw2 = p2.cpu().numpy().view(np.uint16).reshape(2, 2, 2, 64, 8)
+    for rb, kt, lane in ((1, 0, 3), (1, 1, 20), (0, 1, 17), (1, 0, 4)):
+        r, k0 = 16 * rb + lane % 16, 32 * kt + 8 * (lane // 16)
+        for t in (0, 1):
+            exp = np.zeros(8, dtype=np.uint16)
+            if r < m2:
+                for x in range(8):
+                    if k0 + x < k2:
+                        exp[x] = terms[t][r, k0 + x]
+            assert np.array_equal(raw2[rb, kt, t, lane], exp)

@@ -55,14 +55,13 @@ inline bool policy_info(const int policy, PolicyInfo &p) {
   }
 }
 
-constexpr int kKtPad = 2; // packed k tiles are padded to a multiple of this
-
 inline long long ceil_div(const long long a, const long long b) {
   return (a + b - 1) / b;
 }
+// packed operand geometry: 16-row blocks, 32-wide k chunks
 inline long long packed_row_blocks(const int rows) { return ceil_div(rows, 16); }
 inline int packed_k_tiles(const int k) {
-  return static_cast<int>(ceil_div(ceil_div(k, 32), kKtPad) * kKtPad);
+  return static_cast<int>(ceil_div(k, 32));
 }
 // u32x4 elements of one packed matrix
 inline long long packed_elems(const int rows, const int k, const int terms) {
@@ -122,12 +121,19 @@ struct GemmArgs {
   hipStream_t stream;
 };
 
-template <class MT, int TERMS, int BM, int BN, int WGM, int WGN, int KS,
-          bool RN>
+// Deepest LDS ring (at most 4 stages) that fits the 160 KiB of a compute unit.
+constexpr int ring_depth(const int bm, const int bn, const int terms) {
+  const int stage_bytes = (bm / 16 + bn / 16) * terms * 1024;
+  const int fit = (160 * 1024) / stage_bytes;
+  return fit > 4 ? 4 : fit;
+}
+
+template <class MT, int TERMS, int BM, int BN, int WGM, int WGN, bool RN>
 int launch_gemm(const GemmArgs &g) {
-  using Cfg = wmmae_gemm::GemmConfig<MT, TERMS, BM, BN, WGM, WGN, KS, RN>;
-  static_assert(kKtPad % KS == 0, "packed K padding must cover KS");
-  auto kernel = wmmae_gemm::tcec_gemm_kernel<MT, TERMS, BM, BN, WGM, WGN, KS, RN>;
+  constexpr int NSTAGE = ring_depth(BM, BN, TERMS);
+  using Cfg = wmmae_gemm::GemmConfig<MT, TERMS, BM, BN, WGM, WGN, NSTAGE, RN>;
+  auto kernel =
+      wmmae_gemm::tcec_gemm_kernel<MT, TERMS, BM, BN, WGM, WGN, NSTAGE, RN>;
   WMMAE_HIP_TRY(hipFuncSetAttribute(reinterpret_cast<const void *>(kernel),
                                     hipFuncAttributeMaxDynamicSharedMemorySize,
                                     Cfg::LDS_BYTES));
@@ -167,11 +173,11 @@ template <class MT, int TERMS, bool RN> int gemm_by_size(const GemmArgs &g) {
       ceil_div(g.m, 128) * ceil_div(g.n, 128) * static_cast<long long>(g.batch);
   if constexpr (TERMS <= 2) {
     if (big >= cus)
-      return launch_gemm<MT, TERMS, 256, 128, 2, 2, 1, RN>(g);
+      return launch_gemm<MT, TERMS, 256, 128, 2, 2, RN>(g);
   }
   if (mid >= cus || (g.m > 64 && g.n > 64))
-    return launch_gemm<MT, TERMS, 128, 128, 2, 2, TERMS == 3 ? 1 : 2, RN>(g);
-  return launch_gemm<MT, TERMS, 64, 64, 2, 2, 2, RN>(g);
+    return launch_gemm<MT, TERMS, 128, 128, 2, 2, RN>(g);
+  return launch_gemm<MT, TERMS, 64, 64, 2, 2, RN>(g);
 }
 
 int gemm_dispatch(const int policy, const int flags, const GemmArgs &g) {

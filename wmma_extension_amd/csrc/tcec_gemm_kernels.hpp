@@ -8,8 +8,8 @@
 // 16-bit terms that are written to HBM already in the register order of the
 // v_mfma_f32_16x16x32 operand ("fragment-major"):
 //
-//   packed[rb][kt][term][lane] : one 16-byte chunk per lane; lane l of the chunk
-//       holds row 16*rb + l%16, k = 32*kt + 8*(l/16) .. +7 of that term
+//   packed[rb][kt][term][lane] : one 16-byte chunk per lane; lane l holds
+//       row 16*rb + l%16, k = 32*kt + 8*(l/16) .. +7 of that term
 //
 // so one 1 KiB chunk is one MFMA operand for a whole wave.  The GEMM kernel
 // then moves chunks HBM -> LDS -> registers with perfectly linear 128-bit
@@ -17,6 +17,12 @@
 // conversion work in its K loop.  Both operands use the same packing
 // ("rows" are the m index for A and the n index for B), so any BLAS
 // transpose combination is handled by the strides given to the split kernel.
+//
+// Why 16x16x32 and not 32x32x16 (same nominal flop rate, half the
+// instructions): the MFMA rate of this chip is power limited as soon as the
+// operands are not constant.  Measured on MI355X, back-to-back MFMAs on random
+// fp16 data sustain 1.87-1.9 PFLOP/s with 16x16x32 and 1.66 PFLOP/s with
+// 32x32x16 (2.4 PFLOP/s on all-zero data for both).
 #pragma once
 #include <wmma_extension/tcec/tcec.hpp>
 
@@ -26,7 +32,25 @@ typedef unsigned u32x4 __attribute__((ext_vector_type(4)));
 typedef float f32x4 __attribute__((ext_vector_type(4)));
 
 constexpr int kChunkRows = 16; // rows per packed chunk (MFMA M / N)
-constexpr int kChunkK = 32;    // k per packed chunk (MFMA K)
+constexpr int kChunkK = 32;    // k per packed chunk (MFMA K) = one pipeline stage
+
+// Compile-time loop: f(std::integral_constant<int, I>) for I in [B, E).
+template <int B, int E, class F>
+__device__ __forceinline__ void static_for(F &&f) {
+  if constexpr (B < E) {
+    f(std::integral_constant<int, B>{});
+    static_for<B + 1, E>(f);
+  }
+}
+// Number of LDS reads that have been issued once `count` MFMAs of a step are
+// out: read r is due after MFMA number (r+1)*span/nfrag.
+__host__ __device__ constexpr int reads_due(const int count, const int span,
+                                            const int nfrag) {
+  int r = 0;
+  while (r < nfrag && ((r + 1) * span) / nfrag <= count)
+    r++;
+  return r;
+}
 
 // --------------------------------------------------------------------------
 // split_pack_kernel: X (fp32, element (r,k) at X[r*row_stride + k*k_stride])
@@ -34,6 +58,7 @@ constexpr int kChunkK = 32;    // k per packed chunk (MFMA K)
 // zero filled, so the GEMM kernel needs no edge handling on its loads.
 //   T      : split tag (half, bfloat16, precision::tf32)
 //   TERMS  : number of terms stored (1 = leading term only, i.e. no correction)
+//   KT     : number of 32-wide k chunks per row block; chunks = row blocks * KT
 // --------------------------------------------------------------------------
 template <class T, int TERMS>
 __global__ void __launch_bounds__(256)
@@ -52,9 +77,9 @@ __global__ void __launch_bounds__(256)
   if (chunk >= chunks)
     return;
   const long long rb = chunk / KT;
-  const int kt = static_cast<int>(chunk - rb * KT);
+  const int kc = static_cast<int>(chunk - rb * KT);
   const long long r = rb * kChunkRows + (lane & 15u);
-  const int k0 = kt * kChunkK + 8 * static_cast<int>(lane >> 4);
+  const int k0 = kc * kChunkK + 8 * static_cast<int>(lane >> 4);
 
   float v[8];
 #pragma unroll
@@ -115,42 +140,59 @@ __global__ void __launch_bounds__(256)
 //
 //   MT      : MFMA element type (_Float16 or __bf16)
 //   TERMS   : stored terms per operand (1, 2 or 3)
-//   BM x BN : block tile, WGM x WGN waves, each wave (BM/WGM) x (BN/WGN)
-//   KS      : 32-wide k steps per LDS stage
+//   BM x BN : block tile, WGM x WGN waves, each wave (BM/WGM) x (BN/WGN),
+//             built from 16x16 MFMA tiles
+//   NSTAGE  : LDS ring depth; one stage is 32 of k.  Stages are filled by
+//             direct global->LDS loads (global_load_lds_dwordx4, no staging
+//             registers).  While stage s is being multiplied out of
+//             registers, stage s+1 is being read from LDS into the second
+//             fragment set and stages s+2 .. s+NSTAGE are in flight from
+//             HBM/L2, which is what covers memory latency with a single
+//             workgroup per compute unit.
 //   RN_MAIN : accumulate the leading product with fp32 adds outside the
 //             matrix core (the reference's mma_rn_sync, tcec/tcec.hpp:673-694)
-//             instead of chaining it through the MFMA accumulator
+//             instead of chaining it through the MFMA accumulator.  The gfx950
+//             matrix core adds with round-to-nearest-even, so chaining is the
+//             default.
 //
-// Products issued per (16x16 tile, k step), all with fp32 accumulation:
+// Products issued per (16x16 tile, 32 of k), all with fp32 accumulation:
 //   TERMS 1: main += a0*b0
-//   TERMS 2: main += a0*b0;  err += a1*b0 + a0*b1
-//   TERMS 3: main += a0*b0;  err += a2*b0 + a0*b2 + a1*b1 + a1*b0 + a0*b1
+//   TERMS 2: err += a1*b0 + a0*b1;                          main += a0*b0
+//   TERMS 3: err += a2*b0 + a0*b2 + a1*b1 + a1*b0 + a0*b1;  main += a0*b0
 // and the result is main + err * inv_scale (reference: tcec.hpp:332-336).
 // The error terms have their own accumulator so that their low-order bits
 // are not rounded away against the much larger main sum.
 //
 // C is column major (element (i,j) at C[i + j*ldc]); an accumulator lane owns
 // four consecutive rows of one column, i.e. one 16-byte store.
+//
+// ABLATE (tuning only, 0 in the library): bit 0 drops the global->LDS requests
+// of the main loop, bit 1 its LDS reads, bit 2 its barriers, bit 3 the wait
+// for the requests, bit 4 the MFMAs, bit 5 makes every block read tile (0,0).
+// Results are then wrong; the variants exist to time the remaining parts.
 // --------------------------------------------------------------------------
-template <class MT, int TERMS, int BM, int BN, int WGM, int WGN, int KS,
+template <class MT, int TERMS, int BM, int BN, int WGM, int WGN, int NSTAGE,
           bool RN_MAIN>
 struct GemmConfig {
   static constexpr int NW = WGM * WGN;
   static constexpr int NTHREADS = NW * 64;
   static constexpr int WM = BM / WGM, WN = BN / WGN;
   static constexpr int MT_ = WM / 16, NT_ = WN / 16;
-  static constexpr int CH_A = (BM / 16) * KS * TERMS; // chunks per stage
-  static constexpr int CH_B = (BN / 16) * KS * TERMS;
+  static constexpr int CH_PER_RB = TERMS; // chunks of one 16-row block
+  static constexpr int CH_A = (BM / 16) * CH_PER_RB; // chunks per stage
+  static constexpr int CH_B = (BN / 16) * CH_PER_RB;
   static constexpr int NCH = CH_A + CH_B;
-  static constexpr int CPW = NCH / NW; // chunks each wave moves per stage
-  static constexpr int STAGES = 2;
-  static constexpr int LDS_BYTES = STAGES * NCH * 1024;
+  static constexpr int CPW = NCH / NW; // chunks each wave requests per stage
+  static constexpr int LDS_BYTES = NSTAGE * NCH * 1024;
   static_assert(NCH % NW == 0, "chunks must divide evenly over the waves");
   static_assert(WM % 16 == 0 && WN % 16 == 0, "wave tile must be MFMA tiles");
+  static_assert(NSTAGE >= 2 && NSTAGE <= 4, "ring depth");
+  static_assert(CPW * NSTAGE < 64, "vmcnt is a 6-bit counter");
+  static_assert(LDS_BYTES <= 160 * 1024, "LDS of one compute unit");
 };
 
-template <class MT, int TERMS, int BM, int BN, int WGM, int WGN, int KS,
-          bool RN_MAIN>
+template <class MT, int TERMS, int BM, int BN, int WGM, int WGN, int NSTAGE,
+          bool RN_MAIN, int ABLATE = 0>
 __global__ void __launch_bounds__(WGM *WGN * 64)
     tcec_gemm_kernel(const u32x4 *__restrict__ Ap, const u32x4 *__restrict__ Bp,
                      float *__restrict__ C, const int M, const int N,
@@ -161,12 +203,12 @@ __global__ void __launch_bounds__(WGM *WGN * 64)
                      const long long batch_stride_a,
                      const long long batch_stride_b,
                      const long long batch_stride_c) {
-  using Cfg = GemmConfig<MT, TERMS, BM, BN, WGM, WGN, KS, RN_MAIN>;
+  using Cfg = GemmConfig<MT, TERMS, BM, BN, WGM, WGN, NSTAGE, RN_MAIN>;
   typedef MT ab_vec __attribute__((ext_vector_type(8)));
   constexpr int NCH = Cfg::NCH, CH_A = Cfg::CH_A, CPW = Cfg::CPW;
   constexpr int MT_ = Cfg::MT_, NT_ = Cfg::NT_;
   constexpr int RBM = BM / 16, RBN = BN / 16;
-  constexpr int CH_PER_RB = KS * TERMS; // contiguous chunks of one row block
+  constexpr int CH_PER_RB = Cfg::CH_PER_RB;
 
   extern __shared__ __attribute__((aligned(16))) unsigned char lds_raw[];
   u32x4 *const lds = reinterpret_cast<u32x4 *>(lds_raw);
@@ -176,8 +218,8 @@ __global__ void __launch_bounds__(WGM *WGN * 64)
   const int wm = wave % WGM, wn = wave / WGM;
 
   // ---- block -> tile: spread consecutive ids over the 8 XCDs, then walk the
-  // tile grid in groups of 8 tile rows so that the blocks resident on one XCD
-  // share A row panels and B column panels in that XCD's L2.
+  // tile grid in groups of GROUP tile rows so that the blocks resident on one
+  // XCD share A row panels and B column panels in that XCD's L2.
   const int num_tiles = tiles_m * tiles_n;
   int pid = blockIdx.x;
   {
@@ -190,7 +232,9 @@ __global__ void __launch_bounds__(WGM *WGN * 64)
   }
   int tm, tn;
   {
-    constexpr int GROUP = 8;
+    // 32 blocks run on one XCD at a time: a GROUP x (32/GROUP) patch of
+    // tiles that is close to square in elements needs the fewest L2 fills
+    constexpr int GROUP = BM > BN ? 4 : 8;
     const int width = GROUP * tiles_n;
     const int group = pid / width;
     const int first_m = group * GROUP;
@@ -199,30 +243,30 @@ __global__ void __launch_bounds__(WGM *WGN * 64)
     tm = first_m + in_group % gsz;
     tn = in_group / gsz;
   }
+  if constexpr ((ABLATE & 32) != 0)
+    tm = tn = 0;
   const long long batch = blockIdx.y;
 
-  // ---- global sources of the chunks this wave moves every stage
+  // ---- global sources of the chunks this wave requests every stage.
   // Row blocks past the end of a packed operand are clamped to the last real
   // one: the rows / columns computed from them are never stored.
   const u32x4 *gsrc[CPW];
-  int slot[CPW];
 #pragma unroll
   for (int q = 0; q < CPW; q++) {
     const int c = wave + Cfg::NW * q; // chunk index inside the stage
-    slot[q] = c;
     if (c < CH_A) {
       const int rbl = c / CH_PER_RB, j = c % CH_PER_RB;
       int rb = tm * RBM + rbl;
       rb = rb < rb_a ? rb : rb_a - 1;
       gsrc[q] = Ap + batch * batch_stride_a +
-                (static_cast<long long>(rb) * KT * TERMS + j) * 64;
+                (static_cast<long long>(rb) * KT * CH_PER_RB + j) * 64;
     } else {
       const int cb = c - CH_A;
       const int rbl = cb / CH_PER_RB, j = cb % CH_PER_RB;
       int rb = tn * RBN + rbl;
       rb = rb < rb_b ? rb : rb_b - 1;
       gsrc[q] = Bp + batch * batch_stride_b +
-                (static_cast<long long>(rb) * KT * TERMS + j) * 64;
+                (static_cast<long long>(rb) * KT * CH_PER_RB + j) * 64;
     }
   }
 
@@ -235,103 +279,174 @@ __global__ void __launch_bounds__(WGM *WGN * 64)
       acc_err[i][j] = f32x4{0.f, 0.f, 0.f, 0.f};
     }
 
-  u32x4 pre[CPW];
-  const int num_stages = KT / KS; // host guarantees KT % KS == 0
-  auto load_global = [&](const int st) {
+  const int num_stages = KT;
+
+  // Request chunk Q (of this wave's CPW chunks) of stage `st` into LDS buffer
+  // `buf`.  The stage is clamped to the last one: the few redundant loads at
+  // the tail keep the in-flight count constant, so one s_waitcnt immediate
+  // serves the whole loop.
+  auto issue_chunk = [&](int st, const int buf, auto Q) {
+    constexpr int q = decltype(Q)::value;
+    st = st < num_stages ? st : num_stages - 1;
     const long long off = static_cast<long long>(st) * (CH_PER_RB * 64) + lane;
-#pragma unroll
-    for (int q = 0; q < CPW; q++)
-      pre[q] = gsrc[q][off];
-  };
-  auto store_lds = [&](const int buf) {
-#pragma unroll
-    for (int q = 0; q < CPW; q++)
-      lds[(buf * NCH + slot[q]) * 64 + lane] = pre[q];
+    const int c = wave + Cfg::NW * q;
+    __builtin_amdgcn_global_load_lds(
+        (const __attribute__((address_space(1))) void *)(gsrc[q] + off),
+        (__attribute__((address_space(3))) void *)(lds_raw +
+                                                   (buf * NCH + c) * 1024),
+        16, 0, 0);
   };
 
-  load_global(0);
-  store_lds(0);
-  __syncthreads();
+  // In-place accumulate, written as inline assembly so that every accumulator
+  // stays in one fixed accumulation register for the whole K loop (with the
+  // largest tile the accumulators fill the register file exactly, and the
+  // register allocator otherwise shuffles them every iteration).  Used only
+  // when a sweep has at least eight tiles: dependent MFMAs on one accumulator
+  // are then at least eight 16-cycle instructions apart, beyond any software
+  // wait state the matrix core needs; smaller wave tiles use the builtin and
+  // leave the hazards to the compiler.
+  constexpr bool USE_ASM = MT_ * NT_ >= 8;
+  auto mfma_acc = [](f32x4 &z, const ab_vec x, const ab_vec y) {
+    if constexpr (std::is_same<MT, _Float16>::value)
+      asm volatile("v_mfma_f32_16x16x32_f16 %0, %1, %2, %0"
+                   : "+a"(z)
+                   : "v"(x), "v"(y));
+    else
+      asm volatile("v_mfma_f32_16x16x32_bf16 %0, %1, %2, %0"
+                   : "+a"(z)
+                   : "v"(x), "v"(y));
+  };
+  auto mfma = [](const ab_vec x, const ab_vec y, const f32x4 z) -> f32x4 {
+    if constexpr (std::is_same<MT, _Float16>::value)
+      return __builtin_amdgcn_mfma_f32_16x16x32_f16(x, y, z, 0, 0, 0);
+    else
+      return __builtin_amdgcn_mfma_f32_16x16x32_bf16(x, y, z, 0, 0, 0);
+  };
 
-  for (int st = 0; st < num_stages; st++) {
-    const int buf = st & 1;
-    if (st + 1 < num_stages)
-      load_global(st + 1);
-
-    const u32x4 *const sa =
-        lds + (buf * NCH + wm * MT_ * CH_PER_RB) * 64 + lane;
-    const u32x4 *const sb =
-        lds + (buf * NCH + CH_A + wn * NT_ * CH_PER_RB) * 64 + lane;
-#pragma unroll
-    for (int ks = 0; ks < KS; ks++) {
-      ab_vec a[TERMS][MT_], b[TERMS][NT_];
-#pragma unroll
-      for (int i = 0; i < MT_; i++)
-#pragma unroll
-        for (int t = 0; t < TERMS; t++)
-          a[t][i] = __builtin_bit_cast(
-              ab_vec, sa[(i * CH_PER_RB + ks * TERMS + t) * 64]);
-#pragma unroll
-      for (int j = 0; j < NT_; j++)
-#pragma unroll
-        for (int t = 0; t < TERMS; t++)
-          b[t][j] = __builtin_bit_cast(
-              ab_vec, sb[(j * CH_PER_RB + ks * TERMS + t) * 64]);
-
-      auto mfma = [](const ab_vec x, const ab_vec y, const f32x4 z) -> f32x4 {
-        if constexpr (std::is_same<MT, _Float16>::value)
-          return __builtin_amdgcn_mfma_f32_16x16x32_f16(x, y, z, 0, 0, 0);
-        else
-          return __builtin_amdgcn_mfma_f32_16x16x32_bf16(x, y, z, 0, 0, 0);
-      };
-      // error terms first (smallest products first), main product last
-      if constexpr (TERMS >= 3) {
-#pragma unroll
-        for (int i = 0; i < MT_; i++)
-#pragma unroll
-          for (int j = 0; j < NT_; j++)
-            acc_err[i][j] = mfma(a[2][i], b[0][j], acc_err[i][j]);
-#pragma unroll
-        for (int i = 0; i < MT_; i++)
-#pragma unroll
-          for (int j = 0; j < NT_; j++)
-            acc_err[i][j] = mfma(a[0][i], b[2][j], acc_err[i][j]);
-#pragma unroll
-        for (int i = 0; i < MT_; i++)
-#pragma unroll
-          for (int j = 0; j < NT_; j++)
-            acc_err[i][j] = mfma(a[1][i], b[1][j], acc_err[i][j]);
-      }
-      if constexpr (TERMS >= 2) {
-#pragma unroll
-        for (int i = 0; i < MT_; i++)
-#pragma unroll
-          for (int j = 0; j < NT_; j++)
-            acc_err[i][j] = mfma(a[1][i], b[0][j], acc_err[i][j]);
-#pragma unroll
-        for (int i = 0; i < MT_; i++)
-#pragma unroll
-          for (int j = 0; j < NT_; j++)
-            acc_err[i][j] = mfma(a[0][i], b[1][j], acc_err[i][j]);
-      }
-#pragma unroll
-      for (int i = 0; i < MT_; i++)
-#pragma unroll
-        for (int j = 0; j < NT_; j++) {
-          if constexpr (RN_MAIN) {
-            const f32x4 tmp =
-                mfma(a[0][i], b[0][j], f32x4{0.f, 0.f, 0.f, 0.f});
-            acc_main[i][j] += tmp;
-          } else {
-            acc_main[i][j] = mfma(a[0][i], b[0][j], acc_main[i][j]);
-          }
-        }
+  // Operand fragments of one stage: TERMS chunks per 16-row block.
+  struct Frags {
+    ab_vec a[TERMS][MT_];
+    ab_vec b[TERMS][NT_];
+  };
+  constexpr int NFRAG = TERMS * (MT_ + NT_);
+  // fragment IDX of a stage (compile-time index, so that every fragment is a
+  // fixed register): B fragments first, then A
+  auto read_frag = [&](Frags &f, const int buf, auto IDX) {
+    constexpr int r = decltype(IDX)::value;
+    if constexpr (r < TERMS * NT_) {
+      constexpr int j = r / TERMS, t = r % TERMS;
+      const u32x4 *const sb =
+          lds + (buf * NCH + CH_A + wn * NT_ * CH_PER_RB) * 64 + lane;
+      f.b[t][j] = __builtin_bit_cast(ab_vec, sb[(j * CH_PER_RB + t) * 64]);
+    } else {
+      constexpr int i = (r - TERMS * NT_) / TERMS, t = (r - TERMS * NT_) % TERMS;
+      const u32x4 *const sa =
+          lds + (buf * NCH + wm * MT_ * CH_PER_RB) * 64 + lane;
+      f.a[t][i] = __builtin_bit_cast(ab_vec, sa[(i * CH_PER_RB + t) * 64]);
     }
+  };
 
-    if (st + 1 < num_stages)
-      store_lds(buf ^ 1);
-    __syncthreads();
+  // MFMAs of one step in issue order: the error products (smallest first) and
+  // then the main product; every product sweeps all tiles before the next one
+  // starts, so consecutive MFMAs never depend on each other.
+  constexpr int NPROD = TERMS == 1 ? 1 : (TERMS == 2 ? 3 : 6);
+  constexpr int NTILE = MT_ * NT_;
+  constexpr int NMFMA = NPROD * NTILE;
+  // LDS read r of the next stage goes out after MFMA number (r+1)*SPAN/NFRAG:
+  // the reads are spread over the first three quarters of the step (the LGKM
+  // counter only tracks 15 outstanding operations)
+  constexpr int SPAN = (NMFMA * 3) / 4 > 0 ? (NMFMA * 3) / 4 : 1;
+
+  // One pipeline step: multiply the fragments of stage st (already in
+  // registers) while the fragments of stage st+1 are read from LDS and stage
+  // st+NSTAGE is requested from HBM.  After the barrier every wave holds
+  // stage st in registers, so its LDS buffer is free for the new request.
+  // Memory instructions are spread between the MFMAs so that the single wave
+  // of a SIMD never sits on a full memory queue while the matrix core idles.
+  auto step = [&](const Frags &cur, Frags &nxt, const int st, const int wbuf,
+                  const int rbuf) {
+    // own loads of stage st+1 landed; own LDS reads of stage st finished
+    if constexpr ((ABLATE & 4) == 0)
+      asm volatile("s_waitcnt vmcnt(%0) lgkmcnt(0)\n\ts_barrier" ::"n"(
+                       (ABLATE & 8) ? 63 : CPW * (NSTAGE - 2))
+                   : "memory");
+
+    static_for<0, NMFMA>([&](auto N_) {
+      constexpr int n = decltype(N_)::value;
+      constexpr int p = n / NTILE;
+      constexpr int i = (n % NTILE) / NT_, j = n % NT_;
+      // (term of A, term of B) of product p
+      constexpr int ta =
+          TERMS == 1   ? 0
+          : TERMS == 2 ? (p == 0 ? 1 : 0)
+                       : (p == 0 ? 2 : p == 1 ? 0 : p == 2 ? 1 : p == 3 ? 1 : 0);
+      constexpr int tb =
+          TERMS == 1   ? 0
+          : TERMS == 2 ? (p == 1 ? 1 : 0)
+                       : (p == 0 ? 0 : p == 1 ? 2 : p == 2 ? 1 : p == 3 ? 0
+                                                           : p == 4   ? 1
+                                                                      : 0);
+      constexpr bool is_main = p == NPROD - 1;
+      if constexpr ((ABLATE & 16) != 0) {
+        // tuning: no matrix work at all
+      } else if constexpr (is_main && RN_MAIN) {
+        acc_main[i][j] +=
+            mfma(cur.a[0][i], cur.b[0][j], f32x4{0.f, 0.f, 0.f, 0.f});
+      } else if constexpr (USE_ASM) {
+        mfma_acc(is_main ? acc_main[i][j] : acc_err[i][j], cur.a[ta][i],
+                 cur.b[tb][j]);
+      } else if constexpr (is_main) {
+        acc_main[i][j] = mfma(cur.a[ta][i], cur.b[tb][j], acc_main[i][j]);
+      } else {
+        acc_err[i][j] = mfma(cur.a[ta][i], cur.b[tb][j], acc_err[i][j]);
+      }
+      // global->LDS requests due after this MFMA
+      constexpr int qlo = (n * CPW + NMFMA - 1) / NMFMA;
+      constexpr int qhi = ((n + 1) * CPW + NMFMA - 1) / NMFMA;
+      static_for<qlo, (qhi < CPW ? qhi : CPW)>([&](auto Q) {
+        if constexpr ((ABLATE & 1) == 0)
+          issue_chunk(st + NSTAGE, wbuf, Q);
+        __builtin_amdgcn_sched_barrier(0);
+      });
+      // LDS reads due after this MFMA
+      constexpr int lo = n == 0 ? 0 : reads_due(n, SPAN, NFRAG);
+      constexpr int hi = n + 1 == NMFMA ? NFRAG : reads_due(n + 1, SPAN, NFRAG);
+      static_for<lo, hi>([&](auto R_) {
+        if constexpr ((ABLATE & 2) == 0)
+          read_frag(nxt, rbuf, R_);
+        __builtin_amdgcn_sched_barrier(0);
+      });
+    });
+  };
+
+  // ---- prologue: request the first NSTAGE stages, fetch stage 0's fragments
+#pragma unroll
+  for (int s = 0; s < NSTAGE; s++)
+    static_for<0, CPW>([&](auto Q) { issue_chunk(s, s, Q); });
+  Frags f0, f1;
+  asm volatile("s_waitcnt vmcnt(%0)\n\ts_barrier" ::"n"(CPW * (NSTAGE - 1))
+               : "memory");
+  static_for<0, NFRAG>([&](auto R_) { read_frag(f0, 0, R_); });
+
+  // ---- main loop, unrolled by two so that the fragment sets swap by name
+  int wbuf = 0; // buffer of the stage being multiplied == next to be refilled
+  auto next_buf = [](const int b2) { return b2 + 1 == NSTAGE ? 0 : b2 + 1; };
+  int st = 0;
+  for (; st + 1 < num_stages; st += 2) {
+    const int b1 = next_buf(wbuf);
+    step(f0, f1, st, wbuf, b1);
+    const int b2 = next_buf(b1);
+    step(f1, f0, st + 1, b1, b2);
+    wbuf = b2;
   }
+  if (st < num_stages)
+    step(f0, f1, st, wbuf, next_buf(wbuf));
+
+  // the redundant tail loads must not outlive the workgroup's LDS allocation;
+  // the no-ops cover the matrix core's write-to-VALU-read distance for the
+  // last accumulate instructions, which the compiler cannot see
+  asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)\n\ts_nop 15\n\ts_nop 15" ::
+                   : "memory");
 
   // ---- epilogue: recombine, scale, store
   float *const Cb = C + batch * batch_stride_c;
