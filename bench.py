@@ -108,6 +108,9 @@ def main():
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--no-accuracy", action="store_true")
     ap.add_argument("--flags", type=int, default=0)
+    ap.add_argument("--calibrate", action="store_true",
+                    help="after the timed region run one 1 GiB read + 1 GiB write elementwise kernel "
+                         "(the known-size copy that rocprofv3 FETCH_SIZE / WRITE_SIZE are scaled with)")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py: this build measures one GPU only; --gpus must be 1 "
@@ -148,6 +151,13 @@ def main():
         step(events[i])
     torch.cuda.synchronize()
     elapsed = time.perf_counter() - t0
+
+    if args.calibrate:
+        src = torch.ones(1 << 28, dtype=torch.float32, device=dev)
+        dst = torch.empty_like(src)
+        torch.add(src, 1.0, out=dst)
+        torch.cuda.synchronize()
+        del src, dst
 
     flops = 2.0 * m * n * k * batch
     ms_per_step = elapsed / args.steps * 1e3
