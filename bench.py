@@ -130,13 +130,15 @@ def main():
     Ct = torch.empty((batch, n, m), dtype=torch.float32, device=dev)
     pa = torch.empty(tcec.pack_bytes(m, k, batch, policy), dtype=torch.uint8, device=dev)
     pb = torch.empty(tcec.pack_bytes(n, k, batch, policy), dtype=torch.uint8, device=dev)
+    ws_bytes = tcec.gemm_packed_workspace_bytes(policy, m, n, k, batch)
+    ws = torch.empty(ws_bytes, dtype=torch.uint8, device=dev) if ws_bytes else None
 
     def step(ev=None):
         tcec.pack(policy, m, k, A, k, 1, pa, batch, m * k)
         tcec.pack(policy, n, k, Bt, k, 1, pb, batch, n * k)
         if ev is not None:
             ev[0].record()
-        tcec.gemm_packed(policy, m, n, k, 1.0, pa, pb, 0.0, Ct, m, batch, n * m, args.flags)
+        tcec.gemm_packed(policy, m, n, k, 1.0, pa, pb, 0.0, Ct, m, batch, n * m, args.flags, ws)
         if ev is not None:
             ev[1].record()
 

@@ -45,6 +45,11 @@ def test_sizes_are_host_only(h):
     assert out.value == 3 * 2 * 2 * 1024         # batch 3, 2 row blocks x 2 k tiles, one term
     assert h.wmmae_tcec_sgemm_workspace_bytes(4096, 4096, 4096, 1, 0, ctypes.byref(out)) == 0
     assert out.value == 2 * 4096 * 4096 * 4
+    # split-K room: none for square problems, slices of C for the K-heavy shape
+    assert h.wmmae_tcec_gemm_packed_workspace_bytes(0, 4096, 4096, 4096, 1, ctypes.byref(out)) == 0
+    assert out.value == 0
+    assert h.wmmae_tcec_gemm_packed_workspace_bytes(0, 1024, 1024, 262144, 1, ctypes.byref(out)) == 0
+    assert out.value > 0 and out.value % (1024 * 1024 * 4) == 0
     assert h.wmmae_tcec_pack_bytes(16, 32, 1, 9, ctypes.byref(out)) == -1
     assert h.wmmae_tcec_pack_bytes(-1, 32, 1, 0, ctypes.byref(out)) == -1
     assert h.wmmae_tcec_pack_bytes(16, 32, 1, 0, None) == -2
@@ -89,11 +94,11 @@ def test_other_entry_points_validate(h):
     assert h.wmmae_tcec_pack(0, 16, 32, p(16), 32, 1, 0, 1, p(24), 4096, None) == -7
     assert h.wmmae_tcec_pack(0, 16, 32, p(16), 32, 1, 0, 1, p(32), 100, None) == -5
     assert h.wmmae_tcec_gemm_packed(0, 16, 16, 32, ctypes.byref(one), p(16), p(16),
-                                    ctypes.byref(one), p(0), 16, 0, 1, 0, None) == -2
+                                    ctypes.byref(one), p(0), 16, 0, 1, 0, None, 0, None) == -2
     assert h.wmmae_tcec_gemm_packed(0, 16, 16, 32, ctypes.byref(one), p(16), p(16),
-                                    ctypes.byref(one), p(16), 8, 0, 1, 0, None) == -3
+                                    ctypes.byref(one), p(16), 8, 0, 1, 0, None, 0, None) == -3
     assert h.wmmae_tcec_gemm_packed(0, 16, 16, 32, ctypes.byref(one), p(8), p(16),
-                                    ctypes.byref(one), p(16), 16, 0, 1, 0, None) == -7
+                                    ctypes.byref(one), p(16), 16, 0, 1, 0, None, 0, None) == -7
     assert h.wmmae_primitive_tiles(p(0), 4, p(0), p(0), p(0), p(0), p(0), p(0), None) == -2
     assert h.wmmae_primitive_tiles(p(0), -1, p(0), p(0), p(0), p(0), p(0), p(0), None) == -1
     assert h.wmmae_layout_dump(0, 16, 16, 16, 0, p(0), p(0), p(0), p(0), p(0), None) == -2

@@ -1,0 +1,106 @@
+"""The BASELINE workloads at their full sizes on the GPU.  The FP64 reference is
+evaluated on a seeded sample of full rows (a full 16384^3 FP64 product is hours of
+CPU); the gate is the north-star one: max relative error no worse than 2x that of a
+plain fp32 GEMM on the same inputs.  Size-independent properties cover the rest."""
+import numpy as np
+import pytest
+import torch
+
+pytestmark = pytest.mark.gpu
+
+
+def _inputs(dev, shape, dist, seed):
+    g = torch.Generator(device=dev)
+    g.manual_seed(seed)
+    if dist == "uniform":
+        return torch.rand(shape, generator=g, device=dev) * 2 - 1
+    if dist == "normal":
+        return torch.randn(shape, generator=g, device=dev)
+    x = torch.rand(shape, generator=g, device=dev) + 1
+    e = torch.randint(-15, 16, shape, generator=g, device=dev).to(torch.float32)
+    s = torch.randint(0, 2, shape, generator=g, device=dev).to(torch.float32) * 2 - 1
+    return s * x * torch.exp2(e)
+
+
+def _check_rows(orc, A, Bt, Ct, rows, seed=7):
+    """A (m,k), Bt (n,k), Ct (n,m) device tensors -> (tcec err, fp32 err) on sampled rows."""
+    m = A.shape[0]
+    idx = torch.randperm(m, generator=torch.Generator().manual_seed(seed))[:rows].sort().values
+    a = A[idx.to(A.device)].cpu().numpy()
+    bt = Bt.cpu().numpy()
+    c = np.ascontiguousarray(Ct[:, idx.to(Ct.device)].cpu().numpy().T)
+    ref = orc.gemm_f64(a, bt.T)
+    c32 = np.ascontiguousarray(orc.gemm_f32_tn(a, bt).T)
+    return orc.max_rel_err(c, ref), orc.max_rel_err(c32, ref), orc.frobenius_residual(c, ref)
+
+
+def test_config3_4096_fp16_ec(tc, orc, dev):
+    """M=N=K=4096, A row-major, B col-major, uniform[-1,1], alpha=1, beta=0."""
+    n = 4096
+    A = _inputs(dev, (n, n), "uniform", 0x5EED + 3)
+    Bt = _inputs(dev, (n, n), "uniform", 0x5EED + 33)
+    Ct = tc.matmul_tn(A, Bt, tc.Policy.F16_EC)
+    torch.cuda.synchronize()
+    err, e32, fro = _check_rows(orc, A, Bt, Ct, 128)
+    assert err <= 2 * e32, (err, e32)
+    assert fro < 5e-7
+    # without error correction the same product is ~1000x less accurate (the gate has teeth)
+    C0 = tc.matmul_tn(A, Bt, tc.Policy.F16_NOEC)
+    err0, _, _ = _check_rows(orc, A, Bt, C0, 16)
+    assert err0 > 50 * err
+    # determinism: a second run gives the same bits
+    assert torch.equal(Ct, tc.matmul_tn(A, Bt, tc.Policy.F16_EC))
+
+
+def test_config4_16384_bf16_three_terms(tc, orc, dev):
+    """M=N=K=16384, values +-x*2^e (x in [1,2), e in -15..15): outside fp16's range,
+    carried by the three-term bf16 split."""
+    n = 16384
+    A = _inputs(dev, (n, n), "exp", 0x5EED + 4)
+    Bt = _inputs(dev, (n, n), "exp", 0x5EED + 44)
+    ws = torch.empty(tc.workspace_bytes(n, n, n, 1, tc.Policy.BF16X3_EC), dtype=torch.uint8, device=dev)
+    Ct = tc.matmul_tn(A, Bt, tc.Policy.BF16X3_EC, workspace=ws)
+    torch.cuda.synchronize()
+    err, e32, fro = _check_rows(orc, A, Bt, Ct, 48)
+    assert err <= 2 * e32, (err, e32)
+    assert fro < 1e-6
+    # linearity in a power of two: (2A) B == 2 (A B) bit for bit (bf16 terms scale exactly)
+    C2 = tc.matmul_tn(A * 2, Bt, tc.Policy.BF16X3_EC, workspace=ws)
+    assert torch.equal(C2, Ct * 2)
+    # the two-term bf16 split carries ~16 bits per element: visibly worse on the same rows
+    # (at this K its rounding errors average out, so the gap is a factor, not orders)
+    C1 = tc.matmul_tn(A, Bt, tc.Policy.BF16X2_EC, workspace=ws)
+    err1, _, _ = _check_rows(orc, A, Bt, C1, 48)
+    assert err1 > 1.3 * err
+
+
+def test_config5a_strided_batched_256(tc, orc, dev):
+    """1024 independent 256x256x256 products, N(0,1) entries."""
+    batch, n = 1024, 256
+    A = _inputs(dev, (batch, n, n), "normal", 0x5EED + 5)
+    Bt = _inputs(dev, (batch, n, n), "normal", 0x5EED + 55)
+    Ct = torch.empty((batch, n, n), device=dev)
+    tc.sgemm_strided_batched("T", "N", n, n, n, 1.0, A, n, n * n, Bt, n, n * n, 0.0, Ct, n, n * n,
+                             batch, tc.Policy.F16_EC)
+    torch.cuda.synchronize()
+    for b in (0, 1, 511, 1023):
+        ref = orc.gemm_f64(A[b].cpu().numpy(), Bt[b].cpu().numpy().T)
+        c = np.ascontiguousarray(Ct[b].cpu().numpy().T)
+        c32 = orc.gemm_f32(A[b].cpu().numpy(), Bt[b].cpu().numpy().T)
+        assert orc.max_rel_err(c, ref) <= 2 * orc.max_rel_err(c32, ref)
+    # every batch entry equals the same product done alone
+    for b in (3, 700):
+        assert torch.equal(Ct[b], tc.matmul_tn(A[b].contiguous(), Bt[b].contiguous(), tc.Policy.F16_EC))
+
+
+def test_config5b_k_heavy(tc, orc, dev):
+    """M=N=1024, K=262144, N(0,1): long accumulation; error growth vs plain fp32."""
+    m, k = 1024, 262144
+    A = _inputs(dev, (m, k), "normal", 0x5EED + 6)
+    Bt = _inputs(dev, (m, k), "normal", 0x5EED + 66)
+    Ct = tc.matmul_tn(A, Bt, tc.Policy.F16_EC)
+    torch.cuda.synchronize()
+    err, e32, fro = _check_rows(orc, A, Bt, Ct, 16)
+    assert err <= 2 * e32, (err, e32)
+    # the sequential fp32 loop loses ~sqrt(K) ulps here; TCEC stays well below it
+    assert err < e32

@@ -208,3 +208,28 @@ def test_pack_then_gemm_reuses_operands(tc, orc, dev):
                     if k0 + x < k2:
                         exp[x] = terms[t][r, k0 + x]
             assert np.array_equal(raw2[rb, kt, t, lane], exp)
+
+
+@pytest.mark.parametrize("policy", [0, 2])
+@pytest.mark.parametrize("mnk", [(64, 64, 8232), (200, 120, 16384), (256, 128, 32768)])
+def test_split_k(tc, orc, dev, policy, mnk):
+    """K-heavy shapes with few output tiles are cut into K slices (when the caller gives
+    workspace for them); with and without the split the result meets the same gates."""
+    m, n, k = mnk
+    rng = np.random.default_rng(m + k + policy)
+    A = rng.standard_normal((m, k)).astype(np.float32)
+    B = rng.standard_normal((k, n)).astype(np.float32)
+    assert tc.gemm_packed_workspace_bytes(policy, m, n, k) > 0
+    ws = torch.empty(tc.workspace_bytes(m, n, k, 1, policy), dtype=torch.uint8, device=dev)
+    C0 = rng.standard_normal((m, n)).astype(np.float32)
+    split = _gemm(tc, dev, A, B, policy, alpha=0.5, beta=2.0, C=C0, workspace=ws, ld_pad=1)
+    only_pack = torch.empty(tc.pack_bytes(m, k, 1, policy) + tc.pack_bytes(n, k, 1, policy),
+                            dtype=torch.uint8, device=dev)
+    unsplit = _gemm(tc, dev, A, B, policy, alpha=0.5, beta=2.0, C=C0, workspace=only_pack, ld_pad=1)
+    ref = 0.5 * orc.gemm_f64(A, B) + 2.0 * C0
+    e32 = orc.max_rel_err((0.5 * orc.gemm_f32(A, B) + 2.0 * C0).astype(np.float32), ref)
+    for D in (split, unsplit):
+        assert orc.max_rel_err(D, ref) <= 2 * e32
+    assert np.abs(split - unsplit).max() <= 4 * e32 * np.abs(ref).max()   # both within the gate of each other
+    # library-allocated workspace takes the same path as the explicit one
+    assert np.array_equal(_gemm(tc, dev, A, B, policy, alpha=0.5, beta=2.0, C=C0, ld_pad=1), split)

@@ -33,6 +33,7 @@ EXPORTS = [
     "wmmae_tcec_sgemm_strided_batched",
     "wmmae_tcec_pack_bytes",
     "wmmae_tcec_pack",
+    "wmmae_tcec_gemm_packed_workspace_bytes",
     "wmmae_tcec_gemm_packed",
     "wmmae_primitive_tiles",
     "wmmae_layout_dump",
@@ -75,7 +76,9 @@ _SIGNATURES = {
                                               _vp, _sz, _vp]),
     "wmmae_tcec_pack_bytes": (_i, [_i, _i, _i, _i, _c.POINTER(_sz)]),
     "wmmae_tcec_pack": (_i, [_i, _i, _i, _vp, _ll, _ll, _ll, _i, _vp, _sz, _vp]),
-    "wmmae_tcec_gemm_packed": (_i, [_i, _i, _i, _i, _fp, _vp, _vp, _fp, _vp, _i, _ll, _i, _i, _vp]),
+    "wmmae_tcec_gemm_packed_workspace_bytes": (_i, [_i, _i, _i, _i, _i, _c.POINTER(_sz)]),
+    "wmmae_tcec_gemm_packed": (_i, [_i, _i, _i, _i, _fp, _vp, _vp, _fp, _vp, _i, _ll, _i, _i, _vp, _sz,
+                                    _vp]),
     "wmmae_primitive_tiles": (_i, [_vp, _ll, _vp, _vp, _vp, _vp, _vp, _vp, _vp]),
     "wmmae_layout_dump": (_i, [_i, _i, _i, _i, _i, _vp, _vp, _vp, _vp, _vp, _vp]),
     "wmmae_tcec_mma_tile": (_i, [_i, _i, _i, _i, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _vp]),

@@ -118,8 +118,41 @@ struct GemmArgs {
   long long ldc, stride_c;
   float alpha, beta, inv_scale;
   int batch, terms;
+  float *partial;  // split-K slices, or nullptr
+  int splits;      // >= 1
   hipStream_t stream;
 };
+
+inline int device_cus() {
+  static const int cached = [] {
+    int dev = 0;
+    hipDeviceProp_t prop;
+    if (hipGetDevice(&dev) == hipSuccess &&
+        hipGetDeviceProperties(&prop, dev) == hipSuccess &&
+        prop.multiProcessorCount > 0)
+      return prop.multiProcessorCount;
+    return 256; // MI355X; also the answer when no device is visible
+  }();
+  return cached;
+}
+
+// Number of K slices: only when the output tiles cannot fill the chip and
+// every slice still has a long K loop.
+inline int choose_splits(const int m, const int n, const int k,
+                         const int batch) {
+  const long long tiles = ceil_div(m, 256) * ceil_div(n, 128) * batch;
+  const int cus = device_cus();
+  const int kt = static_cast<int>(ceil_div(k, 32));
+  if (tiles * 2 > cus || kt < 128)
+    return 1;
+  long long s = ceil_div(cus, tiles);
+  const long long max_by_k = kt / 64; // at least 64 stages (2048 of k) a slice
+  if (s > max_by_k)
+    s = max_by_k;
+  if (s > 64)
+    s = 64;
+  return s < 1 ? 1 : static_cast<int>(s);
+}
 
 // Deepest LDS ring (at most 4 stages) that fits the 160 KiB of a compute unit.
 constexpr int ring_depth(const int bm, const int bn, const int terms) {
@@ -145,32 +178,38 @@ int launch_gemm(const GemmArgs &g) {
   const int vec_store =
       (g.ldc % 4 == 0) && (reinterpret_cast<uintptr_t>(g.c) % 16 == 0) &&
       (g.stride_c % 4 == 0);
-  hipLaunchKernelGGL(kernel, dim3(tiles_m * tiles_n, g.batch),
+  const int splits = g.partial != nullptr ? g.splits : 1;
+  const int split_stages = static_cast<int>(ceil_div(KT, splits));
+  const int zdim = static_cast<int>(ceil_div(KT, split_stages));
+  hipLaunchKernelGGL(kernel, dim3(tiles_m * tiles_n, g.batch, zdim),
                      dim3(Cfg::NTHREADS), Cfg::LDS_BYTES, g.stream, g.a, g.b,
                      g.c, g.m, g.n, KT, rb_a, rb_b, g.ldc, g.alpha, g.beta,
                      g.inv_scale, tiles_m, tiles_n, vec_store,
                      static_cast<long long>(rb_a) * KT * TERMS * 64,
                      static_cast<long long>(rb_b) * KT * TERMS * 64,
-                     g.stride_c);
-  return launch_status();
+                     g.stride_c, split_stages,
+                     zdim > 1 ? g.partial : static_cast<float *>(nullptr));
+  int st = launch_status();
+  if (st == WMMAE_STATUS_SUCCESS && zdim > 1) {
+    const long long blocks = ceil_div(static_cast<long long>(g.m) * g.n, 256);
+    hipLaunchKernelGGL(wmmae_gemm::reduce_splits_kernel,
+                       dim3(static_cast<unsigned>(blocks), g.batch), dim3(256),
+                       0, g.stream, g.partial, zdim, g.c, g.m, g.n, g.ldc,
+                       g.stride_c, g.alpha, g.beta);
+    st = launch_status();
+  }
+  return st;
 }
 
 // Tile choice: the large tile when it still gives every compute unit work,
 // otherwise smaller tiles so that more blocks exist.
 template <class MT, int TERMS, bool RN> int gemm_by_size(const GemmArgs &g) {
-  int cus = 256;
-  {
-    int dev = 0;
-    hipDeviceProp_t prop;
-    if (hipGetDevice(&dev) == hipSuccess &&
-        hipGetDeviceProperties(&prop, dev) == hipSuccess &&
-        prop.multiProcessorCount > 0)
-      cus = prop.multiProcessorCount;
-  }
+  const int cus = device_cus();
+  const long long z = g.partial != nullptr ? g.splits : 1;
   const long long big =
-      ceil_div(g.m, 256) * ceil_div(g.n, 128) * static_cast<long long>(g.batch);
+      ceil_div(g.m, 256) * ceil_div(g.n, 128) * g.batch * z;
   const long long mid =
-      ceil_div(g.m, 128) * ceil_div(g.n, 128) * static_cast<long long>(g.batch);
+      ceil_div(g.m, 128) * ceil_div(g.n, 128) * g.batch * z;
   if constexpr (TERMS <= 2) {
     if (big >= cus)
       return launch_gemm<MT, TERMS, 256, 128, 2, 2, RN>(g);
@@ -300,7 +339,8 @@ int wmmae_tcec_gemm_packed(const int policy, const int m, const int n,
                            const void *const packed_b, const float *const beta,
                            float *const C, const int ldc,
                            const long long stride_c, const int batch,
-                           const int flags, void *const stream) {
+                           const int flags, void *const workspace,
+                           const size_t workspace_bytes, void *const stream) {
   PolicyInfo p;
   if (!policy_info(policy, p) || m < 0 || n < 0 || k < 0 || batch < 0 ||
       (flags & ~WMMAE_FLAG_RN_MAIN) != 0)
@@ -343,7 +383,32 @@ int wmmae_tcec_gemm_packed(const int policy, const int m, const int n,
   g.batch = batch;
   g.terms = p.terms;
   g.stream = static_cast<hipStream_t>(stream);
+  // split-K only when the caller supplied room for the slices
+  g.splits = choose_splits(m, n, k, batch);
+  g.partial = nullptr;
+  if (g.splits > 1 && workspace != nullptr &&
+      reinterpret_cast<uintptr_t>(workspace) % 16 == 0 &&
+      workspace_bytes >= static_cast<size_t>(g.splits) * batch * m * n * 4u)
+    g.partial = static_cast<float *>(workspace);
+  else
+    g.splits = 1;
   return gemm_dispatch(policy, flags, g);
+}
+
+int wmmae_tcec_gemm_packed_workspace_bytes(const int policy, const int m,
+                                           const int n, const int k,
+                                           const int batch,
+                                           size_t *const bytes) {
+  PolicyInfo p;
+  if (bytes == nullptr)
+    return WMMAE_STATUS_NULL_POINTER;
+  if (!policy_info(policy, p) || m < 0 || n < 0 || k < 0 || batch < 0)
+    return WMMAE_STATUS_INVALID_VALUE;
+  const int splits = (m == 0 || n == 0 || k == 0 || batch == 0)
+                         ? 1
+                         : choose_splits(m, n, k, batch);
+  *bytes = splits > 1 ? static_cast<size_t>(splits) * batch * m * n * 4u : 0;
+  return WMMAE_STATUS_SUCCESS;
 }
 
 int wmmae_tcec_sgemm_workspace_bytes(const int m, const int n, const int k,
@@ -360,7 +425,11 @@ int wmmae_tcec_sgemm_workspace_bytes(const int m, const int n, const int k,
   s = wmmae_tcec_pack_bytes(n, k, batch, policy, &b);
   if (s != WMMAE_STATUS_SUCCESS)
     return s;
-  *bytes = a + b;
+  size_t c = 0;
+  s = wmmae_tcec_gemm_packed_workspace_bytes(policy, m, n, k, batch, &c);
+  if (s != WMMAE_STATUS_SUCCESS)
+    return s;
+  *bytes = a + b + c;
   return WMMAE_STATUS_SUCCESS;
 }
 
@@ -389,24 +458,30 @@ int wmmae_tcec_sgemm_strided_batched(
       ldc < m)
     return WMMAE_STATUS_BAD_LEADING_DIM;
 
-  size_t bytes_a = 0, bytes_b = 0;
+  size_t bytes_a = 0, bytes_b = 0, bytes_c = 0;
   wmmae_tcec_pack_bytes(m, k, batch, policy, &bytes_a);
   wmmae_tcec_pack_bytes(n, k, batch, policy, &bytes_b);
+  wmmae_tcec_gemm_packed_workspace_bytes(policy, m, n, k, batch, &bytes_c);
   hipStream_t s = static_cast<hipStream_t>(stream);
   bool own = false;
   if (workspace == nullptr) {
-    if (bytes_a + bytes_b > 0) {
-      WMMAE_HIP_TRY(hipMallocAsync(&workspace, bytes_a + bytes_b, s));
+    if (bytes_a + bytes_b + bytes_c > 0) {
+      WMMAE_HIP_TRY(hipMallocAsync(&workspace, bytes_a + bytes_b + bytes_c, s));
       own = true;
     }
   } else {
     if (reinterpret_cast<uintptr_t>(workspace) % 16 != 0)
       return WMMAE_STATUS_MISALIGNED;
+    // the packed operands are required; the split-K slices are optional
     if (workspace_bytes < bytes_a + bytes_b)
       return WMMAE_STATUS_WORKSPACE_TOO_SMALL;
+    if (workspace_bytes < bytes_a + bytes_b + bytes_c)
+      bytes_c = 0;
   }
   void *const pa = workspace;
   void *const pb = static_cast<char *>(workspace) + bytes_a;
+  void *const pc =
+      bytes_c > 0 ? static_cast<char *>(workspace) + bytes_a + bytes_b : nullptr;
 
   int st = WMMAE_STATUS_SUCCESS;
   if (k > 0) {
@@ -422,7 +497,7 @@ int wmmae_tcec_sgemm_strided_batched(
   }
   if (st == WMMAE_STATUS_SUCCESS)
     st = wmmae_tcec_gemm_packed(policy, m, n, k, alpha, pa, pb, beta, C, ldc,
-                                stride_c, batch, flags, stream);
+                                stride_c, batch, flags, pc, bytes_c, stream);
   if (own) {
     if (hipFreeAsync(workspace, s) != hipSuccess &&
         st == WMMAE_STATUS_SUCCESS)

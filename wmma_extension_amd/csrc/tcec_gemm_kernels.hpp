@@ -136,6 +136,30 @@ __global__ void __launch_bounds__(256)
 }
 
 // --------------------------------------------------------------------------
+// reduce_splits_kernel: C = alpha * sum_z partial[z] + beta * C for split-K.
+// partial[z][batch] are dense column-major M x N slices; the sum runs over z
+// in ascending order in double precision, so the result does not depend on
+// the launch geometry.
+// --------------------------------------------------------------------------
+__global__ void __launch_bounds__(256)
+    reduce_splits_kernel(const float *__restrict__ partial, const int splits,
+                         float *__restrict__ C, const int M, const int N,
+                         const long long ldc, const long long batch_stride_c,
+                         const float alpha, const float beta) {
+  const long long e = static_cast<long long>(blockIdx.x) * 256 + threadIdx.x;
+  const long long mn = static_cast<long long>(M) * N;
+  if (e >= mn)
+    return;
+  const long long batches = gridDim.y;
+  double s = 0.;
+  for (int z = 0; z < splits; z++)
+    s += static_cast<double>(partial[(z * batches + blockIdx.y) * mn + e]);
+  float *const p = C + blockIdx.y * batch_stride_c + (e % M) + (e / M) * ldc;
+  const float v = alpha * static_cast<float>(s);
+  *p = beta == 0.f ? v : v + beta * *p;
+}
+
+// --------------------------------------------------------------------------
 // tcec_gemm_kernel: C = alpha * (A*B) + beta * C from packed operands.
 //
 //   MT      : MFMA element type (_Float16 or __bf16)
@@ -202,7 +226,8 @@ __global__ void __launch_bounds__(WGM *WGN * 64)
                      const int tiles_n, const int vec_store,
                      const long long batch_stride_a,
                      const long long batch_stride_b,
-                     const long long batch_stride_c) {
+                     const long long batch_stride_c, const int split_stages,
+                     float *__restrict__ partial) {
   using Cfg = GemmConfig<MT, TERMS, BM, BN, WGM, WGN, NSTAGE, RN_MAIN>;
   typedef MT ab_vec __attribute__((ext_vector_type(8)));
   constexpr int NCH = Cfg::NCH, CH_A = Cfg::CH_A, CPW = Cfg::CPW;
@@ -279,7 +304,18 @@ __global__ void __launch_bounds__(WGM *WGN * 64)
       acc_err[i][j] = f32x4{0.f, 0.f, 0.f, 0.f};
     }
 
-  const int num_stages = KT;
+  // Split-K: with `partial` set, blockIdx.z selects a range of split_stages
+  // k stages and the block writes its raw sum (no alpha / beta) to
+  // partial[z][batch] as a dense column-major M x N matrix; reduce_splits_kernel
+  // adds the slices.  Used when there are too few output tiles to fill the chip.
+  const int st_begin = partial != nullptr ? blockIdx.z * split_stages : 0;
+  const int num_stages =
+      partial != nullptr
+          ? (KT - st_begin < split_stages ? KT - st_begin : split_stages)
+          : KT;
+#pragma unroll
+  for (int q = 0; q < CPW; q++)
+    gsrc[q] += static_cast<long long>(st_begin) * (CH_PER_RB * 64);
 
   // Request chunk Q (of this wave's CPW chunks) of stage `st` into LDS buffer
   // `buf`.  The stage is clamped to the last one: the few redundant loads at
@@ -449,7 +485,16 @@ __global__ void __launch_bounds__(WGM *WGN * 64)
                    : "memory");
 
   // ---- epilogue: recombine, scale, store
-  float *const Cb = C + batch * batch_stride_c;
+  const bool to_partial = partial != nullptr;
+  float *const Cb =
+      to_partial ? partial + (static_cast<long long>(blockIdx.z) * gridDim.y +
+                              batch) *
+                                 (static_cast<long long>(M) * N)
+                 : C + batch * batch_stride_c;
+  const long long ld_out = to_partial ? M : ldc;
+  const float a_out = to_partial ? 1.f : alpha;
+  const float b_out = to_partial ? 0.f : beta;
+  const int vec_out = to_partial ? (M % 4 == 0) : vec_store;
   const int row_base = tm * BM + wm * Cfg::WM + 4 * static_cast<int>(lane >> 4);
   const int col_base = tn * BN + wn * Cfg::WN + static_cast<int>(lane & 15u);
 #pragma unroll
@@ -465,19 +510,19 @@ __global__ void __launch_bounds__(WGM *WGN * 64)
       f32x4 v = acc_main[i][j];
       if constexpr (TERMS >= 2)
         v += acc_err[i][j] * inv_scale;
-      v *= alpha;
-      float *const dst = Cb + row + static_cast<long long>(col) * ldc;
-      if (vec_store && row + 3 < M) {
-        if (beta != 0.f)
-          v += beta * *reinterpret_cast<const f32x4 *>(dst);
+      v *= a_out;
+      float *const dst = Cb + row + static_cast<long long>(col) * ld_out;
+      if (vec_out && row + 3 < M) {
+        if (b_out != 0.f)
+          v += b_out * *reinterpret_cast<const f32x4 *>(dst);
         *reinterpret_cast<f32x4 *>(dst) = v;
       } else {
 #pragma unroll
         for (int x = 0; x < 4; x++) {
           if (row + x < M) {
             float o = v[x];
-            if (beta != 0.f)
-              o += beta * dst[x];
+            if (b_out != 0.f)
+              o += b_out * dst[x];
             dst[x] = o;
           }
         }

@@ -99,12 +99,21 @@ def pack(policy, rows, k, X, row_stride, k_stride, packed, batch=1, batch_stride
     _lib.check(st, "wmmae_tcec_pack")
 
 
+def gemm_packed_workspace_bytes(policy, m, n, k, batch=1):
+    out = ctypes.c_size_t(0)
+    _lib.check(_lib.lib().wmmae_tcec_gemm_packed_workspace_bytes(int(policy), m, n, k, batch,
+                                                                 ctypes.byref(out)),
+               "wmmae_tcec_gemm_packed_workspace_bytes")
+    return out.value
+
+
 def gemm_packed(policy, m, n, k, alpha, packed_a, packed_b, beta, C, ldc, batch=1,
-                stride_c=0, flags=0):
-    _need_cuda(packed_a, packed_b, C)
+                stride_c=0, flags=0, workspace=None):
+    _need_cuda(packed_a, packed_b, C, workspace)
+    ws_bytes = workspace.numel() * workspace.element_size() if workspace is not None else 0
     st = _lib.lib().wmmae_tcec_gemm_packed(int(policy), m, n, k, _f(alpha), _ptr(packed_a),
                                            _ptr(packed_b), _f(beta), _ptr(C), ldc, stride_c,
-                                           batch, flags, _stream())
+                                           batch, flags, _ptr(workspace), ws_bytes, _stream())
     _lib.check(st, "wmmae_tcec_gemm_packed")
 
 
