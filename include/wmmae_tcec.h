@@ -101,6 +101,18 @@ int wmmae_tcec_sgemm_strided_batched(char transa, char transb, int m, int n,
                                      void *workspace, size_t workspace_bytes,
                                      void *stream);
 
+/* Batched product on device arrays of matrix pointers, the calling convention
+ * of the reference's launch_bgemm(conf, m, n, k, alpha, a_ptr_array, lda,
+ * b_ptr_array, ldb, beta, c_ptr_array, ldc, batch) (batch_gemm.cu:433-443) and
+ * of cublasSgemmBatched.  A_array, B_array, C_array are DEVICE arrays of
+ * `batch` device pointers. */
+int wmmae_tcec_sgemm_batched(char transa, char transb, int m, int n, int k,
+                             const float *alpha, const float *const *A_array,
+                             int lda, const float *const *B_array, int ldb,
+                             const float *beta, float *const *C_array, int ldc,
+                             int batch, int policy, int flags, void *workspace,
+                             size_t workspace_bytes, void *stream);
+
 /* The two stages, for callers that keep an operand split across many
  * products.  A packed operand is `rows` x k (rows = m for op(A), n for op(B))
  * with element (r, l) read from X[r*row_stride + l*k_stride]; the packed form
@@ -182,6 +194,15 @@ int wmmae_tcec_matvec(int type, int ec, float *y, const float *a,
 int wmmae_tcec_frag_dump(int use, int type, int ec, int frag_col,
                          unsigned short *terms, const float *src,
                          int from_vector, int mem_col, void *stream);
+
+/* Element access on a 32x32 TCEC accumulator: fill_fragment(base), x(i) +=
+ * lane*100 + i, dx(i) = i (with_ec), optional neg(), optional integrate(),
+ * store column-major into out[0..1024); out[1024 + lane] = x(0) + x(last) read
+ * through the const accessors.  inst as in wmmae_tcec_mma_tile.
+ * Replaces: test/tcec/elementwise.cu:7-26 (and the fill part of
+ * test/primitive/fill.cu). */
+int wmmae_tcec_elementwise(int type, int ec, int inst, float *out, float base,
+                           int do_neg, int do_integrate, void *stream);
 
 /* One raw MFMA D = A*B + C on 16-bit patterns (type 0 half, 1 bfloat16);
  * (m,n,k) one of (16,16,16), (16,16,32), (32,32,8), (32,32,16); a: m x k,

@@ -233,3 +233,35 @@ def test_split_k(tc, orc, dev, policy, mnk):
     assert np.abs(split - unsplit).max() <= 4 * e32 * np.abs(ref).max()   # both within the gate of each other
     # library-allocated workspace takes the same path as the explicit one
     assert np.array_equal(_gemm(tc, dev, A, B, policy, alpha=0.5, beta=2.0, C=C0, ld_pad=1), split)
+
+
+def test_pointer_array_batched(tc, orc, dev):
+    """The reference harness's calling convention: device arrays of matrix pointers
+    (test/tcec/batch_gemm.cu:433-443), matrices scattered in memory, ramp inputs
+    A[j] = j/k, B[j] = j/n of that harness for one entry."""
+    batch, m, n, k = 7, 96, 64, 160
+    rng = np.random.default_rng(55)
+    As = [torch.from_numpy(rng.standard_normal((m, k)).astype(np.float32)).to(dev) for _ in range(batch)]
+    Bs = [torch.from_numpy(rng.standard_normal((n, k)).astype(np.float32)).to(dev) for _ in range(batch)]
+    As[3] = (torch.arange(m * k, dtype=torch.float32, device=dev) / k).reshape(m, k)
+    Bs[3] = (torch.arange(k * n, dtype=torch.float32, device=dev) / n).reshape(n, k)
+    Cs = [torch.full((n, m), 3.0, dtype=torch.float32, device=dev) for _ in range(batch)]
+    pa = torch.tensor([t.data_ptr() for t in As], dtype=torch.int64, device=dev)
+    pb = torch.tensor([t.data_ptr() for t in Bs], dtype=torch.int64, device=dev)
+    pc = torch.tensor([t.data_ptr() for t in Cs], dtype=torch.int64, device=dev)
+    for policy in (0, 2):
+        for c in Cs:
+            c.fill_(3.0)
+        tc.sgemm_batched("T", "N", m, n, k, 2.0, pa, k, pb, k, -1.0, pc, m, batch, policy)
+        torch.cuda.synchronize()
+        for b in range(batch):
+            a, bt = As[b].cpu().numpy(), Bs[b].cpu().numpy()
+            ref = 2.0 * orc.gemm_f64(a, bt.T) - 3.0
+            got = Cs[b].cpu().numpy().T
+            e32 = orc.max_rel_err((2.0 * orc.gemm_f32(a, bt.T) - 3.0).astype(np.float32), ref)
+            assert orc.max_rel_err(got, ref) <= 2 * e32 + 2.0**-21
+            single = _gemm(tc, dev, a, bt.T, policy, alpha=2.0, beta=-1.0, C=np.full((m, n), 3.0, np.float32))
+            assert np.array_equal(got, single)
+        # Frobenius residual of the harness's ramp entry, as batch_gemm.cu:559-605 reports it
+        ref3 = orc.gemm_f64(As[3].cpu().numpy(), Bs[3].cpu().numpy().T) * 2.0 - 3.0
+        assert orc.frobenius_residual(Cs[3].cpu().numpy().T, ref3) < 3e-7

@@ -174,3 +174,36 @@ def test_fragment_terms_bit_exact(tc, orc, dev, type_, use):
                 j = ij[lane, reg, 1] + bn * sub_cols
                 for t in range(nterms):
                     assert gotv[t, e, lane] == tv[t][i, j]
+
+
+@pytest.mark.parametrize("type_", [0, 2])
+@pytest.mark.parametrize("ec", [1, 0])
+@pytest.mark.parametrize("inst", [0, 1, 2])
+def test_elementwise_accessors_neg_integrate(tc, orc, dev, type_, ec, inst):
+    """x(i) / dx(i) address sub-fragment i / num_elements, register i % num_elements;
+    fill_fragment sets the main part and clears the error part; neg negates both;
+    integrate folds err/scale into main (test/tcec/elementwise.cu:7-26, tcec.hpp:40-98)."""
+    fm, fn, fk = {0: (16, 16, 32), 1: (16, 16, 16), 2: (32, 32, 16)}[inst]
+    ij = orc.frag_ij_table(2, fm, fn, fk)
+    R = ij.shape[1]
+    nbm = 32 // fm
+    scale = 2048.0 if type_ == 0 else 1.0
+    base = 2.5
+    for do_neg, do_int in itertools.product((0, 1), (0, 1)):
+        out = tc.elementwise(type_, ec, inst, base, do_neg, do_int, dev).cpu().numpy()
+        got = out[:1024].reshape(32, 32).T                     # stored column-major
+        nelem = (32 // fm) * (32 // fn) * R
+        for lane in range(64):
+            assert out[1024 + lane] == (base + lane * 100) + (base + lane * 100 + nelem - 1)
+            for e in range(nelem):
+                block, reg = divmod(e, R)
+                bm, bn = block % nbm, block // nbm
+                i = ij[lane, reg, 0] + bm * fm
+                j = ij[lane, reg, 1] + bn * fn
+                main = np.float32(base + lane * 100 + e)
+                err = np.float32(e) if ec else np.float32(0)
+                if do_neg:
+                    main, err = -main, -err
+                # store and integrate both evaluate main + err/scale in fp32
+                expect = np.float32(main + np.float32(err / np.float32(scale)))
+                assert got[i, j] == expect, (do_neg, do_int, lane, e)

@@ -31,6 +31,7 @@ EXPORTS = [
     "wmmae_tcec_sgemm_workspace_bytes",
     "wmmae_tcec_sgemm",
     "wmmae_tcec_sgemm_strided_batched",
+    "wmmae_tcec_sgemm_batched",
     "wmmae_tcec_pack_bytes",
     "wmmae_tcec_pack",
     "wmmae_tcec_gemm_packed_workspace_bytes",
@@ -41,6 +42,7 @@ EXPORTS = [
     "wmmae_tcec_mma_tile_native",
     "wmmae_tcec_matvec",
     "wmmae_tcec_frag_dump",
+    "wmmae_tcec_elementwise",
     "wmmae_mfma_probe",
 ]
 
@@ -74,6 +76,8 @@ _SIGNATURES = {
     "wmmae_tcec_sgemm_strided_batched": (_i, [_c.c_char, _c.c_char, _i, _i, _i, _fp, _vp, _i, _ll,
                                               _vp, _i, _ll, _fp, _vp, _i, _ll, _i, _i, _i,
                                               _vp, _sz, _vp]),
+    "wmmae_tcec_sgemm_batched": (_i, [_c.c_char, _c.c_char, _i, _i, _i, _fp, _vp, _i, _vp, _i, _fp,
+                                      _vp, _i, _i, _i, _i, _vp, _sz, _vp]),
     "wmmae_tcec_pack_bytes": (_i, [_i, _i, _i, _i, _c.POINTER(_sz)]),
     "wmmae_tcec_pack": (_i, [_i, _i, _i, _vp, _ll, _ll, _ll, _i, _vp, _sz, _vp]),
     "wmmae_tcec_gemm_packed_workspace_bytes": (_i, [_i, _i, _i, _i, _i, _c.POINTER(_sz)]),
@@ -85,6 +89,7 @@ _SIGNATURES = {
     "wmmae_tcec_mma_tile_native": (_i, [_i, _i, _i, _i, _vp, _vp, _vp, _i, _vp]),
     "wmmae_tcec_matvec": (_i, [_i, _i, _vp, _vp, _vp, _i, _i, _vp]),
     "wmmae_tcec_frag_dump": (_i, [_i, _i, _i, _i, _vp, _vp, _i, _i, _vp]),
+    "wmmae_tcec_elementwise": (_i, [_i, _i, _i, _vp, _c.c_float, _i, _i, _vp]),
     "wmmae_mfma_probe": (_i, [_i, _i, _i, _i, _vp, _vp, _vp, _vp, _vp]),
 }
 

@@ -71,9 +71,9 @@ inline long long packed_elems(const int rows, const int k, const int terms) {
 // ------------------------------------------------------------------ pack
 template <class T, int TERMS>
 int launch_pack(const int rows, const int k, const float *X,
-                const long long row_stride, const long long k_stride,
-                const long long batch_stride, const int batch, void *packed,
-                hipStream_t stream) {
+                const float *const *ptrs, const long long row_stride,
+                const long long k_stride, const long long batch_stride,
+                const int batch, void *packed, hipStream_t stream) {
   const int KT = packed_k_tiles(k);
   const long long chunks = packed_row_blocks(rows) * KT;
   const long long blocks = ceil_div(chunks * 64, 256);
@@ -82,17 +82,17 @@ int launch_pack(const int rows, const int k, const float *X,
   hipLaunchKernelGGL((wmmae_gemm::split_pack_kernel<T, TERMS>),
                      dim3(static_cast<unsigned>(blocks), batch), dim3(256), 0,
                      stream, X, row_stride, k_stride, rows, k, KT, chunks,
-                     batch_stride, static_cast<u32x4 *>(packed),
+                     batch_stride, ptrs, static_cast<u32x4 *>(packed),
                      chunks * TERMS * 64);
   return launch_status();
 }
 
 int pack_dispatch(const int policy, const int rows, const int k, const float *X,
-                  const long long row_stride, const long long k_stride,
-                  const long long batch_stride, const int batch, void *packed,
-                  hipStream_t stream) {
+                  const float *const *ptrs, const long long row_stride,
+                  const long long k_stride, const long long batch_stride,
+                  const int batch, void *packed, hipStream_t stream) {
 #define WMMAE_PACK_ARGS                                                        \
-  rows, k, X, row_stride, k_stride, batch_stride, batch, packed, stream
+  rows, k, X, ptrs, row_stride, k_stride, batch_stride, batch, packed, stream
   switch (policy) {
   case WMMAE_POLICY_F16_EC:
     return launch_pack<w::half, 2>(WMMAE_PACK_ARGS);
@@ -118,6 +118,7 @@ struct GemmArgs {
   long long ldc, stride_c;
   float alpha, beta, inv_scale;
   int batch, terms;
+  float *const *c_ptrs; // device array of C pointers, or nullptr
   float *partial;  // split-K slices, or nullptr
   int splits;      // >= 1
   hipStream_t stream;
@@ -175,9 +176,12 @@ int launch_gemm(const GemmArgs &g) {
   const int KT = packed_k_tiles(g.k);
   const int rb_a = static_cast<int>(packed_row_blocks(g.m));
   const int rb_b = static_cast<int>(packed_row_blocks(g.n));
+  // 16-byte stores need ldc % 4 == 0 and an aligned base; the base of each
+  // batch entry is checked again inside the kernel
   const int vec_store =
-      (g.ldc % 4 == 0) && (reinterpret_cast<uintptr_t>(g.c) % 16 == 0) &&
-      (g.stride_c % 4 == 0);
+      (g.ldc % 4 == 0) &&
+      (g.c_ptrs != nullptr || (reinterpret_cast<uintptr_t>(g.c) % 16 == 0 &&
+                               g.stride_c % 4 == 0));
   const int splits = g.partial != nullptr ? g.splits : 1;
   const int split_stages = static_cast<int>(ceil_div(KT, splits));
   const int zdim = static_cast<int>(ceil_div(KT, split_stages));
@@ -188,14 +192,15 @@ int launch_gemm(const GemmArgs &g) {
                      static_cast<long long>(rb_a) * KT * TERMS * 64,
                      static_cast<long long>(rb_b) * KT * TERMS * 64,
                      g.stride_c, split_stages,
-                     zdim > 1 ? g.partial : static_cast<float *>(nullptr));
+                     zdim > 1 ? g.partial : static_cast<float *>(nullptr),
+                     g.c_ptrs);
   int st = launch_status();
   if (st == WMMAE_STATUS_SUCCESS && zdim > 1) {
     const long long blocks = ceil_div(static_cast<long long>(g.m) * g.n, 256);
     hipLaunchKernelGGL(wmmae_gemm::reduce_splits_kernel,
                        dim3(static_cast<unsigned>(blocks), g.batch), dim3(256),
                        0, g.stream, g.partial, zdim, g.c, g.m, g.n, g.ldc,
-                       g.stride_c, g.alpha, g.beta);
+                       g.stride_c, g.c_ptrs, g.alpha, g.beta);
     st = launch_status();
   }
   return st;
@@ -309,17 +314,22 @@ int wmmae_tcec_pack_bytes(const int rows, const int k, const int batch,
   return WMMAE_STATUS_SUCCESS;
 }
 
-int wmmae_tcec_pack(const int policy, const int rows, const int k,
-                    const float *const X, const long long row_stride,
-                    const long long k_stride, const long long batch_stride,
-                    const int batch, void *const packed,
-                    const size_t packed_bytes, void *const stream) {
+} // extern "C"
+
+namespace {
+// Shared implementations; X / C may be given as a base pointer with a batch
+// stride or as a device array of per-matrix pointers.
+int pack_impl(const int policy, const int rows, const int k,
+              const float *const X, const float *const *const ptrs,
+              const long long row_stride, const long long k_stride,
+              const long long batch_stride, const int batch, void *const packed,
+              const size_t packed_bytes, void *const stream) {
   PolicyInfo p;
   if (!policy_info(policy, p) || rows < 0 || k < 0 || batch < 0)
     return WMMAE_STATUS_INVALID_VALUE;
   if (rows == 0 || k == 0 || batch == 0)
     return WMMAE_STATUS_SUCCESS;
-  if (X == nullptr || packed == nullptr)
+  if ((X == nullptr && ptrs == nullptr) || packed == nullptr)
     return WMMAE_STATUS_NULL_POINTER;
   if (row_stride < 1 || k_stride < 1 || (row_stride != 1 && k_stride != 1))
     return WMMAE_STATUS_BAD_LEADING_DIM;
@@ -329,18 +339,18 @@ int wmmae_tcec_pack(const int policy, const int rows, const int k,
   wmmae_tcec_pack_bytes(rows, k, batch, policy, &need);
   if (packed_bytes < need)
     return WMMAE_STATUS_WORKSPACE_TOO_SMALL;
-  return pack_dispatch(policy, rows, k, X, row_stride, k_stride, batch_stride,
-                       batch, packed, static_cast<hipStream_t>(stream));
+  return pack_dispatch(policy, rows, k, X, ptrs, row_stride, k_stride,
+                       batch_stride, batch, packed,
+                       static_cast<hipStream_t>(stream));
 }
 
-int wmmae_tcec_gemm_packed(const int policy, const int m, const int n,
-                           const int k, const float *const alpha,
-                           const void *const packed_a,
-                           const void *const packed_b, const float *const beta,
-                           float *const C, const int ldc,
-                           const long long stride_c, const int batch,
-                           const int flags, void *const workspace,
-                           const size_t workspace_bytes, void *const stream) {
+int gemm_packed_impl(const int policy, const int m, const int n, const int k,
+                     const float *const alpha, const void *const packed_a,
+                     const void *const packed_b, const float *const beta,
+                     float *const C, float *const *const c_ptrs, const int ldc,
+                     const long long stride_c, const int batch, const int flags,
+                     void *const workspace, const size_t workspace_bytes,
+                     void *const stream) {
   PolicyInfo p;
   if (!policy_info(policy, p) || m < 0 || n < 0 || k < 0 || batch < 0 ||
       (flags & ~WMMAE_FLAG_RN_MAIN) != 0)
@@ -349,7 +359,8 @@ int wmmae_tcec_gemm_packed(const int policy, const int m, const int n,
     return WMMAE_STATUS_NULL_POINTER;
   if (m == 0 || n == 0 || batch == 0)
     return WMMAE_STATUS_SUCCESS;
-  if (C == nullptr || (k > 0 && (packed_a == nullptr || packed_b == nullptr)))
+  if ((C == nullptr && c_ptrs == nullptr) ||
+      (k > 0 && (packed_a == nullptr || packed_b == nullptr)))
     return WMMAE_STATUS_NULL_POINTER;
   if (ldc < m)
     return WMMAE_STATUS_BAD_LEADING_DIM;
@@ -365,13 +376,14 @@ int wmmae_tcec_gemm_packed(const int policy, const int m, const int n,
     hipLaunchKernelGGL(wmmae_gemm::scale_c_kernel,
                        dim3(static_cast<unsigned>(blocks), batch), dim3(256), 0,
                        static_cast<hipStream_t>(stream), C, m, n,
-                       static_cast<long long>(ldc), stride_c, *beta);
+                       static_cast<long long>(ldc), stride_c, c_ptrs, *beta);
     return launch_status();
   }
   GemmArgs g;
   g.a = static_cast<const u32x4 *>(packed_a);
   g.b = static_cast<const u32x4 *>(packed_b);
   g.c = C;
+  g.c_ptrs = c_ptrs;
   g.m = m;
   g.n = n;
   g.k = k;
@@ -395,52 +407,16 @@ int wmmae_tcec_gemm_packed(const int policy, const int m, const int n,
   return gemm_dispatch(policy, flags, g);
 }
 
-int wmmae_tcec_gemm_packed_workspace_bytes(const int policy, const int m,
-                                           const int n, const int k,
-                                           const int batch,
-                                           size_t *const bytes) {
-  PolicyInfo p;
-  if (bytes == nullptr)
-    return WMMAE_STATUS_NULL_POINTER;
-  if (!policy_info(policy, p) || m < 0 || n < 0 || k < 0 || batch < 0)
-    return WMMAE_STATUS_INVALID_VALUE;
-  const int splits = (m == 0 || n == 0 || k == 0 || batch == 0)
-                         ? 1
-                         : choose_splits(m, n, k, batch);
-  *bytes = splits > 1 ? static_cast<size_t>(splits) * batch * m * n * 4u : 0;
-  return WMMAE_STATUS_SUCCESS;
-}
-
-int wmmae_tcec_sgemm_workspace_bytes(const int m, const int n, const int k,
-                                     const int batch, const int policy,
-                                     size_t *const bytes) {
-  size_t a = 0, b = 0;
-  if (bytes == nullptr)
-    return WMMAE_STATUS_NULL_POINTER;
-  if (m < 0 || n < 0)
-    return WMMAE_STATUS_INVALID_VALUE;
-  int s = wmmae_tcec_pack_bytes(m, k, batch, policy, &a);
-  if (s != WMMAE_STATUS_SUCCESS)
-    return s;
-  s = wmmae_tcec_pack_bytes(n, k, batch, policy, &b);
-  if (s != WMMAE_STATUS_SUCCESS)
-    return s;
-  size_t c = 0;
-  s = wmmae_tcec_gemm_packed_workspace_bytes(policy, m, n, k, batch, &c);
-  if (s != WMMAE_STATUS_SUCCESS)
-    return s;
-  *bytes = a + b + c;
-  return WMMAE_STATUS_SUCCESS;
-}
-
-int wmmae_tcec_sgemm_strided_batched(
-    const char transa, const char transb, const int m, const int n, const int k,
-    const float *const alpha, const float *const A, const int lda,
-    const long long stride_a, const float *const B, const int ldb,
-    const long long stride_b, const float *const beta, float *const C,
-    const int ldc, const long long stride_c, const int batch, const int policy,
-    const int flags, void *workspace, const size_t workspace_bytes,
-    void *const stream) {
+int sgemm_impl(const char transa, const char transb, const int m, const int n,
+               const int k, const float *const alpha, const float *const A,
+               const float *const *const a_ptrs, const int lda,
+               const long long stride_a, const float *const B,
+               const float *const *const b_ptrs, const int ldb,
+               const long long stride_b, const float *const beta,
+               float *const C, float *const *const c_ptrs, const int ldc,
+               const long long stride_c, const int batch, const int policy,
+               const int flags, void *workspace, const size_t workspace_bytes,
+               void *const stream) {
   PolicyInfo p;
   if ((!is_n(transa) && !is_t(transa)) || (!is_n(transb) && !is_t(transb)) ||
       m < 0 || n < 0 || k < 0 || batch < 0 || !policy_info(policy, p) ||
@@ -450,7 +426,9 @@ int wmmae_tcec_sgemm_strided_batched(
     return WMMAE_STATUS_NULL_POINTER;
   if (m == 0 || n == 0 || batch == 0)
     return WMMAE_STATUS_SUCCESS;
-  if (C == nullptr || (k > 0 && (A == nullptr || B == nullptr)))
+  if ((C == nullptr && c_ptrs == nullptr) ||
+      (k > 0 && ((A == nullptr && a_ptrs == nullptr) ||
+                 (B == nullptr && b_ptrs == nullptr))))
     return WMMAE_STATUS_NULL_POINTER;
   const int a_rows = is_n(transa) ? m : k; // rows of A as stored (column major)
   const int b_rows = is_n(transb) ? k : n;
@@ -486,24 +464,113 @@ int wmmae_tcec_sgemm_strided_batched(
   int st = WMMAE_STATUS_SUCCESS;
   if (k > 0) {
     // op(A)(i,l): 'N' -> A[i + l*lda], 'T' -> A[l + i*lda]
-    st = wmmae_tcec_pack(policy, m, k, A, is_n(transa) ? 1 : lda,
-                         is_n(transa) ? lda : 1, stride_a, batch, pa, bytes_a,
-                         stream);
+    st = pack_impl(policy, m, k, A, a_ptrs, is_n(transa) ? 1 : lda,
+                   is_n(transa) ? lda : 1, stride_a, batch, pa, bytes_a, stream);
     // op(B)(l,j): 'N' -> B[l + j*ldb], 'T' -> B[j + l*ldb]; packed rows = j
     if (st == WMMAE_STATUS_SUCCESS)
-      st = wmmae_tcec_pack(policy, n, k, B, is_n(transb) ? ldb : 1,
-                           is_n(transb) ? 1 : ldb, stride_b, batch, pb, bytes_b,
-                           stream);
+      st = pack_impl(policy, n, k, B, b_ptrs, is_n(transb) ? ldb : 1,
+                     is_n(transb) ? 1 : ldb, stride_b, batch, pb, bytes_b,
+                     stream);
   }
   if (st == WMMAE_STATUS_SUCCESS)
-    st = wmmae_tcec_gemm_packed(policy, m, n, k, alpha, pa, pb, beta, C, ldc,
-                                stride_c, batch, flags, pc, bytes_c, stream);
+    st = gemm_packed_impl(policy, m, n, k, alpha, pa, pb, beta, C, c_ptrs, ldc,
+                          stride_c, batch, flags, pc, bytes_c, stream);
   if (own) {
     if (hipFreeAsync(workspace, s) != hipSuccess &&
         st == WMMAE_STATUS_SUCCESS)
       st = WMMAE_STATUS_RUNTIME_ERROR;
   }
   return st;
+}
+} // namespace
+
+extern "C" {
+
+int wmmae_tcec_pack(const int policy, const int rows, const int k,
+                    const float *const X, const long long row_stride,
+                    const long long k_stride, const long long batch_stride,
+                    const int batch, void *const packed,
+                    const size_t packed_bytes, void *const stream) {
+  return pack_impl(policy, rows, k, X, nullptr, row_stride, k_stride,
+                   batch_stride, batch, packed, packed_bytes, stream);
+}
+
+int wmmae_tcec_gemm_packed(const int policy, const int m, const int n,
+                           const int k, const float *const alpha,
+                           const void *const packed_a,
+                           const void *const packed_b, const float *const beta,
+                           float *const C, const int ldc,
+                           const long long stride_c, const int batch,
+                           const int flags, void *const workspace,
+                           const size_t workspace_bytes, void *const stream) {
+  return gemm_packed_impl(policy, m, n, k, alpha, packed_a, packed_b, beta, C,
+                          nullptr, ldc, stride_c, batch, flags, workspace,
+                          workspace_bytes, stream);
+}
+
+int wmmae_tcec_gemm_packed_workspace_bytes(const int policy, const int m,
+                                           const int n, const int k,
+                                           const int batch,
+                                           size_t *const bytes) {
+  PolicyInfo p;
+  if (bytes == nullptr)
+    return WMMAE_STATUS_NULL_POINTER;
+  if (!policy_info(policy, p) || m < 0 || n < 0 || k < 0 || batch < 0)
+    return WMMAE_STATUS_INVALID_VALUE;
+  const int splits = (m == 0 || n == 0 || k == 0 || batch == 0)
+                         ? 1
+                         : choose_splits(m, n, k, batch);
+  *bytes = splits > 1 ? static_cast<size_t>(splits) * batch * m * n * 4u : 0;
+  return WMMAE_STATUS_SUCCESS;
+}
+
+int wmmae_tcec_sgemm_workspace_bytes(const int m, const int n, const int k,
+                                     const int batch, const int policy,
+                                     size_t *const bytes) {
+  size_t a = 0, b = 0, c = 0;
+  if (bytes == nullptr)
+    return WMMAE_STATUS_NULL_POINTER;
+  if (m < 0 || n < 0)
+    return WMMAE_STATUS_INVALID_VALUE;
+  int s = wmmae_tcec_pack_bytes(m, k, batch, policy, &a);
+  if (s != WMMAE_STATUS_SUCCESS)
+    return s;
+  s = wmmae_tcec_pack_bytes(n, k, batch, policy, &b);
+  if (s != WMMAE_STATUS_SUCCESS)
+    return s;
+  s = wmmae_tcec_gemm_packed_workspace_bytes(policy, m, n, k, batch, &c);
+  if (s != WMMAE_STATUS_SUCCESS)
+    return s;
+  *bytes = a + b + c;
+  return WMMAE_STATUS_SUCCESS;
+}
+
+int wmmae_tcec_sgemm_strided_batched(
+    const char transa, const char transb, const int m, const int n, const int k,
+    const float *const alpha, const float *const A, const int lda,
+    const long long stride_a, const float *const B, const int ldb,
+    const long long stride_b, const float *const beta, float *const C,
+    const int ldc, const long long stride_c, const int batch, const int policy,
+    const int flags, void *const workspace, const size_t workspace_bytes,
+    void *const stream) {
+  return sgemm_impl(transa, transb, m, n, k, alpha, A, nullptr, lda, stride_a,
+                    B, nullptr, ldb, stride_b, beta, C, nullptr, ldc, stride_c,
+                    batch, policy, flags, workspace, workspace_bytes, stream);
+}
+
+int wmmae_tcec_sgemm_batched(const char transa, const char transb, const int m,
+                             const int n, const int k, const float *const alpha,
+                             const float *const *const A_array, const int lda,
+                             const float *const *const B_array, const int ldb,
+                             const float *const beta,
+                             float *const *const C_array, const int ldc,
+                             const int batch, const int policy, const int flags,
+                             void *const workspace,
+                             const size_t workspace_bytes,
+                             void *const stream) {
+  return sgemm_impl(transa, transb, m, n, k, alpha, nullptr, A_array, lda, 0,
+                    nullptr, B_array, ldb, 0, beta, nullptr, C_array, ldc, 0,
+                    batch, policy, flags, workspace, workspace_bytes, stream);
 }
 
 int wmmae_tcec_sgemm(const char transa, const char transb, const int m,
@@ -513,10 +580,9 @@ int wmmae_tcec_sgemm(const char transa, const char transb, const int m,
                      const int ldc, const int policy, const int flags,
                      void *const workspace, const size_t workspace_bytes,
                      void *const stream) {
-  return wmmae_tcec_sgemm_strided_batched(transa, transb, m, n, k, alpha, A,
-                                          lda, 0, B, ldb, 0, beta, C, ldc, 0, 1,
-                                          policy, flags, workspace,
-                                          workspace_bytes, stream);
+  return sgemm_impl(transa, transb, m, n, k, alpha, A, nullptr, lda, 0, B,
+                    nullptr, ldb, 0, beta, C, nullptr, ldc, 0, 1, policy, flags,
+                    workspace, workspace_bytes, stream);
 }
 
 // ------------------------------------------------------------ harness
@@ -753,6 +819,36 @@ int wmmae_tcec_frag_dump(const int use, const int type, const int ec,
               dim3(1), dim3(64), 0, s, terms, src, from_vector, mem_col);
         return launch_status();
       });
+    });
+  });
+}
+
+int wmmae_tcec_elementwise(const int type, const int ec, const int inst,
+                           float *const out, const float base,
+                           const int do_neg, const int do_integrate,
+                           void *const stream) {
+  if (!out)
+    return WMMAE_STATUS_NULL_POINTER;
+  if (inst < 0 || inst > 2)
+    return WMMAE_STATUS_INVALID_VALUE;
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  return with_type(type, [&](auto tt) {
+    using T = typename decltype(tt)::type;
+    return with_ec(ec, [&](auto te) {
+      using EC = typename decltype(te)::type;
+      auto go = [&](auto kernel) {
+        hipLaunchKernelGGL(kernel, dim3(1), dim3(64), 0, s, out, base, do_neg,
+                           do_integrate);
+        return launch_status();
+      };
+      if (inst == 0)
+        return go(wmmae_harness::tcec_elementwise_kernel<
+                  32, T, tcec::Policy<tcec::op_mfma, EC, 16, 16, 32>>);
+      if (inst == 1)
+        return go(wmmae_harness::tcec_elementwise_kernel<
+                  32, T, tcec::Policy<tcec::op_mfma, EC, 16, 16, 16>>);
+      return go(wmmae_harness::tcec_elementwise_kernel<
+                32, T, tcec::Policy<tcec::op_mfma, EC, 32, 32, 16>>);
     });
   });
 }

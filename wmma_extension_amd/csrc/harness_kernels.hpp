@@ -14,6 +14,8 @@
 //                             (reference: test/tcec/mma.cu:23-100)
 //   tcec_matvec_kernel      : y = A*x through tcec::load_vector / store_vector
 //                             (reference: test/tcec/matvec.cu:21-50)
+//   tcec_elementwise_kernel : x(i) / dx(i) accessors, fill_fragment, neg, integrate
+//                             (reference: test/tcec/elementwise.cu:7-26)
 //   tcec_frag_dump_kernel   : split terms held by an operand fragment after
 //                             load_matrix_sync or load_vector
 //                             (reference: test/tcec/vector.cu:15-61)
@@ -306,6 +308,38 @@ __global__ void __launch_bounds__(64)
       terms[(2 * F::num_elements + e) * 64 + lane] =
           __builtin_bit_cast(unsigned short, f.sub_d2_frag[b].x[r]);
   }
+}
+
+// --------------------------------------------------------------------------
+// Element access on a TCEC accumulator (N = 32): fill_fragment(base), then
+// x(i) = lane*100 + i as in the reference's test, dx(i) = i (with_ec only),
+// optional neg(), optional integrate(), then store column-major.
+// out[0 .. N*N) receives the stored matrix; out[N*N + lane] the value of
+// x(0) + x(num_elements-1) read back through the const accessors after the
+// edits (before neg / integrate).
+// (reference: test/tcec/elementwise.cu:7-26; tcec.hpp:40-98 accessors, neg,
+// integrate; test/primitive/fill.cu)
+// --------------------------------------------------------------------------
+template <int N, class T, class Policy>
+__global__ void __launch_bounds__(64)
+    tcec_elementwise_kernel(float *const out, const float base,
+                            const int do_neg, const int do_integrate) {
+  using F = tcec::fragment<w::accumulator, N, N, N, T, void, Policy>;
+  F frag;
+  tcec::fill_fragment(frag, base);
+  const unsigned lane = w::detail::common::get_lane_id();
+  for (unsigned i = 0; i < F::num_elements; i++) {
+    frag.x(i) += static_cast<float>(lane * 100 + i);
+    if constexpr (F::num_terms >= 2)
+      frag.dx(i) = static_cast<float>(i);
+  }
+  const F &cref = frag;
+  out[N * N + lane] = cref.x(0) + cref.x(F::num_elements - 1);
+  if (do_neg)
+    frag = tcec::neg(frag);
+  if (do_integrate)
+    frag.integrate();
+  tcec::store_matrix_sync(out, frag, N, w::mem_col_major);
 }
 
 // --------------------------------------------------------------------------

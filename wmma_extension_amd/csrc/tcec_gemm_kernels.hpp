@@ -56,6 +56,9 @@ __host__ __device__ constexpr int reads_due(const int count, const int span,
 // split_pack_kernel: X (fp32, element (r,k) at X[r*row_stride + k*k_stride])
 // -> packed terms.  One thread per (chunk, lane).  Rows >= rows and k >= K are
 // zero filled, so the GEMM kernel needs no edge handling on its loads.
+// Batch entry y reads X + y*in_batch_stride, or in_ptrs[y] when in_ptrs is set
+// (the reference's harness passes arrays of matrix pointers,
+// test/tcec/batch_gemm.cu:433-443).
 //   T      : split tag (half, bfloat16, precision::tf32)
 //   TERMS  : number of terms stored (1 = leading term only, i.e. no correction)
 //   KT     : number of 32-wide k chunks per row block; chunks = row blocks * KT
@@ -66,6 +69,7 @@ __global__ void __launch_bounds__(256)
                       const long long k_stride, const int rows, const int K,
                       const int KT, const long long chunks,
                       const long long in_batch_stride,
+                      const float *const *__restrict__ in_ptrs,
                       u32x4 *__restrict__ out,
                       const long long out_batch_stride) {
   using traits = mtk::wmma::tcec::detail::split_traits<T>;
@@ -86,8 +90,12 @@ __global__ void __launch_bounds__(256)
   for (int x = 0; x < 8; x++)
     v[x] = 0.f;
   if (r < rows && k0 < K) {
-    const float *p = X + blockIdx.y * in_batch_stride + r * row_stride +
-                     static_cast<long long>(k0) * k_stride;
+    // batch entry: base + stride, or a device array of matrix pointers
+    const float *const base = in_ptrs != nullptr
+                                  ? in_ptrs[blockIdx.y]
+                                  : X + blockIdx.y * in_batch_stride;
+    const float *p =
+        base + r * row_stride + static_cast<long long>(k0) * k_stride;
     if (k_stride == 1 && k0 + 8 <= K &&
         (reinterpret_cast<uintptr_t>(p) & 15u) == 0) {
       const f32x4 lo = *reinterpret_cast<const f32x4 *>(p);
@@ -127,11 +135,13 @@ __global__ void __launch_bounds__(256)
 __global__ void __launch_bounds__(256)
     scale_c_kernel(float *__restrict__ C, const int M, const int N,
                    const long long ldc, const long long batch_stride_c,
-                   const float beta) {
+                   float *const *__restrict__ c_ptrs, const float beta) {
   const long long e = static_cast<long long>(blockIdx.x) * 256 + threadIdx.x;
   if (e >= static_cast<long long>(M) * N)
     return;
-  float *const p = C + blockIdx.y * batch_stride_c + (e % M) + (e / M) * ldc;
+  float *const cb =
+      c_ptrs != nullptr ? c_ptrs[blockIdx.y] : C + blockIdx.y * batch_stride_c;
+  float *const p = cb + (e % M) + (e / M) * ldc;
   *p = beta == 0.f ? 0.f : beta * *p;
 }
 
@@ -145,7 +155,8 @@ __global__ void __launch_bounds__(256)
     reduce_splits_kernel(const float *__restrict__ partial, const int splits,
                          float *__restrict__ C, const int M, const int N,
                          const long long ldc, const long long batch_stride_c,
-                         const float alpha, const float beta) {
+                         float *const *__restrict__ c_ptrs, const float alpha,
+                         const float beta) {
   const long long e = static_cast<long long>(blockIdx.x) * 256 + threadIdx.x;
   const long long mn = static_cast<long long>(M) * N;
   if (e >= mn)
@@ -154,7 +165,9 @@ __global__ void __launch_bounds__(256)
   double s = 0.;
   for (int z = 0; z < splits; z++)
     s += static_cast<double>(partial[(z * batches + blockIdx.y) * mn + e]);
-  float *const p = C + blockIdx.y * batch_stride_c + (e % M) + (e / M) * ldc;
+  float *const cb =
+      c_ptrs != nullptr ? c_ptrs[blockIdx.y] : C + blockIdx.y * batch_stride_c;
+  float *const p = cb + (e % M) + (e / M) * ldc;
   const float v = alpha * static_cast<float>(s);
   *p = beta == 0.f ? v : v + beta * *p;
 }
@@ -227,7 +240,8 @@ __global__ void __launch_bounds__(WGM *WGN * 64)
                      const long long batch_stride_a,
                      const long long batch_stride_b,
                      const long long batch_stride_c, const int split_stages,
-                     float *__restrict__ partial) {
+                     float *__restrict__ partial,
+                     float *const *__restrict__ c_ptrs) {
   using Cfg = GemmConfig<MT, TERMS, BM, BN, WGM, WGN, NSTAGE, RN_MAIN>;
   typedef MT ab_vec __attribute__((ext_vector_type(8)));
   constexpr int NCH = Cfg::NCH, CH_A = Cfg::CH_A, CPW = Cfg::CPW;
@@ -391,7 +405,14 @@ __global__ void __launch_bounds__(WGM *WGN * 64)
   // LDS read r of the next stage goes out after MFMA number (r+1)*SPAN/NFRAG:
   // the reads are spread over the first three quarters of the step (the LGKM
   // counter only tracks 15 outstanding operations)
-  constexpr int SPAN = (NMFMA * 3) / 4 > 0 ? (NMFMA * 3) / 4 : 1;
+#ifndef WMMAE_TUNE_SPAN_NUM
+#define WMMAE_TUNE_SPAN_NUM 3
+#define WMMAE_TUNE_SPAN_DEN 4
+#endif
+  constexpr int SPAN =
+      (NMFMA * WMMAE_TUNE_SPAN_NUM) / WMMAE_TUNE_SPAN_DEN > 0
+          ? (NMFMA * WMMAE_TUNE_SPAN_NUM) / WMMAE_TUNE_SPAN_DEN
+          : 1;
 
   // One pipeline step: multiply the fragments of stage st (already in
   // registers) while the fragments of stage st+1 are read from LDS and stage
@@ -490,11 +511,14 @@ __global__ void __launch_bounds__(WGM *WGN * 64)
       to_partial ? partial + (static_cast<long long>(blockIdx.z) * gridDim.y +
                               batch) *
                                  (static_cast<long long>(M) * N)
-                 : C + batch * batch_stride_c;
+                 : (c_ptrs != nullptr ? c_ptrs[batch]
+                                      : C + batch * batch_stride_c);
   const long long ld_out = to_partial ? M : ldc;
   const float a_out = to_partial ? 1.f : alpha;
   const float b_out = to_partial ? 0.f : beta;
-  const int vec_out = to_partial ? (M % 4 == 0) : vec_store;
+  const int vec_out =
+      to_partial ? (M % 4 == 0)
+                 : (vec_store && (reinterpret_cast<uintptr_t>(Cb) & 15u) == 0);
   const int row_base = tm * BM + wm * Cfg::WM + 4 * static_cast<int>(lane >> 4);
   const int col_base = tn * BN + wn * Cfg::WN + static_cast<int>(lane & 15u);
 #pragma unroll

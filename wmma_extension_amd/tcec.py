@@ -91,6 +91,18 @@ def sgemm_strided_batched(transa, transb, m, n, k, alpha, A, lda, stride_a, B, l
     _lib.check(st, "wmmae_tcec_sgemm_strided_batched")
 
 
+def sgemm_batched(transa, transb, m, n, k, alpha, A_array, lda, B_array, ldb, beta, C_array, ldc,
+                  batch, policy=Policy.F16_EC, flags=0, workspace=None):
+    """A_array / B_array / C_array: int64 device tensors holding `batch` device pointers
+    (the launch_bgemm / cublasSgemmBatched convention)."""
+    _need_cuda(A_array, B_array, C_array, workspace)
+    ws_bytes = workspace.numel() * workspace.element_size() if workspace is not None else 0
+    st = _lib.lib().wmmae_tcec_sgemm_batched(
+        transa.encode(), transb.encode(), m, n, k, _f(alpha), _ptr(A_array), lda, _ptr(B_array), ldb,
+        _f(beta), _ptr(C_array), ldc, batch, int(policy), flags, _ptr(workspace), ws_bytes, _stream())
+    _lib.check(st, "wmmae_tcec_sgemm_batched")
+
+
 def pack(policy, rows, k, X, row_stride, k_stride, packed, batch=1, batch_stride=0):
     _need_cuda(X, packed)
     st = _lib.lib().wmmae_tcec_pack(int(policy), rows, k, _ptr(X), row_stride, k_stride,
@@ -200,6 +212,14 @@ def frag_dump(use, type_, ec, frag_col, src, from_vector, mem_col):
     st = _lib.lib().wmmae_tcec_frag_dump(use, type_, int(ec), int(frag_col), _ptr(out), _ptr(src),
                                          int(from_vector), int(mem_col), _stream())
     _lib.check(st, "wmmae_tcec_frag_dump")
+    return out
+
+
+def elementwise(type_, ec, inst, base, do_neg, do_integrate, device="cuda"):
+    out = torch.zeros(32 * 32 + 64, dtype=torch.float32, device=device)
+    st = _lib.lib().wmmae_tcec_elementwise(type_, int(ec), inst, _ptr(out), float(base), int(do_neg),
+                                           int(do_integrate), _stream())
+    _lib.check(st, "wmmae_tcec_elementwise")
     return out
 
 
