@@ -204,6 +204,18 @@ int wmmae_tcec_frag_dump(int use, int type, int ec, int frag_col,
 int wmmae_tcec_elementwise(int type, int ec, int inst, float *out, float base,
                            int do_neg, int do_integrate, void *stream);
 
+/* C = alpha*A*B + beta*C by a tiled kernel written only against the public
+ * tcec:: device API (fp32 tiles in LDS, split at fragment load in every wave).
+ * A row-major m x k (lda), B column-major k x n (ldb), C column-major (ldc);
+ * m, n multiples of 128, k of 32, lda/ldb multiples of 4, 16-byte aligned.
+ * type/ec as in wmmae_tcec_mma_tile.
+ * Replaces: bgemm_kernel + mma_core, test/tcec/batch_gemm.cu:196-386, kept as
+ * the API-level comparator of wmmae_tcec_sgemm. */
+int wmmae_tcec_api_gemm(int type, int ec, int m, int n, int k,
+                        const float *alpha, const float *A, int lda,
+                        const float *B, int ldb, const float *beta, float *C,
+                        int ldc, void *stream);
+
 /* One raw MFMA D = A*B + C on 16-bit patterns (type 0 half, 1 bfloat16);
  * (m,n,k) one of (16,16,16), (16,16,32), (32,32,8), (32,32,16); a: m x k,
  * b: k x n, c/d: m x n, all row-major.

@@ -265,3 +265,30 @@ def test_pointer_array_batched(tc, orc, dev):
         # Frobenius residual of the harness's ramp entry, as batch_gemm.cu:559-605 reports it
         ref3 = orc.gemm_f64(As[3].cpu().numpy(), Bs[3].cpu().numpy().T) * 2.0 - 3.0
         assert orc.frobenius_residual(Cs[3].cpu().numpy().T, ref3) < 3e-7
+
+
+@pytest.mark.parametrize("type_ec", [(0, 1), (0, 0), (2, 1)])
+def test_api_level_gemm_matches_driver(tc, orc, dev, type_ec):
+    """A GEMM written only against the public tcec:: API (split at fragment load, as in
+    the reference's bgemm_kernel) against the oracle and against the packed driver."""
+    type_, ec = type_ec
+    policy = {(0, 1): 0, (0, 0): 1, (2, 1): 2}[type_ec]
+    m, n, k = 256, 384, 160
+    rng = np.random.default_rng(77 + policy)
+    A = rng.uniform(-1, 1, (m, k)).astype(np.float32)
+    Bt = rng.uniform(-1, 1, (n, k)).astype(np.float32)
+    C0 = rng.uniform(-1, 1, (m, n)).astype(np.float32)
+    dA, dB = torch.from_numpy(A).to(dev), torch.from_numpy(Bt).to(dev)
+    for alpha, beta in ((1.0, 0.0), (-0.5, 1.5)):
+        dC = torch.from_numpy(np.ascontiguousarray(C0.T)).to(dev)
+        tc.api_gemm(type_, ec, m, n, k, alpha, dA, k, dB, k, beta, dC, m)
+        torch.cuda.synchronize()
+        got = dC.cpu().numpy().T
+        ref = alpha * orc.gemm_f64(A, Bt.T) + beta * C0
+        _check(orc, got, A, Bt.T, policy, ref=ref, C=C0, alpha=alpha, beta=beta)
+        drv = _gemm(tc, dev, A, Bt.T, policy, alpha=alpha, beta=beta, C=C0)
+        assert np.abs(got - drv).max() <= 16 * 2.0**-24 * max(1.0, np.abs(ref).max())
+    from wmma_extension_amd._lib import WmmaeError
+    with pytest.raises(WmmaeError) as e:
+        tc.api_gemm(type_, ec, 100, n, k, 1.0, dA, k, dB, k, 0.0, dC, 100)
+    assert e.value.status == -4

@@ -43,6 +43,7 @@ EXPORTS = [
     "wmmae_tcec_matvec",
     "wmmae_tcec_frag_dump",
     "wmmae_tcec_elementwise",
+    "wmmae_tcec_api_gemm",
     "wmmae_mfma_probe",
 ]
 
@@ -90,6 +91,7 @@ _SIGNATURES = {
     "wmmae_tcec_matvec": (_i, [_i, _i, _vp, _vp, _vp, _i, _i, _vp]),
     "wmmae_tcec_frag_dump": (_i, [_i, _i, _i, _i, _vp, _vp, _i, _i, _vp]),
     "wmmae_tcec_elementwise": (_i, [_i, _i, _i, _vp, _c.c_float, _i, _i, _vp]),
+    "wmmae_tcec_api_gemm": (_i, [_i, _i, _i, _i, _i, _fp, _vp, _i, _vp, _i, _fp, _vp, _i, _vp]),
     "wmmae_mfma_probe": (_i, [_i, _i, _i, _i, _vp, _vp, _vp, _vp, _vp]),
 }
 

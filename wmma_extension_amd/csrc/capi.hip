@@ -853,6 +853,37 @@ int wmmae_tcec_elementwise(const int type, const int ec, const int inst,
   });
 }
 
+int wmmae_tcec_api_gemm(const int type, const int ec, const int m, const int n,
+                        const int k, const float *const alpha,
+                        const float *const A, const int lda,
+                        const float *const B, const int ldb,
+                        const float *const beta, float *const C, const int ldc,
+                        void *const stream) {
+  if (!alpha || !beta || !A || !B || !C)
+    return WMMAE_STATUS_NULL_POINTER;
+  if (m <= 0 || n <= 0 || k <= 0)
+    return WMMAE_STATUS_INVALID_VALUE;
+  if (lda < k || ldb < k || ldc < m)
+    return WMMAE_STATUS_BAD_LEADING_DIM;
+  if (m % 128 != 0 || n % 128 != 0 || k % 32 != 0 || lda % 4 != 0 ||
+      ldb % 4 != 0 || reinterpret_cast<uintptr_t>(A) % 16 != 0 ||
+      reinterpret_cast<uintptr_t>(B) % 16 != 0)
+    return WMMAE_STATUS_NOT_SUPPORTED;
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  const float al = *alpha, be = *beta;
+  return with_type(type, [&](auto tt) {
+    using T = typename decltype(tt)::type;
+    return with_ec(ec, [&](auto te) {
+      using EC = typename decltype(te)::type;
+      using P = tcec::Policy<tcec::op_mfma, EC, 16, 16, 32>;
+      hipLaunchKernelGGL((wmmae_harness::tcec_api_gemm_kernel<T, P>),
+                         dim3(m / 128, n / 128), dim3(256), 0, s, m, n, k, al,
+                         A, lda, B, ldb, be, C, ldc);
+      return launch_status();
+    });
+  });
+}
+
 int wmmae_mfma_probe(const int type, const int m, const int n, const int k,
                      float *const d, const unsigned short *const a,
                      const unsigned short *const b, const float *const c,

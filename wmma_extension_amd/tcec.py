@@ -223,6 +223,14 @@ def elementwise(type_, ec, inst, base, do_neg, do_integrate, device="cuda"):
     return out
 
 
+def api_gemm(type_, ec, m, n, k, alpha, A, lda, B, ldb, beta, C, ldc):
+    """Tiled GEMM written against the public device API only (comparator)."""
+    _need_cuda(A, B, C)
+    st = _lib.lib().wmmae_tcec_api_gemm(type_, int(ec), m, n, k, _f(alpha), _ptr(A), lda, _ptr(B), ldb,
+                                        _f(beta), _ptr(C), ldc, _stream())
+    _lib.check(st, "wmmae_tcec_api_gemm")
+
+
 def mfma_probe(type_, m, n, k, a_bits, b_bits, c):
     """a_bits (m,k) / b_bits (k,n): int16 tensors of raw 16-bit patterns; c (m,n) fp32."""
     _need_cuda(a_bits, b_bits, c)
