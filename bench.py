@@ -27,13 +27,27 @@ WORKLOADS = {
                desc="TCEC SGEMM bf16 three-term split (tf32-policy replacement), M=N=K=16384"),
     "c4f16": dict(m=16384, n=16384, k=16384, batch=1, policy="F16_EC", dist="uniform", mult=3,
                   desc="TCEC SGEMM fp16 hi+lo with EC, M=N=K=16384"),
-    "c5a": dict(m=256, n=256, k=256, batch=1024, policy="F16_EC", dist="normal", mult=3,
-                desc="strided-batched TCEC SGEMM, 1024 x 256^3"),
+    "c2": dict(kind="prim", tiles=1 << 20, dist="uniform",
+               desc="fragment primitives over 1,048,576 16x16 tiles (foreach_ij fills of A/B row+col, "
+                    "accumulator store, load_vector/store_vector)"),
+    "c5a": dict(m=256, n=256, k=256, batch=1024, policy="F16_EC", dist="normal", mult=3, fused=True,
+                desc="strided-batched TCEC SGEMM, 1024 x 256^3 (split inside the GEMM kernel)"),
+    "c5a_packed": dict(m=256, n=256, k=256, batch=1024, policy="F16_EC", dist="normal", mult=3,
+                       desc="strided-batched TCEC SGEMM, 1024 x 256^3, through packed operands"),
     "c5b": dict(m=1024, n=1024, k=262144, batch=1, policy="F16_EC", dist="normal", mult=3,
                 desc="K-heavy TCEC SGEMM, M=N=1024, K=262144"),
 }
 PEAK_MFMA_TFLOPS = 2500.0      # dense fp16 / bf16 MFMA, MI355X
 PEAK_HBM_GBS = 8000.0
+# workloads whose dominant kernel is bound by HBM rather than by the matrix cores
+HBM_BOUND = {"c2", "c5a", "c5a_packed"}
+# Bytes per launch of the dominant kernel that crossed the fabric side of L2, from
+# rocprofv3 --pmc FETCH_SIZE and --pmc WRITE_SIZE runs of this script (--calibrate),
+# scaled by the same counters of a 1 GiB copy (x2.000 and x1.000); see profiles/.
+MEASURED_TRAFFIC_BYTES = {
+    "c4": (75_497_800 + 1_048_580) * 1024,
+    "c3": (524_670 + 65_536) * 1024,
+}
 
 
 def make_inputs(torch, w, dev, seed):
@@ -99,6 +113,69 @@ def cpu_baseline(orc, w, target_s=15.0):
                       f"block of the workload, best of 2, {best:.2f} s"}
 
 
+def bench_primitives(args, torch, tcec, dev, w):
+    """Workload c2: the fragment-primitive kernel over a stream of tiles (HBM bound)."""
+    import ctypes
+    from wmma_extension_amd import _lib
+    T = w["tiles"]
+    g = torch.Generator(device=dev)
+    g.manual_seed(0x5EED + 2)
+    tiles = torch.rand((T, 256), generator=g, device=dev, dtype=torch.float32) * 2 - 1
+    out = tcec.primitive_tiles(tiles)
+    h = _lib.lib()
+    stream = ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
+    ptrs = [ctypes.c_void_p(out[k].data_ptr()) for k in ("a_row", "a_col", "b_row", "b_col", "acc", "vec")]
+
+    def step():
+        st = h.wmmae_primitive_tiles(ctypes.c_void_p(tiles.data_ptr()), T, *ptrs, stream)
+        assert st == 0
+    for _ in range(args.warmup):
+        step()
+    torch.cuda.synchronize()
+    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    t0 = time.perf_counter()
+    e0.record()
+    for _ in range(args.steps):
+        step()
+    e1.record()
+    torch.cuda.synchronize()
+    elapsed = time.perf_counter() - t0
+    kernel_ms = e0.elapsed_time(e1) / args.steps
+    # per tile: 1024 B fp32 in, 4 x 512 B fp16 fragment dumps, 1024 B accumulator, 2 x 64 B vectors
+    nbytes = T * (1024 + 4 * 512 + 1024 + 128)
+    gbs = nbytes / (kernel_ms * 1e-3) / 1e9
+    res = {
+        "metric": "fragment-primitive tile stream, algorithmic GB/s", "value": round(gbs, 1), "unit": "GB/s",
+        "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+        "ms_per_step": round(elapsed / args.steps * 1e3, 4), "higher_is_better": True, "scaling": "weak",
+        "vs_baseline": None, "dtype": "f16", "data": "synthetic",
+        "config": {"workload": f"c2: {w['desc']}", "tiles": T},
+        "roofline": {"bound": "hbm", "achieved": round(gbs, 1), "peak": PEAK_HBM_GBS, "unit": "GB/s",
+                     "frac": round(gbs / PEAK_HBM_GBS, 4), "traffic": None, "kernel": "primitive_tiles_kernel",
+                     "kernel_ms": round(kernel_ms, 4), "algorithmic_bytes": nbytes},
+        "tiles_per_s": round(T / (kernel_ms * 1e-3), 1),
+        "cpu_baseline": None,
+    }
+    if not args.no_cpu:
+        # the oracle's layout tables applied with numpy to a sample of the tiles
+        import numpy as np
+        from oracle import oracle as orc
+        sample = 1 << 16
+        x = tiles[:sample].cpu().numpy()
+        tables = [orc.foreach_tables(use, 16, 16, 16, col)[0] for use, col in ((0, 0), (0, 1), (1, 0), (1, 1))]
+        t0 = time.perf_counter()
+        x16 = x.astype(np.float16)
+        outs = [x16[:, tb] for tb in tables]
+        acc = np.ascontiguousarray(x.reshape(-1, 16, 16).transpose(0, 2, 1))
+        vec = x[:, :32].copy()
+        dt = time.perf_counter() - t0
+        del outs, acc, vec
+        res["cpu_baseline"] = {"value": round(sample * (1024 + 4 * 512 + 1024 + 128) / dt / 1e9, 3), "unit": "GB/s",
+                               "cores": 1, "kind": "port",
+                               "sample": f"oracle layout tables applied with numpy to {sample} tiles, {dt:.2f} s"}
+    print(json.dumps(res))
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -123,17 +200,30 @@ def main():
     dev = torch.device("cuda:0")
     torch.cuda.set_device(dev)
     w = WORKLOADS[args.workload]
+    if w.get("kind") == "prim":
+        return bench_primitives(args, torch, tcec, dev, w)
     policy = tcec.Policy[w["policy"]]
     m, n, k, batch = w["m"], w["n"], w["k"], w["batch"]
 
     A, Bt = make_inputs(torch, w, dev, 0x5EED + 3)
     Ct = torch.empty((batch, n, m), dtype=torch.float32, device=dev)
-    pa = torch.empty(tcec.pack_bytes(m, k, batch, policy), dtype=torch.uint8, device=dev)
-    pb = torch.empty(tcec.pack_bytes(n, k, batch, policy), dtype=torch.uint8, device=dev)
-    ws_bytes = tcec.gemm_packed_workspace_bytes(policy, m, n, k, batch)
-    ws = torch.empty(ws_bytes, dtype=torch.uint8, device=dev) if ws_bytes else None
+    fused = bool(w.get("fused"))
+    if not fused:
+        pa = torch.empty(tcec.pack_bytes(m, k, batch, policy), dtype=torch.uint8, device=dev)
+        pb = torch.empty(tcec.pack_bytes(n, k, batch, policy), dtype=torch.uint8, device=dev)
+        ws_bytes = tcec.gemm_packed_workspace_bytes(policy, m, n, k, batch)
+        ws = torch.empty(ws_bytes, dtype=torch.uint8, device=dev) if ws_bytes else None
 
     def step(ev=None):
+        if fused:
+            # small products: one kernel reads fp32 A and B, splits in registers, writes C
+            if ev is not None:
+                ev[0].record()
+            tcec.sgemm_strided_batched("T", "N", m, n, k, 1.0, A, k, m * k, Bt, k, n * k, 0.0,
+                                       Ct, m, n * m, batch, policy, args.flags)
+            if ev is not None:
+                ev[1].record()
+            return
         tcec.pack(policy, m, k, A, k, 1, pa, batch, m * k)
         tcec.pack(policy, n, k, Bt, k, 1, pb, batch, n * k)
         if ev is not None:
@@ -168,6 +258,24 @@ def main():
     achieved = flops * w["mult"] / (gemm_ms * 1e-3) / 1e12
     bytes_min = 4.0 * (m * k + k * n + m * n) * batch
 
+    if args.workload in HBM_BOUND:
+        # packed operands in (2*terms bytes per element), C out: the GEMM kernel's own minimum
+        terms = {"F16_EC": 2, "BF16X3_EC": 3, "BF16X2_EC": 2, "F16_NOEC": 1, "BF16_NOEC": 1}[w["policy"]]
+        kbytes = (2.0 * terms * (m * k + k * n) + 4.0 * m * n) * batch
+        if fused:
+            kbytes = bytes_min              # fp32 A and B in, fp32 C out
+        hbm = kbytes / (gemm_ms * 1e-3) / 1e9
+        roofline = {"bound": "hbm", "achieved": round(hbm, 1), "peak": PEAK_HBM_GBS, "unit": "GB/s",
+                    "frac": round(hbm / PEAK_HBM_GBS, 4), "traffic": MEASURED_TRAFFIC_BYTES.get(args.workload),
+                    "kernel": "tcec_gemm_fused_kernel" if fused else "tcec_gemm_kernel",
+                    "kernel_ms": round(gemm_ms, 4), "algorithmic_bytes": kbytes, "mfma_frac": round(achieved / PEAK_MFMA_TFLOPS, 4)}
+    else:
+        roofline = {"bound": "mfma", "achieved": round(achieved, 2), "peak": PEAK_MFMA_TFLOPS,
+                    "unit": "TFLOP/s", "frac": round(achieved / PEAK_MFMA_TFLOPS, 4),
+                    "traffic": MEASURED_TRAFFIC_BYTES.get(args.workload),
+                    "kernel": "tcec_gemm_kernel", "kernel_ms": round(gemm_ms, 4),
+                    "issued_flop_multiplier": w["mult"],
+                    "hbm_frac_of_min_traffic": round(bytes_min / (gemm_ms * 1e-3) / 1e9 / PEAK_HBM_GBS, 4)}
     out = {
         "metric": "TCEC SGEMM effective fp32 TFLOPS",
         "value": round(value, 3),
@@ -183,12 +291,9 @@ def main():
         "data": "synthetic",
         "config": {"workload": f"{args.workload}: {w['desc']}", "m": m, "n": n, "k": k, "batch": batch,
                    "policy": w["policy"], "distribution": w["dist"], "flags": args.flags,
-                   "step": "split+pack A, split+pack B, MFMA GEMM; inputs and workspace resident in HBM"},
-        "roofline": {"bound": "mfma", "achieved": round(achieved, 2), "peak": PEAK_MFMA_TFLOPS,
-                     "unit": "TFLOP/s", "frac": round(achieved / PEAK_MFMA_TFLOPS, 4), "traffic": None,
-                     "kernel": "tcec_gemm_kernel", "kernel_ms": round(gemm_ms, 4),
-                     "issued_flop_multiplier": w["mult"],
-                     "hbm_frac_of_min_traffic": round(bytes_min / (gemm_ms * 1e-3) / 1e9 / PEAK_HBM_GBS, 4)},
+                   "step": ("one fused split+MFMA GEMM kernel; inputs resident in HBM" if fused else
+                            "split+pack A, split+pack B, MFMA GEMM; inputs and workspace resident in HBM")},
+        "roofline": roofline,
         "gemm_only_effective_tflops": round(flops / (gemm_ms * 1e-3) / 1e12, 3),
         "fp32_vector_peak_tflops": 157.3,
     }

@@ -58,7 +58,8 @@ def _check(orc, D, A, B, policy, ref=None, C=None, alpha=1.0, beta=0.0):
 
 
 @pytest.mark.parametrize("policy", [0, 1, 2, 3, 4])
-@pytest.mark.parametrize("mnk", [(128, 128, 128), (256, 128, 64), (64, 64, 32), (512, 256, 160)])
+@pytest.mark.parametrize("mnk", [(128, 128, 128), (256, 128, 64), (64, 64, 32), (512, 256, 160),
+                                 (1024, 640, 96)])
 def test_sgemm_aligned_shapes(tc, orc, dev, policy, mnk):
     m, n, k = mnk
     rng = np.random.default_rng(m + n + k + policy)
@@ -73,7 +74,7 @@ def test_sgemm_aligned_shapes(tc, orc, dev, policy, mnk):
 
 @pytest.mark.parametrize("policy", [0, 2])
 @pytest.mark.parametrize("mnk", [(1, 1, 1), (17, 5, 3), (100, 37, 77), (129, 255, 33), (300, 200, 100),
-                                 (16, 16, 1000), (1000, 3, 8)])
+                                 (16, 16, 1000), (1000, 3, 8), (700, 37, 77), (130, 1031, 45)])
 def test_sgemm_ragged_shapes(tc, orc, dev, policy, mnk):
     m, n, k = mnk
     rng = np.random.default_rng(m * 7 + n * 3 + k + policy)
@@ -114,6 +115,10 @@ def test_sgemm_k_zero_and_workspace(tc, orc, dev):
     A = rng.uniform(-1, 1, (64, 64)).astype(np.float32)
     B = rng.uniform(-1, 1, (64, 64)).astype(np.float32)
     ws = torch.empty(tc.workspace_bytes(64, 64, 64), dtype=torch.uint8, device=dev)
+    assert np.array_equal(_gemm(tc, dev, A, B, 0, workspace=ws), _gemm(tc, dev, A, B, 0))
+    # a product large enough to go through the packed operands needs room for them
+    A = rng.uniform(-1, 1, (640, 64)).astype(np.float32)
+    ws = torch.empty(tc.workspace_bytes(640, 64, 64), dtype=torch.uint8, device=dev)
     assert np.array_equal(_gemm(tc, dev, A, B, 0, workspace=ws), _gemm(tc, dev, A, B, 0))
     small = torch.empty(16, dtype=torch.uint8, device=dev)
     from wmma_extension_amd._lib import WmmaeError
@@ -208,6 +213,32 @@ def test_pack_then_gemm_reuses_operands(tc, orc, dev):
                     if k0 + x < k2:
                         exp[x] = terms[t][r, k0 + x]
             assert np.array_equal(raw2[rb, kt, t, lane], exp)
+
+
+@pytest.mark.parametrize("policy", [0, 1, 2, 3, 4])
+@pytest.mark.parametrize("trans", ["TN", "NT"])
+def test_small_products_split_in_kernel_match_packed_path(tc, orc, dev, policy, trans):
+    """Products up to 512 x 512 are split inside the GEMM kernel (no packed copy in
+    memory); the result is bit for bit that of pack + gemm_packed."""
+    rng = np.random.default_rng(91 + policy)
+    for m, n, k in ((64, 64, 64), (40, 24, 50), (256, 256, 256), (500, 130, 77), (512, 512, 33)):
+        A = rng.standard_normal((m, k)).astype(np.float32)
+        B = rng.standard_normal((k, n)).astype(np.float32)
+        C0 = rng.standard_normal((m, n)).astype(np.float32)
+        for ld_pad in (0, 1):
+            fused = _gemm(tc, dev, A, B, policy, alpha=1.25, beta=-0.5, C=C0, ta=trans[0], tb=trans[1],
+                          ld_pad=ld_pad)
+            dA = torch.from_numpy(A).to(dev)
+            dB = torch.from_numpy(np.ascontiguousarray(B.T)).to(dev)
+            pa = torch.empty(tc.pack_bytes(m, k, 1, policy), dtype=torch.uint8, device=dev)
+            pb = torch.empty(tc.pack_bytes(n, k, 1, policy), dtype=torch.uint8, device=dev)
+            tc.pack(policy, m, k, dA, k, 1, pa)
+            tc.pack(policy, n, k, dB, k, 1, pb)
+            dC = torch.from_numpy(np.ascontiguousarray(C0.T)).to(dev)
+            tc.gemm_packed(policy, m, n, k, 1.25, pa, pb, -0.5, dC, m)
+            torch.cuda.synchronize()
+            assert np.array_equal(dC.cpu().numpy().T, fused), (m, n, k, ld_pad)
+        _check(orc, fused, A, B, policy, C=C0, alpha=1.25, beta=-0.5)
 
 
 @pytest.mark.parametrize("policy", [0, 2])

@@ -2,6 +2,7 @@
 // selection and launches.  Declarations and per-entry documentation live in
 // include/wmmae_tcec.h.
 #include "harness_kernels.hpp"
+#include "tcec_gemm_fused_kernel.hpp"
 #include "tcec_gemm_kernels.hpp"
 #include <wmmae_tcec.h>
 
@@ -246,6 +247,69 @@ int gemm_dispatch(const int policy, const int flags, const GemmArgs &g) {
   }
 }
 
+// ------------------------------------------------------ fused small GEMM
+struct FusedArgs {
+  wmmae_gemm::FusedParams p;
+  hipStream_t stream;
+};
+
+template <class T, int TERMS, int BM, int BN> int launch_fused(FusedArgs f) {
+  using Cfg = wmmae_gemm::FusedConfig<TERMS, BM, BN>;
+  auto kernel = wmmae_gemm::tcec_gemm_fused_kernel<T, TERMS, BM, BN>;
+  WMMAE_HIP_TRY(hipFuncSetAttribute(reinterpret_cast<const void *>(kernel),
+                                    hipFuncAttributeMaxDynamicSharedMemorySize,
+                                    Cfg::LDS_BYTES));
+  wmmae_gemm::FusedParams &p = f.p;
+  p.tiles_m = static_cast<int>(ceil_div(p.M, BM));
+  p.tiles_per_batch = p.tiles_m * static_cast<int>(ceil_div(p.N, BN));
+  // one persistent workgroup per compute unit at most; with 8 or more batch
+  // entries an XCD (block index mod 8) owns whole entries
+  const int per_xcd_max = device_cus() / 8 > 0 ? device_cus() / 8 : 1;
+  long long per_xcd = p.batch >= 8
+                          ? ceil_div(p.batch, 8) * p.tiles_per_batch
+                          : ceil_div(static_cast<long long>(p.batch) *
+                                         p.tiles_per_batch,
+                                     8);
+  if (per_xcd > per_xcd_max)
+    per_xcd = per_xcd_max;
+  const int grid = 8 * static_cast<int>(per_xcd);
+  hipLaunchKernelGGL(kernel, dim3(grid), dim3(256), Cfg::LDS_BYTES, f.stream,
+                     p);
+  return launch_status();
+}
+
+template <class T, int TERMS> int fused_by_size(const FusedArgs &f) {
+  if (f.p.M > 64 || f.p.N > 64)
+    return launch_fused<T, TERMS, 128, 128>(f);
+  return launch_fused<T, TERMS, 64, 64>(f);
+}
+
+int fused_dispatch(const int policy, const FusedArgs &f) {
+  switch (policy) {
+  case WMMAE_POLICY_F16_EC:
+    return fused_by_size<w::half, 2>(f);
+  case WMMAE_POLICY_F16_NOEC:
+    return fused_by_size<w::half, 1>(f);
+  case WMMAE_POLICY_BF16X3_EC:
+    return fused_by_size<w::precision::tf32, 3>(f);
+  case WMMAE_POLICY_BF16X2_EC:
+    return fused_by_size<w::bfloat16, 2>(f);
+  case WMMAE_POLICY_BF16_NOEC:
+    return fused_by_size<w::bfloat16, 1>(f);
+  default:
+    return WMMAE_STATUS_INVALID_VALUE;
+  }
+}
+
+// Products this small are bound by HBM: every operand element is needed by at
+// most four blocks, and a separate split pass would double the traffic.
+// K-heavy single products that want K slices stay on the packed path.
+inline bool use_fused(const int m, const int n, const int k, const int batch,
+                      const int flags) {
+  return m <= 512 && n <= 512 && k > 0 && (flags & WMMAE_FLAG_RN_MAIN) == 0 &&
+         choose_splits(m, n, k, batch) == 1;
+}
+
 inline bool is_n(const char t) { return t == 'N' || t == 'n'; }
 inline bool is_t(const char t) {
   return t == 'T' || t == 't' || t == 'C' || t == 'c';
@@ -436,6 +500,45 @@ int sgemm_impl(const char transa, const char transb, const int m, const int n,
       ldc < m)
     return WMMAE_STATUS_BAD_LEADING_DIM;
 
+  if (use_fused(m, n, k, batch, flags)) {
+    if (batch > (1 << 26)) // tile indices are 32-bit
+      return WMMAE_STATUS_NOT_SUPPORTED;
+    FusedArgs f;
+    wmmae_gemm::FusedParams &q = f.p;
+    q.A = A;
+    q.a_ptrs = a_ptrs;
+    q.a_rs = is_n(transa) ? 1 : lda;
+    q.a_ks = is_n(transa) ? lda : 1;
+    q.a_bs = stride_a;
+    q.B = B;
+    q.b_ptrs = b_ptrs;
+    q.b_rs = is_n(transb) ? ldb : 1;
+    q.b_ks = is_n(transb) ? 1 : ldb;
+    q.b_bs = stride_b;
+    q.C = C;
+    q.c_ptrs = c_ptrs;
+    q.ldc = ldc;
+    q.c_bs = stride_c;
+    q.M = m;
+    q.N = n;
+    q.K = k;
+    q.batch = batch;
+    const auto aligned16 = [](const void *ptr) {
+      return reinterpret_cast<uintptr_t>(ptr) % 16 == 0;
+    };
+    q.vec_a = q.a_ks == 1 && k % 4 == 0 && q.a_rs % 4 == 0 &&
+              (a_ptrs != nullptr || (aligned16(A) && stride_a % 4 == 0));
+    q.vec_b = q.b_ks == 1 && k % 4 == 0 && q.b_rs % 4 == 0 &&
+              (b_ptrs != nullptr || (aligned16(B) && stride_b % 4 == 0));
+    q.vec_store = (ldc % 4 == 0) &&
+                  (c_ptrs != nullptr || (aligned16(C) && stride_c % 4 == 0));
+    q.alpha = *alpha;
+    q.beta = *beta;
+    q.inv_scale = p.inv_scale;
+    f.stream = static_cast<hipStream_t>(stream);
+    return fused_dispatch(policy, f);
+  }
+
   size_t bytes_a = 0, bytes_b = 0, bytes_c = 0;
   wmmae_tcec_pack_bytes(m, k, batch, policy, &bytes_a);
   wmmae_tcec_pack_bytes(n, k, batch, policy, &bytes_b);
@@ -598,8 +701,8 @@ int wmmae_primitive_tiles(const float *const tiles, const long long num_tiles,
   if (!tiles || !a_row || !a_col || !b_row || !b_col || !acc_out || !vec_out)
     return WMMAE_STATUS_NULL_POINTER;
   long long blocks = (num_tiles + 3) / 4; // 4 waves per block, one tile per wave
-  if (blocks > 256 * 32)
-    blocks = 256 * 32; // grid-stride beyond this
+  if (blocks > (1 << 20))
+    blocks = 1 << 20; // grid-stride beyond this
   hipLaunchKernelGGL(wmmae_harness::primitive_tiles_kernel,
                      dim3(static_cast<unsigned>(blocks)), dim3(256), 0,
                      static_cast<hipStream_t>(stream), tiles, num_tiles,

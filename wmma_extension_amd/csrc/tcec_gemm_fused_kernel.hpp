@@ -1,0 +1,417 @@
+// TCEC SGEMM for gfx950 straight from the fp32 operands, for products that are
+// bound by HBM rather than by the matrix cores (small matrices, usually
+// batched: every element is needed by only a few workgroups).  The packed path
+// (split_pack_kernel + tcec_gemm_kernel) would read and write every operand
+// once more.  Here one kernel does it all:
+//
+//   HBM --global_load_lds--> raw fp32 ring in LDS (NRAW stages of 32 k)
+//       --split in registers--> 16-bit terms in LDS, two stages, in the same
+//         fragment-major chunk order the packed kernel uses
+//       --ds_read_b128--> MFMA operands
+//
+// The reference's tiled GEMM has the same shape of data flow (fp32 tiles in
+// shared memory, split at fragment load: test/tcec/batch_gemm.cu:196-386,
+// tcec/tcec.hpp:213-229) but splits every element once per warp that needs it;
+// here every element of a tile is split once per workgroup.
+//
+// Each wave requests, and later converts, the same row blocks, so the raw ring
+// needs no workgroup barrier: the wave's own s_waitcnt vmcnt is enough.  The
+// only barrier of a stage publishes the converted terms.
+//
+// Workgroups are persistent.  A workgroup walks a list of output tiles and
+// treats (tile, k stage) pairs as one stream, so the loads of the next tile
+// are in flight while the current one finishes and is written back: with
+// 8 stages a tile (k = 256) a pipeline refill per tile would cost as much as
+// the tile.  With eight or more batch entries, an XCD (blockIdx % 8) takes
+// whole batch entries, so the tiles that share an operand panel share an L2.
+//
+// Raw layout of one 16-row block of a stage (2 KiB): when k is contiguous and
+// 16-byte aligned, two 16-byte requests per lane, lane l fetching row l%16,
+// k = 8*(l/16) + 4*h .. +3 for h = 0, 1 into slot [h][l]; otherwise eight
+// 4-byte requests, element e of the lane's eight into slot [e][l].  Either
+// way lane l later reads its own eight floats from consecutive-lane slots.
+// Rows past the matrix are clamped to the last row (their results are never
+// stored); k past K is clamped in the request and zeroed at the conversion.
+//
+// Operand element (r, l) of op(A) is A[r*a_rs + l*a_ks] (rows = m), of op(B) it
+// is B[r*b_rs + l*b_ks] (rows = n); batch entry y is base + y*stride or ptrs[y].
+// The products, their order and the epilogue are those of tcec_gemm_kernel, so
+// both paths give the same bits.
+#pragma once
+#include "tcec_gemm_kernels.hpp"
+
+namespace wmmae_gemm {
+
+struct FusedParams {
+  const float *A;
+  const float *const *a_ptrs;
+  long long a_rs, a_ks, a_bs;
+  const float *B;
+  const float *const *b_ptrs;
+  long long b_rs, b_ks, b_bs;
+  float *C;
+  float *const *c_ptrs;
+  long long ldc, c_bs;
+  int M, N, K, batch;
+  int tiles_m, tiles_per_batch;
+  // 16-byte requests are possible as far as the host can tell: k contiguous,
+  // K and the strides multiples of 4, base pointers aligned (pointer-array
+  // entries are checked by the kernel)
+  int vec_a, vec_b;
+  int vec_store;
+  float alpha, beta, inv_scale;
+};
+
+template <int TERMS, int BM, int BN> struct FusedConfig {
+  static constexpr int RBA = BM / 16, RBB = BN / 16, NRB = RBA + RBB;
+  static constexpr int NQ = NRB / 4; // row blocks per wave and stage
+  static constexpr int RAW_STAGE_BYTES = NRB * 2048;
+  static constexpr int FRAG_BYTES = 2 * NRB * TERMS * 1024;
+  static constexpr int FIT = (160 * 1024 - FRAG_BYTES) / RAW_STAGE_BYTES;
+  static constexpr int NRAW = FIT > 4 ? 4 : FIT;
+  static constexpr int LDS_BYTES = NRAW * RAW_STAGE_BYTES + FRAG_BYTES;
+  static_assert(RBA % 4 == 0 && RBB % 4 == 0, "row blocks divide over 4 waves");
+  static_assert(NRAW >= 2, "raw ring too shallow");
+};
+
+template <int N> __device__ __forceinline__ void wait_vmcnt_at_most() {
+  asm volatile("s_waitcnt vmcnt(%0)" ::"n"(N > 63 ? 63 : N) : "memory");
+}
+
+template <class T, int TERMS, int BM, int BN>
+__global__ void __launch_bounds__(256)
+    tcec_gemm_fused_kernel(const FusedParams p) {
+  using traits = mtk::wmma::tcec::detail::split_traits<T>;
+  using S = typename traits::storage;
+  typedef S ab_vec __attribute__((ext_vector_type(8)));
+  using Cfg = FusedConfig<TERMS, BM, BN>;
+  constexpr int RBA = Cfg::RBA, NRB = Cfg::NRB, NQ = Cfg::NQ;
+  constexpr int NRAW = Cfg::NRAW;
+  constexpr int WM = BM / 2, WN = BN / 2; // 2 x 2 waves
+  constexpr int MT_ = WM / 16, NT_ = WN / 16;
+
+  extern __shared__ __attribute__((aligned(1024))) unsigned char lds_raw[];
+  u32x4 *const frag =
+      reinterpret_cast<u32x4 *>(lds_raw + NRAW * Cfg::RAW_STAGE_BYTES);
+
+  const unsigned lane = threadIdx.x & 63u;
+  const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+  const int wm = wave & 1, wn = wave >> 1;
+  const int r16 = static_cast<int>(lane & 15u);
+  const int g8 = 8 * static_cast<int>(lane >> 4);
+  const int M = p.M, N = p.N, K = p.K;
+
+  // ---- this workgroup's tiles: v = first + i*stride while v < count
+  const int tpb = p.tiles_per_batch;
+  const bool grouped = p.batch >= 8;
+  const int xcd = grouped ? static_cast<int>(blockIdx.x & 7u) : 0;
+  const int first = grouped ? static_cast<int>(blockIdx.x >> 3)
+                            : static_cast<int>(blockIdx.x);
+  const int stride = grouped ? static_cast<int>(gridDim.x >> 3)
+                             : static_cast<int>(gridDim.x);
+  const int count = grouped ? ((p.batch - xcd + 7) >> 3) * tpb : p.batch * tpb;
+  if (first >= count)
+    return;
+  const int n_my = (count - first + stride - 1) / stride;
+  auto decode = [&](const int i, int &entry, int &tm, int &tn) __attribute__((always_inline)) {
+    const int v = first + i * stride;
+    const int bi = v / tpb;
+    const int t = v - bi * tpb;
+    entry = grouped ? bi * 8 + xcd : bi;
+    tn = t / p.tiles_m;
+    tm = t - tn * p.tiles_m;
+  };
+
+  // ---- request width (uniform over the workgroup)
+  int vec_a = p.vec_a, vec_b = p.vec_b;
+  if (p.a_ptrs != nullptr || p.b_ptrs != nullptr) {
+    int low_a = 0, low_b = 0;
+    for (int i = threadIdx.x; i < n_my; i += 256) {
+      int entry, tm, tn;
+      decode(i, entry, tm, tn);
+      if (p.a_ptrs != nullptr)
+        low_a |= static_cast<int>(
+            reinterpret_cast<uintptr_t>(p.a_ptrs[entry]) & 15u);
+      if (p.b_ptrs != nullptr)
+        low_b |= static_cast<int>(
+            reinterpret_cast<uintptr_t>(p.b_ptrs[entry]) & 15u);
+    }
+    // workgroup-wide OR through the (still unused) start of the LDS ring
+    int *const flags = reinterpret_cast<int *>(lds_raw);
+    const int any_a = __builtin_amdgcn_ballot_w64(low_a != 0) != 0;
+    const int any_b = __builtin_amdgcn_ballot_w64(low_b != 0) != 0;
+    if (lane == 0)
+      flags[wave] = any_a | (any_b << 1);
+    __syncthreads();
+    const int all = flags[0] | flags[1] | flags[2] | flags[3];
+    __syncthreads();
+    if (all & 1)
+      vec_a = 0;
+    if (all & 2)
+      vec_b = 0;
+  }
+  vec_a = __builtin_amdgcn_readfirstlane(vec_a);
+  vec_b = __builtin_amdgcn_readfirstlane(vec_b);
+
+  const int num_k = (K + 31) / 32;
+  const int total = n_my * num_k; // stages in this workgroup's stream
+
+  // ---- requests
+  typedef const __attribute__((address_space(1))) float *gptr_t;
+  gptr_t rowptr[NQ];
+  auto set_rows = [&](const int i) __attribute__((always_inline)) {
+    int entry, tm, tn;
+    decode(i, entry, tm, tn);
+    // the pointer arrays are read with scalar loads (constant address space):
+    // a vector load here would make the compiler wait for every outstanding
+    // request of the ring before it can use the pointer
+    typedef const float *const __attribute__((address_space(4))) *ptr_array_t;
+    const float *const Ab = p.a_ptrs != nullptr
+                                ? ((ptr_array_t)p.a_ptrs)[entry]
+                                : p.A + static_cast<long long>(entry) * p.a_bs;
+    const float *const Bb = p.b_ptrs != nullptr
+                                ? ((ptr_array_t)p.b_ptrs)[entry]
+                                : p.B + static_cast<long long>(entry) * p.b_bs;
+#pragma unroll
+    for (int q = 0; q < NQ; q++) {
+      const int rbl = wave + 4 * q;
+      if (4 * q < RBA) {
+        int r = tm * BM + rbl * 16 + r16;
+        r = r < M ? r : M - 1;
+        rowptr[q] = (gptr_t)(Ab + static_cast<long long>(r) * p.a_rs);
+      } else {
+        int r = tn * BN + (rbl - RBA) * 16 + r16;
+        r = r < N ? r : N - 1;
+        rowptr[q] = (gptr_t)(Bb + static_cast<long long>(r) * p.b_rs);
+      }
+    }
+  };
+  // VEC: std::true_type for 16-byte requests (both operands), else 4-byte ones
+  auto issue = [&](auto VEC, const int ks, const int slot) __attribute__((always_inline)) {
+#pragma unroll
+    for (int q = 0; q < NQ; q++) {
+      const int rbl = wave + 4 * q;
+      unsigned char *const dst =
+          lds_raw + slot * Cfg::RAW_STAGE_BYTES + rbl * 2048;
+      if constexpr (decltype(VEC)::value) {
+#pragma unroll
+        for (int h = 0; h < 2; h++) {
+          int k = ks * 32 + g8 + 4 * h;
+          k = k < K ? k : 0; // K % 4 == 0 here: a piece is all in or all out
+          __builtin_amdgcn_global_load_lds(
+              (const __attribute__((address_space(1))) void *)(rowptr[q] + k),
+              (__attribute__((address_space(3))) void *)(dst + h * 1024), 16, 0,
+              0);
+        }
+      } else {
+        const long long kst = 4 * q < RBA ? p.a_ks : p.b_ks;
+#pragma unroll
+        for (int e = 0; e < 8; e++) {
+          int k = ks * 32 + g8 + e;
+          k = k < K ? k : K - 1;
+          __builtin_amdgcn_global_load_lds(
+              (const __attribute__((address_space(1))) void *)(rowptr[q] +
+                                                                k * kst),
+              (__attribute__((address_space(3))) void *)(dst + e * 256), 4, 0,
+              0);
+        }
+      }
+    }
+  };
+  // leave NRAW-1 stages of this wave's requests in flight
+  auto wait_oldest_stage = [&](auto VEC) __attribute__((always_inline)) {
+    constexpr int per_stage = NQ * (decltype(VEC)::value ? 2 : 8);
+    wait_vmcnt_at_most<(NRAW - 1) * per_stage>();
+  };
+  // raw slot -> split terms of fragment buffer `buf`
+  auto convert = [&](auto VEC, const int ks, const int slot, const int buf) __attribute__((always_inline)) {
+#pragma unroll
+    for (int q = 0; q < NQ; q++) {
+      const int rbl = wave + 4 * q;
+      const unsigned char *const src =
+          lds_raw + slot * Cfg::RAW_STAGE_BYTES + rbl * 2048;
+      float v[8];
+      if constexpr (decltype(VEC)::value) {
+        const f32x4 lo = reinterpret_cast<const f32x4 *>(src)[lane];
+        const f32x4 hi = reinterpret_cast<const f32x4 *>(src)[64 + lane];
+#pragma unroll
+        for (int x = 0; x < 4; x++) {
+          v[x] = lo[x];
+          v[4 + x] = hi[x];
+        }
+      } else {
+#pragma unroll
+        for (int e = 0; e < 8; e++)
+          v[e] = reinterpret_cast<const float *>(src)[e * 64 + lane];
+      }
+      const int left = K - (ks * 32 + g8); // k past K was clamped: zero it
+      ab_vec t[3];
+#pragma unroll
+      for (int x = 0; x < 8; x++) {
+        S t0, t1, t2;
+        traits::split(x < left ? v[x] : 0.f, t0, t1, t2);
+        t[0][x] = t0;
+        t[1][x] = t1;
+        t[2][x] = t2;
+      }
+#pragma unroll
+      for (int c = 0; c < TERMS; c++)
+        frag[((buf * NRB + rbl) * TERMS + c) * 64 + lane] =
+            __builtin_bit_cast(u32x4, t[c]);
+    }
+  };
+  auto mfma = [](const ab_vec x, const ab_vec y, const f32x4 z) -> f32x4 {
+    if constexpr (std::is_same<S, _Float16>::value)
+      return __builtin_amdgcn_mfma_f32_16x16x32_f16(x, y, z, 0, 0, 0);
+    else
+      return __builtin_amdgcn_mfma_f32_16x16x32_bf16(x, y, z, 0, 0, 0);
+  };
+
+  f32x4 acc_main[MT_][NT_], acc_err[MT_][NT_];
+  auto clear_acc = [&]() __attribute__((always_inline)) {
+#pragma unroll
+    for (int i = 0; i < MT_; i++)
+#pragma unroll
+      for (int j = 0; j < NT_; j++) {
+        acc_main[i][j] = f32x4{0.f, 0.f, 0.f, 0.f};
+        acc_err[i][j] = f32x4{0.f, 0.f, 0.f, 0.f};
+      }
+  };
+  auto store_tile = [&](const int i_tile) __attribute__((always_inline)) {
+    int entry, tm, tn;
+    decode(i_tile, entry, tm, tn);
+    typedef float *const __attribute__((address_space(4))) *out_array_t;
+    float *const Cb = p.c_ptrs != nullptr
+                          ? ((out_array_t)p.c_ptrs)[entry]
+                          : p.C + static_cast<long long>(entry) * p.c_bs;
+    const int vec_out =
+        p.vec_store && (reinterpret_cast<uintptr_t>(Cb) & 15u) == 0;
+    const float alpha = p.alpha, beta = p.beta;
+    const int row_base = tm * BM + wm * WM + 4 * static_cast<int>(lane >> 4);
+    const int col_base = tn * BN + wn * WN + r16;
+#pragma unroll
+    for (int j = 0; j < NT_; j++) {
+      const int col = col_base + 16 * j;
+      if (col >= N)
+        continue;
+#pragma unroll
+      for (int i = 0; i < MT_; i++) {
+        const int row = row_base + 16 * i;
+        if (row >= M)
+          continue;
+        f32x4 o = acc_main[i][j];
+        if constexpr (TERMS >= 2)
+          o += acc_err[i][j] * p.inv_scale;
+        o *= alpha;
+        float *const dst = Cb + row + static_cast<long long>(col) * p.ldc;
+        if (vec_out && row + 3 < M) {
+          if (beta != 0.f)
+            o += beta * *reinterpret_cast<const f32x4 *>(dst);
+          *reinterpret_cast<f32x4 *>(dst) = o;
+        } else {
+#pragma unroll
+          for (int x = 0; x < 4; x++) {
+            if (row + x < M) {
+              float e = o[x];
+              if (beta != 0.f)
+                e += beta * dst[x];
+              dst[x] = e;
+            }
+          }
+        }
+      }
+    }
+  };
+
+  auto run = [&](auto VEC) __attribute__((always_inline)) {
+    // ---- prologue: fill the raw ring, convert stage 0
+    int req_tile = 0, req_ks = 0; // next (tile, k stage) to request
+    auto advance_request = [&]() __attribute__((always_inline)) {
+      if (req_ks + 1 < num_k) {
+        req_ks++;
+      } else if (req_tile + 1 < n_my) {
+        req_tile++;
+        req_ks = 0;
+        set_rows(req_tile);
+      } // else: stay on the last stage; the redundant requests land in free
+        // slots and keep the in-flight count constant
+    };
+    set_rows(0);
+    for (int s = 0; s < NRAW; s++) {
+      issue(VEC, req_ks, s);
+      advance_request();
+    }
+    wait_oldest_stage(VEC);
+    convert(VEC, 0, 0, 0);
+    clear_acc();
+    asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");
+
+    int cur_tile = 0, cur_ks = 0; // stage being multiplied
+    int slot_cur = 0;             // its raw slot (already converted, free)
+    for (int s = 0; s < total; s++) {
+      const int buf = s & 1;
+      // refill the slot that stage s has left
+      issue(VEC, req_ks, slot_cur);
+      advance_request();
+
+      const u32x4 *const sa =
+          frag + ((buf * NRB + wm * MT_) * TERMS) * 64 + lane;
+      const u32x4 *const sb =
+          frag + ((buf * NRB + RBA + wn * NT_) * TERMS) * 64 + lane;
+      ab_vec a[TERMS][MT_], b[TERMS][NT_];
+#pragma unroll
+      for (int j = 0; j < NT_; j++)
+#pragma unroll
+        for (int t = 0; t < TERMS; t++)
+          b[t][j] = __builtin_bit_cast(ab_vec, sb[(j * TERMS + t) * 64]);
+#pragma unroll
+      for (int i = 0; i < MT_; i++)
+#pragma unroll
+        for (int t = 0; t < TERMS; t++)
+          a[t][i] = __builtin_bit_cast(ab_vec, sa[(i * TERMS + t) * 64]);
+
+      // next stage: raw -> terms, into the other fragment buffer.  After the
+      // last stage this converts a redundant tail request; nobody reads it.
+      const int slot_next = slot_cur + 1 == NRAW ? 0 : slot_cur + 1;
+      const int next_ks = cur_ks + 1 == num_k ? 0 : cur_ks + 1;
+      wait_oldest_stage(VEC);
+      convert(VEC, next_ks, slot_next, buf ^ 1);
+
+      auto sweep = [&](f32x4(&acc)[MT_][NT_], const int ta, const int tb) {
+#pragma unroll
+        for (int i = 0; i < MT_; i++)
+#pragma unroll
+          for (int j = 0; j < NT_; j++)
+            acc[i][j] = mfma(a[ta][i], b[tb][j], acc[i][j]);
+      };
+      // same products and order as tcec_gemm_kernel
+      if constexpr (TERMS >= 3) {
+        sweep(acc_err, 2, 0);
+        sweep(acc_err, 0, 2);
+        sweep(acc_err, 1, 1);
+      }
+      if constexpr (TERMS >= 2) {
+        sweep(acc_err, 1, 0);
+        sweep(acc_err, 0, 1);
+      }
+      sweep(acc_main, 0, 0);
+
+      if (next_ks == 0) { // the tile is complete
+        store_tile(cur_tile);
+        clear_acc();
+        cur_tile++;
+      }
+      cur_ks = next_ks;
+      slot_cur = slot_next;
+      asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");
+    }
+  };
+  if (vec_a && vec_b)
+    run(std::true_type{});
+  else
+    run(std::false_type{});
+  // the redundant tail requests still write LDS: drain them before the end
+  asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)" ::: "memory");
+}
+
+} // namespace wmmae_gemm
