@@ -273,7 +273,8 @@ template <class T, int TERMS, int BM, int BN> int launch_fused(FusedArgs f) {
   if (per_xcd > per_xcd_max)
     per_xcd = per_xcd_max;
   const int grid = 8 * static_cast<int>(per_xcd);
-  hipLaunchKernelGGL(kernel, dim3(grid), dim3(256), Cfg::LDS_BYTES, f.stream,
+  hipLaunchKernelGGL(kernel, dim3(grid), dim3(Cfg::NTHREADS), Cfg::LDS_BYTES,
+                     f.stream,
                      p);
   return launch_status();
 }

@@ -62,15 +62,19 @@ struct FusedParams {
   float alpha, beta, inv_scale;
 };
 
-template <int TERMS, int BM, int BN> struct FusedConfig {
+template <int TERMS, int BM, int BN, int NW = (BM * BN >= 128 * 128 ? 8 : 4)>
+struct FusedConfig {
+  static constexpr int NWAVES = NW;       // 2 x NW/2 waves
+  static constexpr int NTHREADS = 64 * NW;
   static constexpr int RBA = BM / 16, RBB = BN / 16, NRB = RBA + RBB;
-  static constexpr int NQ = NRB / 4; // row blocks per wave and stage
+  static constexpr int NQ = NRB / NW; // row blocks per wave and stage
   static constexpr int RAW_STAGE_BYTES = NRB * 2048;
   static constexpr int FRAG_BYTES = 2 * NRB * TERMS * 1024;
   static constexpr int FIT = (160 * 1024 - FRAG_BYTES) / RAW_STAGE_BYTES;
   static constexpr int NRAW = FIT > 4 ? 4 : FIT;
   static constexpr int LDS_BYTES = NRAW * RAW_STAGE_BYTES + FRAG_BYTES;
-  static_assert(RBA % 4 == 0 && RBB % 4 == 0, "row blocks divide over 4 waves");
+  static_assert(RBA % NW == 0 && RBB % NW == 0,
+                "row blocks divide over the waves");
   static_assert(NRAW >= 2, "raw ring too shallow");
 };
 
@@ -78,16 +82,21 @@ template <int N> __device__ __forceinline__ void wait_vmcnt_at_most() {
   asm volatile("s_waitcnt vmcnt(%0)" ::"n"(N > 63 ? 63 : N) : "memory");
 }
 
-template <class T, int TERMS, int BM, int BN>
-__global__ void __launch_bounds__(256)
+// ABLATE (tuning only, 0 in the library): bit 0 drops the global->LDS requests,
+// bit 1 the conversion, bit 2 the MFMAs, bit 3 the per-stage barrier, bit 4 the
+// stores of C.
+template <class T, int TERMS, int BM, int BN, int ABLATE = 0,
+          int NW = FusedConfig<TERMS, BM, BN>::NWAVES>
+__global__ void __launch_bounds__(64 * NW)
     tcec_gemm_fused_kernel(const FusedParams p) {
   using traits = mtk::wmma::tcec::detail::split_traits<T>;
   using S = typename traits::storage;
   typedef S ab_vec __attribute__((ext_vector_type(8)));
-  using Cfg = FusedConfig<TERMS, BM, BN>;
+  using Cfg = FusedConfig<TERMS, BM, BN, NW>;
   constexpr int RBA = Cfg::RBA, NRB = Cfg::NRB, NQ = Cfg::NQ;
   constexpr int NRAW = Cfg::NRAW;
-  constexpr int WM = BM / 2, WN = BN / 2; // 2 x 2 waves
+  constexpr int WGN = NW / 2;
+  constexpr int WM = BM / 2, WN = BN / WGN; // 2 x NW/2 waves
   constexpr int MT_ = WM / 16, NT_ = WN / 16;
 
   extern __shared__ __attribute__((aligned(1024))) unsigned char lds_raw[];
@@ -126,7 +135,7 @@ __global__ void __launch_bounds__(256)
   int vec_a = p.vec_a, vec_b = p.vec_b;
   if (p.a_ptrs != nullptr || p.b_ptrs != nullptr) {
     int low_a = 0, low_b = 0;
-    for (int i = threadIdx.x; i < n_my; i += 256) {
+    for (int i = threadIdx.x; i < n_my; i += 64 * NW) {
       int entry, tm, tn;
       decode(i, entry, tm, tn);
       if (p.a_ptrs != nullptr)
@@ -143,7 +152,10 @@ __global__ void __launch_bounds__(256)
     if (lane == 0)
       flags[wave] = any_a | (any_b << 1);
     __syncthreads();
-    const int all = flags[0] | flags[1] | flags[2] | flags[3];
+    int all = 0;
+#pragma unroll
+    for (int w = 0; w < NW; w++)
+      all |= flags[w];
     __syncthreads();
     if (all & 1)
       vec_a = 0;
@@ -174,8 +186,8 @@ __global__ void __launch_bounds__(256)
                                 : p.B + static_cast<long long>(entry) * p.b_bs;
 #pragma unroll
     for (int q = 0; q < NQ; q++) {
-      const int rbl = wave + 4 * q;
-      if (4 * q < RBA) {
+      const int rbl = wave + NW * q;
+      if (NW * q < RBA) {
         int r = tm * BM + rbl * 16 + r16;
         r = r < M ? r : M - 1;
         rowptr[q] = (gptr_t)(Ab + static_cast<long long>(r) * p.a_rs);
@@ -188,9 +200,11 @@ __global__ void __launch_bounds__(256)
   };
   // VEC: std::true_type for 16-byte requests (both operands), else 4-byte ones
   auto issue = [&](auto VEC, const int ks, const int slot) __attribute__((always_inline)) {
+    if constexpr ((ABLATE & 1) != 0)
+      return;
 #pragma unroll
     for (int q = 0; q < NQ; q++) {
-      const int rbl = wave + 4 * q;
+      const int rbl = wave + NW * q;
       unsigned char *const dst =
           lds_raw + slot * Cfg::RAW_STAGE_BYTES + rbl * 2048;
       if constexpr (decltype(VEC)::value) {
@@ -204,7 +218,7 @@ __global__ void __launch_bounds__(256)
               0);
         }
       } else {
-        const long long kst = 4 * q < RBA ? p.a_ks : p.b_ks;
+        const long long kst = NW * q < RBA ? p.a_ks : p.b_ks;
 #pragma unroll
         for (int e = 0; e < 8; e++) {
           int k = ks * 32 + g8 + e;
@@ -225,9 +239,11 @@ __global__ void __launch_bounds__(256)
   };
   // raw slot -> split terms of fragment buffer `buf`
   auto convert = [&](auto VEC, const int ks, const int slot, const int buf) __attribute__((always_inline)) {
+    if constexpr ((ABLATE & 2) != 0)
+      return;
 #pragma unroll
     for (int q = 0; q < NQ; q++) {
-      const int rbl = wave + 4 * q;
+      const int rbl = wave + NW * q;
       const unsigned char *const src =
           lds_raw + slot * Cfg::RAW_STAGE_BYTES + rbl * 2048;
       float v[8];
@@ -244,15 +260,37 @@ __global__ void __launch_bounds__(256)
         for (int e = 0; e < 8; e++)
           v[e] = reinterpret_cast<const float *>(src)[e * 64 + lane];
       }
-      const int left = K - (ks * 32 + g8); // k past K was clamped: zero it
+      // k past K was clamped in the request: zero it (last stage only)
+      if (ks * 32 + 32 > K) {
+        const int left = K - (ks * 32 + g8);
+#pragma unroll
+        for (int x = 0; x < 8; x++)
+          v[x] = x < left ? v[x] : 0.f;
+      }
+      // the split of split_traits<T>, two elements at a time so that the
+      // packed conversions are used: t0 = RN16(v), t1 = RN16((v - t0) * scale),
+      // t2 = RN16((v - t0) - t1)
+      typedef S s2_t __attribute__((ext_vector_type(2)));
+      typedef float f2_t __attribute__((ext_vector_type(2)));
       ab_vec t[3];
 #pragma unroll
-      for (int x = 0; x < 8; x++) {
-        S t0, t1, t2;
-        traits::split(x < left ? v[x] : 0.f, t0, t1, t2);
-        t[0][x] = t0;
-        t[1][x] = t1;
-        t[2][x] = t2;
+      for (int x = 0; x < 8; x += 2) {
+        const f2_t vv = {v[x], v[x + 1]};
+        const s2_t h0 = __builtin_convertvector(vv, s2_t);
+        f2_t r = vv - __builtin_convertvector(h0, f2_t);
+        if constexpr (traits::scale != 1.f)
+          r *= traits::scale;
+        const s2_t h1 = __builtin_convertvector(r, s2_t);
+        s2_t h2 = h1;
+        if constexpr (traits::num_terms >= 3)
+          h2 = __builtin_convertvector(r - __builtin_convertvector(h1, f2_t),
+                                       s2_t);
+        t[0][x] = h0[0];
+        t[0][x + 1] = h0[1];
+        t[1][x] = h1[0];
+        t[1][x + 1] = h1[1];
+        t[2][x] = h2[0];
+        t[2][x + 1] = h2[1];
       }
 #pragma unroll
       for (int c = 0; c < TERMS; c++)
@@ -261,7 +299,10 @@ __global__ void __launch_bounds__(256)
     }
   };
   auto mfma = [](const ab_vec x, const ab_vec y, const f32x4 z) -> f32x4 {
-    if constexpr (std::is_same<S, _Float16>::value)
+    if constexpr ((ABLATE & 4) != 0)
+      return z + f32x4{static_cast<float>(x[0]), static_cast<float>(y[0]), 0.f,
+                       0.f};
+    else if constexpr (std::is_same<S, _Float16>::value)
       return __builtin_amdgcn_mfma_f32_16x16x32_f16(x, y, z, 0, 0, 0);
     else
       return __builtin_amdgcn_mfma_f32_16x16x32_bf16(x, y, z, 0, 0, 0);
@@ -346,64 +387,70 @@ __global__ void __launch_bounds__(256)
     clear_acc();
     asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");
 
-    int cur_tile = 0, cur_ks = 0; // stage being multiplied
-    int slot_cur = 0;             // its raw slot (already converted, free)
-    for (int s = 0; s < total; s++) {
-      const int buf = s & 1;
-      // refill the slot that stage s has left
-      issue(VEC, req_ks, slot_cur);
-      advance_request();
+    // The k loop of a tile is a loop of its own so that the accumulators are
+    // touched by nothing but MFMAs inside it (they stay in AGPRs); the stream
+    // of requests and conversions runs on across the tile boundary.
+    int slot_cur = 0; // raw slot of the stage being multiplied (converted, free)
+    int s = 0;        // its index in the stream
+    for (int cur_tile = 0; cur_tile < n_my; cur_tile++) {
+      clear_acc();
+      for (int cur_ks = 0; cur_ks < num_k; cur_ks++, s++) {
+        const int buf = s & 1;
+        // refill the slot that stage s has left
+        issue(VEC, req_ks, slot_cur);
+        advance_request();
 
-      const u32x4 *const sa =
-          frag + ((buf * NRB + wm * MT_) * TERMS) * 64 + lane;
-      const u32x4 *const sb =
-          frag + ((buf * NRB + RBA + wn * NT_) * TERMS) * 64 + lane;
-      ab_vec a[TERMS][MT_], b[TERMS][NT_];
+        const u32x4 *const sa =
+            frag + ((buf * NRB + wm * MT_) * TERMS) * 64 + lane;
+        const u32x4 *const sb =
+            frag + ((buf * NRB + RBA + wn * NT_) * TERMS) * 64 + lane;
+        ab_vec a[TERMS][MT_], b[TERMS][NT_];
 #pragma unroll
-      for (int j = 0; j < NT_; j++)
+        for (int j = 0; j < NT_; j++)
 #pragma unroll
-        for (int t = 0; t < TERMS; t++)
-          b[t][j] = __builtin_bit_cast(ab_vec, sb[(j * TERMS + t) * 64]);
-#pragma unroll
-      for (int i = 0; i < MT_; i++)
-#pragma unroll
-        for (int t = 0; t < TERMS; t++)
-          a[t][i] = __builtin_bit_cast(ab_vec, sa[(i * TERMS + t) * 64]);
-
-      // next stage: raw -> terms, into the other fragment buffer.  After the
-      // last stage this converts a redundant tail request; nobody reads it.
-      const int slot_next = slot_cur + 1 == NRAW ? 0 : slot_cur + 1;
-      const int next_ks = cur_ks + 1 == num_k ? 0 : cur_ks + 1;
-      wait_oldest_stage(VEC);
-      convert(VEC, next_ks, slot_next, buf ^ 1);
-
-      auto sweep = [&](f32x4(&acc)[MT_][NT_], const int ta, const int tb) {
+          for (int t = 0; t < TERMS; t++)
+            b[t][j] = __builtin_bit_cast(ab_vec, sb[(j * TERMS + t) * 64]);
 #pragma unroll
         for (int i = 0; i < MT_; i++)
 #pragma unroll
-          for (int j = 0; j < NT_; j++)
-            acc[i][j] = mfma(a[ta][i], b[tb][j], acc[i][j]);
-      };
-      // same products and order as tcec_gemm_kernel
-      if constexpr (TERMS >= 3) {
-        sweep(acc_err, 2, 0);
-        sweep(acc_err, 0, 2);
-        sweep(acc_err, 1, 1);
-      }
-      if constexpr (TERMS >= 2) {
-        sweep(acc_err, 1, 0);
-        sweep(acc_err, 0, 1);
-      }
-      sweep(acc_main, 0, 0);
+          for (int t = 0; t < TERMS; t++)
+            a[t][i] = __builtin_bit_cast(ab_vec, sa[(i * TERMS + t) * 64]);
 
-      if (next_ks == 0) { // the tile is complete
-        store_tile(cur_tile);
-        clear_acc();
-        cur_tile++;
+        // next stage: raw -> terms, into the other fragment buffer.  After
+        // the last stage this converts a redundant tail request; nobody
+        // reads it.
+        const int slot_next = slot_cur + 1 == NRAW ? 0 : slot_cur + 1;
+        const int next_ks = cur_ks + 1 == num_k ? 0 : cur_ks + 1;
+        wait_oldest_stage(VEC);
+        convert(VEC, next_ks, slot_next, buf ^ 1);
+
+        auto sweep = [&](f32x4(&acc)[MT_][NT_], const int ta, const int tb) __attribute__((always_inline)) {
+#pragma unroll
+          for (int i = 0; i < MT_; i++)
+#pragma unroll
+            for (int j = 0; j < NT_; j++)
+              acc[i][j] = mfma(a[ta][i], b[tb][j], acc[i][j]);
+        };
+        // same products and order as tcec_gemm_kernel
+        if constexpr (TERMS >= 3) {
+          sweep(acc_err, 2, 0);
+          sweep(acc_err, 0, 2);
+          sweep(acc_err, 1, 1);
+        }
+        if constexpr (TERMS >= 2) {
+          sweep(acc_err, 1, 0);
+          sweep(acc_err, 0, 1);
+        }
+        sweep(acc_main, 0, 0);
+
+        slot_cur = slot_next;
+        if constexpr ((ABLATE & 8) == 0)
+          asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");
       }
-      cur_ks = next_ks;
-      slot_cur = slot_next;
-      asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");
+      if constexpr ((ABLATE & 16) == 0)
+        store_tile(cur_tile);
+      else if (acc_main[0][0][0] == 123.456f) // keep the accumulators alive
+        store_tile(cur_tile);
     }
   };
   if (vec_a && vec_b)
