@@ -44,17 +44,36 @@ def test_bf16_conversion_matches_torch(orc):
     assert ok.all(), f"{np.count_nonzero(~ok)} mismatches"
 
 
-@pytest.mark.slow
-def test_f16_conversion_exhaustive(orc):
-    """All 2^32 fp32 patterns against numpy (minutes; run with -m slow)."""
+def test_f16_conversion_sweep(orc):
+    """fp32 -> fp16 of the oracle against numpy over the whole 32-bit pattern space:
+    every 61st pattern by default (70 M values, all exponents, ties and subnormals
+    included through the halfway patterns added below); all 2^32 patterns with
+    WMMAE_EXHAUSTIVE=1 (about ten minutes)."""
+    import os
+    stride = 1 if os.environ.get("WMMAE_EXHAUSTIVE") == "1" else 61
     step = 1 << 26
     for start in range(0, 1 << 32, step):
-        bits = np.arange(start, start + step, dtype=np.uint64).astype(np.uint32)
+        bits = np.arange(start, start + step, stride, dtype=np.uint64).astype(np.uint32)
         v = bits.view(np.float32)
         hi = orc.split(orc.SPLIT_F16, v)[0]
         with np.errstate(all="ignore"):
             ref = v.astype(np.float16).view(np.uint16)
         assert (np.isnan(v) | (hi == ref)).all()
+    # every exact halfway case and its two neighbours, for all exponents and both signs:
+    # mantissa patterns x * 2^13 + {2^12 - 1, 2^12, 2^12 + 1} (normal range) and the wider
+    # ties of the fp16 subnormal range
+    expo = np.arange(0, 256, dtype=np.uint32)[:, None, None] << np.uint32(23)
+    hi10 = np.arange(0, 1024, dtype=np.uint32)[None, :, None] << np.uint32(13)
+    for shift in range(12, 24):
+        half = np.uint32(1) << np.uint32(shift)
+        tail = np.array([half - 1, half, half + 1], dtype=np.uint32)[None, None, :]
+        bits = ((expo | hi10) & ~np.uint32((1 << (shift + 1)) - 1) & np.uint32(0x7FFFFFFF)) | tail
+        for sign in (np.uint32(0), np.uint32(0x80000000)):
+            v = (bits | sign).ravel().view(np.float32)
+            got = orc.split(orc.SPLIT_F16, v)[0]
+            with np.errstate(all="ignore"):
+                ref = v.astype(np.float16).view(np.uint16)
+            assert (np.isnan(v) | (got == ref)).all()
 
 
 def test_f16_split_closed_form(orc):
