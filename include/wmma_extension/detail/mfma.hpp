@@ -76,6 +76,32 @@ template <> struct mfma_op<float, 32, 32, 2> {
   }
 };
 
+// A 16x16x16 fp32 product as four chained 16x16x4 steps.  Register x of an
+// operand fragment holds k = 4*(lane/16) + x, and step x of the chain consumes
+// register x of both operands, so every k is used exactly once; inside a step
+// the four lane groups supply k = x, 4+x, 8+x, 12+x.
+template <> struct mfma_op<float, 16, 16, 16> {
+  using ab_vec = vec_t<float, 4>;
+  using c_vec = vec_t<float, 4>;
+  static WMMAE_D c_vec run(const ab_vec a, const ab_vec b, c_vec c) {
+#pragma unroll
+    for (int x = 0; x < 4; x++)
+      c = __builtin_amdgcn_mfma_f32_16x16x4f32(a[x], b[x], c, 0, 0, 0);
+    return c;
+  }
+};
+// 32x32x8 fp32 as four chained 32x32x2 steps (k = 4*(lane/32) + x).
+template <> struct mfma_op<float, 32, 32, 8> {
+  using ab_vec = vec_t<float, 4>;
+  using c_vec = vec_t<float, 16>;
+  static WMMAE_D c_vec run(const ab_vec a, const ab_vec b, c_vec c) {
+#pragma unroll
+    for (int x = 0; x < 4; x++)
+      c = __builtin_amdgcn_mfma_f32_32x32x2f32(a[x], b[x], c, 0, 0, 0);
+    return c;
+  }
+};
+
 } // namespace gfx950
 } // namespace detail
 

@@ -17,6 +17,13 @@ namespace tcec {
 struct op_mfma;
 using op_mma = op_mfma;
 using op_wmma = op_mfma;
+// Plain fp32 operands, no split (reference: tcec/detail/policy_simt.hpp:14,
+// docs/mma_f32.md:139-152, where this policy runs on the SIMT cores with
+// warp shuffles).  On gfx950 the matrix core has an fp32 path
+// (v_mfma_f32_16x16x4_f32) at the rate of the vector ALUs, so the policy keeps
+// its name and its 16x16x16 shape but issues four fp32 MFMAs per sub-block.
+struct op_simt;
+using op_fp32 = op_simt;
 
 // Error correction policy
 struct with_ec;
@@ -44,8 +51,21 @@ struct default_policy {
   using type = Policy<op_mfma, ErrorCorrection, 16, 16, 32>;
 };
 
+// default_policy<float, without_ec, op_simt>::type
+// (reference: tcec/detail/policy_simt.hpp:21-27)
+template <class T, class Sm>
+struct default_policy<T, without_ec, op_simt, Sm> {
+  using type = Policy<op_simt, without_ec, 16, 16, 16>;
+};
+
 template <class Use, class T, class Layout, class Policy>
 struct default_fragment;
+template <class Use, class T, class Layout, class ErrorCorrection, int fm,
+          int fn, int fk>
+struct default_fragment<Use, T, Layout,
+                        Policy<op_simt, ErrorCorrection, fm, fn, fk>> {
+  using type = mtk::wmma::fragment<Use, fm, fn, fk, float, Layout>;
+};
 template <class Use, class T, class Layout, class ErrorCorrection, int fm,
           int fn, int fk>
 struct default_fragment<Use, T, Layout,

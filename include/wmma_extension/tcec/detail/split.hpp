@@ -6,6 +6,7 @@
 //                 (reference: tcec/tcec.hpp:219-223 with tcec/detail/scale.hpp:8-20)
 //   bfloat16    : v ~ hi + lo            two bf16 terms, ~16 significand bits
 //   precision::tf32 : v ~ hi + mid + lo  three bf16 terms, ~24 significand bits
+//   float       : v itself (op_simt policy, fp32 MFMA)
 // gfx950 has no xf32 MFMA; the reference's tf32 policy (two 11-bit terms,
 // ~22 bits, no scaling) is replaced by the three-term bf16 split, which keeps
 // fp32's exponent range and needs no scaling.
@@ -58,6 +59,18 @@ template <> struct split_traits<mtk::wmma::precision::tf32> {
     t1 = static_cast<storage>(r1);
     const float r2 = r1 - static_cast<float>(t1);
     t2 = static_cast<storage>(r2);
+  }
+};
+
+// fp32 operands kept whole (the op_simt policy): one term, nothing to correct.
+template <> struct split_traits<float> {
+  using mma_tag = float;
+  using storage = float;
+  static constexpr int num_terms = 1;
+  static constexpr float scale = 1.f;
+  static WMMAE_HD void split(const float v, storage &t0, storage &,
+                             storage &) {
+    t0 = v;
   }
 };
 

@@ -169,7 +169,10 @@ int wmmae_layout_dump(int use, int m, int n, int k, int col, int *ij,
 
 /* One-wave TCEC product D = A*B (+C), every operand in one tcec::fragment.
  * shape: 0 -> m=n=k=32, 1 -> (m,n,k) = (16,48,64) [(32,64,32) for inst 2];
- * type: 0 half, 1 bfloat16, 2 tf32; ec: 1 with_ec, 0 without_ec;
+ * type: 0 half, 1 bfloat16, 2 tf32, 3 float (the fp32 policy
+ * default_policy<float, without_ec, op_simt>, reference docs/mma_f32.md:139-152:
+ * ec must be 0, inst is ignored, the shape is 16x16x16; with ec != 0 the
+ * entry points return WMMAE_STATUS_NOT_SUPPORTED); ec: 1 with_ec, 0 without_ec;
  * inst: 0 -> 16x16x32, 1 -> 16x16x16, 2 -> 32x32x16; *_col: memory layouts
  * (1 = column major, dense leading dimension); c may be NULL;
  * rounding: 0 mma_sync, 1 mma_rn_sync, 2 mma_rz_sync.
@@ -194,6 +197,7 @@ int wmmae_tcec_matvec(int type, int ec, float *y, const float *a,
 /* 16-bit split terms held by a 32x32x32 operand fragment (use 0/1) after
  * load_matrix_sync (from_vector == 0) or load_vector (from_vector != 0):
  * terms[(term*E + e)*64 + lane], E = fragment num_elements, e = index of x(e).
+ * type 0..2 only (fp32 fragments hold no 16-bit terms).
  * Replaces: test/tcec/vector.cu:15-61 and test/tcec/elementwise.cu:7-26. */
 int wmmae_tcec_frag_dump(int use, int type, int ec, int frag_col,
                          unsigned short *terms, const float *src,

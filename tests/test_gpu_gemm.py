@@ -323,3 +323,29 @@ def test_api_level_gemm_matches_driver(tc, orc, dev, type_ec):
     with pytest.raises(WmmaeError) as e:
         tc.api_gemm(type_, ec, 100, n, k, 1.0, dA, k, dB, k, 0.0, dC, 100)
     assert e.value.status == -4
+
+
+def test_api_level_gemm_fp32_policy(tc, orc, dev):
+    """The same API-level GEMM with default_policy<float, without_ec, op_simt>: a plain
+    fp32 product on the matrix core's fp32 path, the on-GPU comparator of the 2x gate."""
+    m, n, k = 256, 128, 2048
+    rng = np.random.default_rng(99)
+    A = rng.uniform(-1, 1, (m, k)).astype(np.float32)
+    Bt = rng.uniform(-1, 1, (n, k)).astype(np.float32)
+    dA, dB = torch.from_numpy(A).to(dev), torch.from_numpy(Bt).to(dev)
+    dC = torch.zeros((n, m), dtype=torch.float32, device=dev)
+    tc.api_gemm(3, 0, m, n, k, 1.0, dA, k, dB, k, 0.0, dC, m)
+    torch.cuda.synchronize()
+    got = dC.cpu().numpy().T
+    ref = orc.gemm_f64(A, Bt.T)
+    e_gpu = orc.max_rel_err(got, ref)
+    e_cpu = orc.max_rel_err(orc.gemm_f32(A, Bt.T), ref)
+    # two fp32 summations in different orders: same error scale, neither exact
+    assert e_gpu <= 4 * e_cpu and e_gpu > 0
+    # and TCEC with error correction on the same inputs is no worse than 2x either of them
+    e_tcec = orc.max_rel_err(_gemm(tc, dev, A, Bt.T, 0), ref)
+    assert e_tcec <= 2 * min(e_gpu, e_cpu)
+    from wmma_extension_amd._lib import WmmaeError
+    with pytest.raises(WmmaeError) as e:
+        tc.api_gemm(3, 1, m, n, k, 1.0, dA, k, dB, k, 0.0, dC, m)
+    assert e.value.status == -4

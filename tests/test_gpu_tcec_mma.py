@@ -207,3 +207,73 @@ def test_elementwise_accessors_neg_integrate(tc, orc, dev, type_, ec, inst):
                 # store and integrate both evaluate main + err/scale in fp32
                 expect = np.float32(main + np.float32(err / np.float32(scale)))
                 assert got[i, j] == expect, (do_neg, do_int, lane, e)
+
+
+# ---------------------------------------------------------------- fp32 policy (op_simt)
+def test_fp32_policy_mma_tile(tc, orc, dev):
+    """default_policy<float, without_ec, op_simt>: fp32 operands, no split
+    (docs/mma_f32.md:139-152).  All layouts; the result is a plain fp32 product, so it
+    sits within a few fp32 ulps of the oracle's fp32 loop and meets the with_ec gate of
+    the reference's mma test although nothing is corrected."""
+    for shape in (0, 1):
+        m, n, k = _dims(shape, 1)
+        rng = np.random.default_rng(300 + shape)
+        for a_col, b_col, c_col, d_col, with_c in itertools.product((0, 1), repeat=5):
+            A = rng.uniform(-1, 1, (m, k)).astype(np.float32)
+            B = rng.uniform(-1, 1, (k, n)).astype(np.float32)
+            C = rng.uniform(-1, 1, (m, n)).astype(np.float32) if with_c else None
+            D = _run(tc, dev, shape, 3, 0, 1, A, B, C, a_col, b_col, c_col, d_col, 0)
+            ref = orc.gemm_f64(A, B) + (C if with_c else 0)
+            f32 = orc.gemm_f32(A, B) + (C if with_c else 0)
+            assert orc.max_abs_err(D, ref) < TH_EC
+            assert np.abs(D - f32).max() <= 16 * 2.0**-24 * max(1.0, np.abs(ref).max())
+    # error correction does not exist for fp32 operands
+    from wmma_extension_amd._lib import WmmaeError
+    with pytest.raises(WmmaeError) as e:
+        _run(tc, dev, 0, 3, 1, 1, A[:32, :32], B[:32, :32], None, 0, 0, 0, 0, 0)
+    assert e.value.status == -4
+
+
+def test_fp32_policy_exact_and_identity(tc, orc, dev):
+    rng = np.random.default_rng(78)
+    A = (rng.integers(-8, 9, (32, 32)) * 0.25).astype(np.float32)
+    B = (rng.integers(-8, 9, (32, 32)) * 0.5).astype(np.float32)
+    C = rng.integers(-100, 100, (32, 32)).astype(np.float32)
+    exact = (A.astype(np.float64) @ B.astype(np.float64) + C).astype(np.float32)
+    for rounding in (0, 1, 2):
+        assert np.array_equal(_run(tc, dev, 0, 3, 0, 1, A, B, C, 0, 1, 1, 1, rounding), exact)
+    # nothing is rounded away on the way in: B = I returns A bit for bit, including values
+    # that no 16-bit split represents
+    A = (rng.uniform(-1, 1, (32, 32)) * np.exp2(rng.integers(-60, 60, (32, 32)))).astype(np.float32)
+    D = _run(tc, dev, 0, 3, 0, 1, A, np.eye(32, dtype=np.float32), None, 0, 0, 0, 0, 0)
+    assert np.array_equal(D, A)
+
+
+def test_fp32_policy_matvec(tc, orc, dev):
+    rng = np.random.default_rng(10)
+    for a_col, left in itertools.product((0, 1), (0, 1)):
+        A = rng.uniform(-1, 1, (32, 32)).astype(np.float32)
+        x = rng.uniform(-1, 1, 32).astype(np.float32)
+        y = tc.matvec(3, 0, torch.from_numpy(_mem(A, a_col)).to(dev),
+                      torch.from_numpy(x).to(dev), a_col, left).cpu().numpy()
+        ref = (x.astype(np.float64) @ A.astype(np.float64)) if left else \
+            (A.astype(np.float64) @ x.astype(np.float64))
+        assert np.abs(y - ref).max() < TH_EC
+
+
+def test_fp32_policy_elementwise(tc, orc, dev):
+    """x(i), fill_fragment, neg on the fp32 fragment (no error part; integrate is a no-op)."""
+    ij = orc.frag_ij_table(2, 16, 16, 16)
+    R = ij.shape[1]
+    base = 2.5
+    for do_neg, do_int in itertools.product((0, 1), (0, 1)):
+        out = tc.elementwise(3, 0, 1, base, do_neg, do_int, dev).cpu().numpy()
+        got = out[:1024].reshape(32, 32).T
+        nelem = 4 * R
+        for lane in range(64):
+            for e in range(nelem):
+                block, reg = divmod(e, R)
+                i = ij[lane, reg, 0] + (block % 2) * 16
+                j = ij[lane, reg, 1] + (block // 2) * 16
+                main = np.float32(base + lane * 100 + e)
+                assert got[i, j] == (-main if do_neg else main)

@@ -783,9 +783,25 @@ template <class F> int with_type(const int type, F f) {
     return f(tag<w::bfloat16>{});
   case 2:
     return f(tag<w::precision::tf32>{});
+  case 3:
+    return f(tag<float>{});
   default:
     return WMMAE_STATUS_INVALID_VALUE;
   }
+}
+// Policy a harness kernel is instantiated with: the MFMA policy of the asked
+// instruction shape, or, for fp32 operands, the one op_simt policy.
+template <class T, class EC, int fm, int fn, int fk> struct harness_policy {
+  using type = tcec::Policy<tcec::op_mfma, EC, fm, fn, fk>;
+};
+template <class EC, int fm, int fn, int fk>
+struct harness_policy<float, EC, fm, fn, fk> {
+  using type = typename tcec::default_policy<float, tcec::without_ec,
+                                             tcec::op_simt>::type;
+};
+// fp32 operands exist without error correction only
+inline bool type_ec_supported(const int type, const int ec) {
+  return !(type == 3 && ec != 0);
 }
 template <class F> int with_ec(const int ec, F f) {
   if (ec)
@@ -812,6 +828,8 @@ int wmmae_tcec_mma_tile(const int shape, const int type, const int ec,
   if (shape < 0 || shape > 1 || inst < 0 || inst > 2 || rounding < 0 ||
       rounding > 2)
     return WMMAE_STATUS_INVALID_VALUE;
+  if (!type_ec_supported(type, ec))
+    return WMMAE_STATUS_NOT_SUPPORTED;
   hipStream_t s = static_cast<hipStream_t>(stream);
   return with_type(type, [&](auto tt) {
     using T = typename decltype(tt)::type;
@@ -825,7 +843,7 @@ int wmmae_tcec_mma_tile(const int shape, const int type, const int ec,
       using R = w::row_major;
       using Cm = w::col_major;
       if (inst == 0) {
-        using P = tcec::Policy<tcec::op_mfma, EC, 16, 16, 32>;
+        using P = typename harness_policy<T, EC, 16, 16, 32>::type;
         return shape == 0
                    ? go(wmmae_harness::tcec_mma_tile_kernel<32, 32, 32, T, P, R,
                                                             Cm>)
@@ -833,14 +851,14 @@ int wmmae_tcec_mma_tile(const int shape, const int type, const int ec,
                                                             Cm>);
       }
       if (inst == 1) {
-        using P = tcec::Policy<tcec::op_mfma, EC, 16, 16, 16>;
+        using P = typename harness_policy<T, EC, 16, 16, 16>::type;
         return shape == 0
                    ? go(wmmae_harness::tcec_mma_tile_kernel<32, 32, 32, T, P, R,
                                                             Cm>)
                    : go(wmmae_harness::tcec_mma_tile_kernel<16, 48, 64, T, P, R,
                                                             Cm>);
       }
-      using P = tcec::Policy<tcec::op_mfma, EC, 32, 32, 16>;
+      using P = typename harness_policy<T, EC, 32, 32, 16>::type;
       return shape == 0
                  ? go(wmmae_harness::tcec_mma_tile_kernel<32, 32, 32, T, P, R,
                                                           Cm>)
@@ -857,12 +875,14 @@ int wmmae_tcec_mma_tile_native(const int type, const int ec,
                                void *const stream) {
   if (!d || !a || !b)
     return WMMAE_STATUS_NULL_POINTER;
+  if (!type_ec_supported(type, ec))
+    return WMMAE_STATUS_NOT_SUPPORTED;
   hipStream_t s = static_cast<hipStream_t>(stream);
   return with_type(type, [&](auto tt) {
     using T = typename decltype(tt)::type;
     return with_ec(ec, [&](auto te) {
       using EC = typename decltype(te)::type;
-      using P = tcec::Policy<tcec::op_mfma, EC, 16, 16, 32>;
+      using P = typename harness_policy<T, EC, 16, 16, 32>::type;
       return with_layout(a_frag_col, [&](auto la) {
         using AL = typename decltype(la)::type;
         return with_layout(b_frag_col, [&](auto lb) {
@@ -884,12 +904,14 @@ int wmmae_tcec_matvec(const int type, const int ec, float *const y,
                       void *const stream) {
   if (!y || !a || !x)
     return WMMAE_STATUS_NULL_POINTER;
+  if (!type_ec_supported(type, ec))
+    return WMMAE_STATUS_NOT_SUPPORTED;
   hipStream_t s = static_cast<hipStream_t>(stream);
   return with_type(type, [&](auto tt) {
     using T = typename decltype(tt)::type;
     return with_ec(ec, [&](auto te) {
       using EC = typename decltype(te)::type;
-      using P = tcec::Policy<tcec::op_mfma, EC, 16, 16, 32>;
+      using P = typename harness_policy<T, EC, 16, 16, 32>::type;
       hipLaunchKernelGGL((wmmae_harness::tcec_matvec_kernel<32, T, P>), dim3(1),
                          dim3(64), 0, s, y, a, x, a_col, left_vector);
       return launch_status();
@@ -905,12 +927,17 @@ int wmmae_tcec_frag_dump(const int use, const int type, const int ec,
     return WMMAE_STATUS_NULL_POINTER;
   if (use < 0 || use > 1)
     return WMMAE_STATUS_INVALID_VALUE;
+  if (type == 3) // fp32 fragments hold no 16-bit terms
+    return WMMAE_STATUS_NOT_SUPPORTED;
   hipStream_t s = static_cast<hipStream_t>(stream);
   return with_type(type, [&](auto tt) {
     using T = typename decltype(tt)::type;
+    if constexpr (std::is_same<T, float>::value)
+      return static_cast<int>(WMMAE_STATUS_NOT_SUPPORTED);
+    else
     return with_ec(ec, [&](auto te) {
       using EC = typename decltype(te)::type;
-      using P = tcec::Policy<tcec::op_mfma, EC, 16, 16, 32>;
+      using P = typename harness_policy<T, EC, 16, 16, 32>::type;
       return with_layout(frag_col, [&](auto ll) {
         using L = typename decltype(ll)::type;
         if (use == 0)
@@ -935,6 +962,8 @@ int wmmae_tcec_elementwise(const int type, const int ec, const int inst,
     return WMMAE_STATUS_NULL_POINTER;
   if (inst < 0 || inst > 2)
     return WMMAE_STATUS_INVALID_VALUE;
+  if (!type_ec_supported(type, ec))
+    return WMMAE_STATUS_NOT_SUPPORTED;
   hipStream_t s = static_cast<hipStream_t>(stream);
   return with_type(type, [&](auto tt) {
     using T = typename decltype(tt)::type;
@@ -947,12 +976,12 @@ int wmmae_tcec_elementwise(const int type, const int ec, const int inst,
       };
       if (inst == 0)
         return go(wmmae_harness::tcec_elementwise_kernel<
-                  32, T, tcec::Policy<tcec::op_mfma, EC, 16, 16, 32>>);
+                  32, T, typename harness_policy<T, EC, 16, 16, 32>::type>);
       if (inst == 1)
         return go(wmmae_harness::tcec_elementwise_kernel<
-                  32, T, tcec::Policy<tcec::op_mfma, EC, 16, 16, 16>>);
+                  32, T, typename harness_policy<T, EC, 16, 16, 16>::type>);
       return go(wmmae_harness::tcec_elementwise_kernel<
-                32, T, tcec::Policy<tcec::op_mfma, EC, 32, 32, 16>>);
+                32, T, typename harness_policy<T, EC, 32, 32, 16>::type>);
     });
   });
 }
@@ -973,13 +1002,15 @@ int wmmae_tcec_api_gemm(const int type, const int ec, const int m, const int n,
       ldb % 4 != 0 || reinterpret_cast<uintptr_t>(A) % 16 != 0 ||
       reinterpret_cast<uintptr_t>(B) % 16 != 0)
     return WMMAE_STATUS_NOT_SUPPORTED;
+  if (!type_ec_supported(type, ec))
+    return WMMAE_STATUS_NOT_SUPPORTED;
   hipStream_t s = static_cast<hipStream_t>(stream);
   const float al = *alpha, be = *beta;
   return with_type(type, [&](auto tt) {
     using T = typename decltype(tt)::type;
     return with_ec(ec, [&](auto te) {
       using EC = typename decltype(te)::type;
-      using P = tcec::Policy<tcec::op_mfma, EC, 16, 16, 32>;
+      using P = typename harness_policy<T, EC, 16, 16, 32>::type;
       hipLaunchKernelGGL((wmmae_harness::tcec_api_gemm_kernel<T, P>),
                          dim3(m / 128, n / 128), dim3(256), 0, s, m, n, k, al,
                          A, lda, B, ldb, be, C, ldc);
