@@ -224,6 +224,21 @@ int wmmae_tcec_api_gemm(int type, int ec, int m, int n, int k,
                         const float *B, int ldb, const float *beta, float *C,
                         int ldc, void *stream);
 
+/* utils::cp_async<size> (size 4, 8 or 16 bytes per lane): 128 threads move 256
+ * elements from src to dst through LDS.  mode 0: lane-linear destinations
+ * (the reference's test), 1: scattered destinations, 2: every third thread
+ * inactive (its element comes back as zero), 3: two copies in flight released
+ * one after the other.  src must be `size`-aligned.
+ * Replaces: cp_async_test_kernel, test/utils/cp_async.cu:15-25. */
+int wmmae_utils_cp_async(int size, int mode, void *dst, const void *src,
+                         void *stream);
+
+/* out[i] = utils::cast<DST>(in[i]); dst_type 0 half, 1 bfloat16 (out: 16-bit
+ * patterns), 2 tf32, 3 float (out: fp32).
+ * Replaces: test/utils/cast.cu. */
+int wmmae_utils_cast(int dst_type, const float *in, void *out, long long n,
+                     void *stream);
+
 /* One raw MFMA D = A*B + C on 16-bit patterns (type 0 half, 1 bfloat16);
  * (m,n,k) one of (16,16,16), (16,16,32), (32,32,8), (32,32,16); a: m x k,
  * b: k x n, c/d: m x n, all row-major.

@@ -1,0 +1,56 @@
+"""utils::cp_async and utils::cast on the GPU (reference: test/utils/cp_async.cu,
+test/utils/cast.cu), through the C-ABI harness entries."""
+import numpy as np
+import pytest
+import torch
+
+pytestmark = pytest.mark.gpu
+
+
+@pytest.mark.parametrize("size", [4, 8, 16])
+@pytest.mark.parametrize("mode", [0, 1, 2, 3])
+def test_cp_async_copies_every_byte(tc, dev, size, mode):
+    """The reference's check: input word i holds float(i); the copy through LDS returns
+    it unchanged (error = 0), for lane-linear, scattered, partially masked and pipelined use."""
+    words = 256 * size // 4
+    src = torch.arange(words, dtype=torch.float32, device=dev)
+    got = tc.utils_cp_async(size, mode, src).cpu().numpy()
+    expect = np.arange(words, dtype=np.float32)
+    if mode == 2:
+        elem = (np.arange(words) // (size // 4)) % 128
+        expect = np.where(elem % 3 != 0, expect, 0.0).astype(np.float32)
+    assert np.array_equal(got, expect)
+
+
+def test_cp_async_argument_checks(tc, dev):
+    from wmma_extension_amd._lib import WmmaeError
+    src = torch.zeros(1024, dtype=torch.float32, device=dev)
+    with pytest.raises(WmmaeError) as e:
+        tc.utils_cp_async(12, 0, src)
+    assert e.value.status == -1
+    with pytest.raises(WmmaeError) as e:
+        tc.utils_cp_async(16, 0, src[1:])
+    assert e.value.status == -7
+
+
+def test_cast_matches_oracle_conversions(tc, orc, dev):
+    rng = np.random.default_rng(5)
+    bits = rng.integers(0, 2**32, size=1 << 20, dtype=np.uint64).astype(np.uint32)
+    v = bits.view(np.float32)
+    v = v[np.isfinite(v)]
+    special = np.array([0.0, -0.0, 1.0, 65504.0, 65520.0, 2.0**-24, 2.0**-25, 1.0 + 2.0**-11,
+                        1.0 + 3 * 2.0**-11, 3.0e38], dtype=np.float32)
+    v = np.concatenate([v, special])
+    x = torch.from_numpy(v).to(dev)
+    h = tc.utils_cast(0, x).cpu().numpy().view(np.uint16)
+    assert np.array_equal(h, orc.split(orc.SPLIT_F16, v)[0])
+    b = tc.utils_cast(1, x).cpu().numpy().view(np.uint16)
+    assert np.array_equal(b, orc.split(orc.SPLIT_BF16X2, v)[0])
+    # tf32: round to nearest even at 10 mantissa bits, kept in an fp32 container
+    t = tc.utils_cast(2, x).cpu().numpy()
+    u = v.view(np.uint32).astype(np.uint64)
+    r = ((u + 0xFFF + ((u >> 13) & 1)) & ~np.uint64(0x1FFF)).astype(np.uint32).view(np.float32)
+    ok = np.isfinite(r)
+    assert np.array_equal(t[ok], r[ok]) and (t.view(np.uint32) & 0x1FFF == 0).all()
+    f = tc.utils_cast(3, x).cpu().numpy()
+    assert np.array_equal(f.view(np.uint32), v.view(np.uint32))

@@ -44,6 +44,8 @@ EXPORTS = [
     "wmmae_tcec_frag_dump",
     "wmmae_tcec_elementwise",
     "wmmae_tcec_api_gemm",
+    "wmmae_utils_cp_async",
+    "wmmae_utils_cast",
     "wmmae_mfma_probe",
 ]
 
@@ -92,6 +94,8 @@ _SIGNATURES = {
     "wmmae_tcec_frag_dump": (_i, [_i, _i, _i, _i, _vp, _vp, _i, _i, _vp]),
     "wmmae_tcec_elementwise": (_i, [_i, _i, _i, _vp, _c.c_float, _i, _i, _vp]),
     "wmmae_tcec_api_gemm": (_i, [_i, _i, _i, _i, _i, _fp, _vp, _i, _vp, _i, _fp, _vp, _i, _vp]),
+    "wmmae_utils_cp_async": (_i, [_i, _i, _vp, _vp, _vp]),
+    "wmmae_utils_cast": (_i, [_i, _vp, _vp, _ll, _vp]),
     "wmmae_mfma_probe": (_i, [_i, _i, _i, _i, _vp, _vp, _vp, _vp, _vp]),
 }
 

@@ -1019,6 +1019,48 @@ int wmmae_tcec_api_gemm(const int type, const int ec, const int m, const int n,
   });
 }
 
+int wmmae_utils_cp_async(const int size, const int mode, void *const dst,
+                         const void *const src, void *const stream) {
+  if (!dst || !src)
+    return WMMAE_STATUS_NULL_POINTER;
+  if (mode < 0 || mode > 3 || (size != 4 && size != 8 && size != 16))
+    return WMMAE_STATUS_INVALID_VALUE;
+  if (reinterpret_cast<uintptr_t>(src) % size != 0 ||
+      reinterpret_cast<uintptr_t>(dst) % 4 != 0)
+    return WMMAE_STATUS_MISALIGNED;
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  uint32_t *const d = static_cast<uint32_t *>(dst);
+  const uint32_t *const g = static_cast<const uint32_t *>(src);
+  if (size == 4)
+    hipLaunchKernelGGL(wmmae_harness::cp_async_kernel<4>, dim3(1), dim3(128), 0,
+                       s, d, g, mode);
+  else if (size == 8)
+    hipLaunchKernelGGL(wmmae_harness::cp_async_kernel<8>, dim3(1), dim3(128), 0,
+                       s, d, g, mode);
+  else
+    hipLaunchKernelGGL(wmmae_harness::cp_async_kernel<16>, dim3(1), dim3(128),
+                       0, s, d, g, mode);
+  return launch_status();
+}
+
+int wmmae_utils_cast(const int dst_type, const float *const in, void *const out,
+                     const long long n, void *const stream) {
+  if (!in || !out)
+    return WMMAE_STATUS_NULL_POINTER;
+  if (n < 0 || n > (1ll << 38))
+    return WMMAE_STATUS_INVALID_VALUE;
+  if (n == 0)
+    return WMMAE_STATUS_SUCCESS;
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  const dim3 grid(static_cast<unsigned>(ceil_div(n, 256)));
+  return with_type(dst_type, [&](auto tt) {
+    using T = typename decltype(tt)::type;
+    hipLaunchKernelGGL(wmmae_harness::cast_kernel<T>, grid, dim3(256), 0, s, in,
+                       out, n);
+    return launch_status();
+  });
+}
+
 int wmmae_mfma_probe(const int type, const int m, const int n, const int k,
                      float *const d, const unsigned short *const a,
                      const unsigned short *const b, const float *const c,

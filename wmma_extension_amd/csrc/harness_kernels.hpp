@@ -22,8 +22,12 @@
 //   tcec_api_gemm_kernel    : a tiled GEMM written against the public tcec:: API only
 //                             (reference: test/tcec/batch_gemm.cu:196-386)
 //   mfma_probe_kernel       : one raw MFMA on caller-supplied bit patterns
+//   cp_async_kernel         : utils::cp_async global -> LDS copies
+//                             (reference: test/utils/cp_async.cu:15-25)
+//   cast_kernel             : utils::cast (reference: test/utils/cast.cu)
 #pragma once
 #include <wmma_extension/tcec/tcec.hpp>
+#include <wmma_extension/utils.hpp>
 #include <wmma_extension/wmma_mma.hpp>
 
 namespace wmmae_harness {
@@ -431,6 +435,83 @@ __global__ void __launch_bounds__(64)
   w::load_matrix_sync(fc, c, N, w::mem_row_major);
   w::mma_sync(fc, fa, fb, fc);
   w::store_matrix_sync(d, fc, N, w::mem_row_major);
+}
+
+// --------------------------------------------------------------------------
+// utils::cp_async: 128 threads move 256 elements of Size bytes through LDS.
+//   mode 0: dst[t] <- smem[t] <- src[t] (the reference's test; lane-linear
+//           destinations, served by the direct global->LDS load), both halves
+//   mode 1: scattered destinations smem[(37 t + 5) % 128] (register path)
+//   mode 2: only threads with t % 3 != 0 copy; the others' slots are zeroed
+//           first (direct load under a partial execution mask)
+//   mode 3: two groups in flight, wait_pending<1> releases the first
+// --------------------------------------------------------------------------
+template <unsigned Size>
+__global__ void __launch_bounds__(128)
+    cp_async_kernel(uint32_t *const dst, const uint32_t *const src,
+                    const int mode) {
+  namespace cpa = w::utils::cp_async;
+  constexpr unsigned W = Size / 4; // words per element
+  __shared__ __attribute__((aligned(16))) uint32_t smem[2][128 * W];
+  const unsigned t = threadIdx.x;
+  auto out = [&](const unsigned elem, const uint32_t *const from) {
+    for (unsigned i = 0; i < W; i++)
+      dst[elem * W + i] = from[i];
+  };
+  if (mode == 0) {
+    cpa::cp_async<Size>(&smem[0][t * W], src + t * W);
+    cpa::cp_async<Size>(&smem[1][t * W], src + (128 + t) * W);
+    cpa::commit();
+    cpa::wait_all();
+    out(t, &smem[0][t * W]);
+    out(128 + t, &smem[1][t * W]);
+  } else if (mode == 1) {
+    const unsigned p = (37 * t + 5) % 128;
+    cpa::cp_async<Size>(&smem[0][p * W], src + t * W);
+    cpa::cp_async<Size>(&smem[1][p * W], src + (128 + t) * W);
+    cpa::commit();
+    cpa::wait_group<0>();
+    out(t, &smem[0][p * W]);
+    out(128 + t, &smem[1][p * W]);
+  } else if (mode == 2) {
+    for (unsigned i = 0; i < W; i++)
+      smem[0][t * W + i] = smem[1][t * W + i] = 0u;
+    __syncthreads();
+    if (t % 3 != 0) {
+      cpa::cp_async<Size>(&smem[0][t * W], src + t * W);
+      cpa::cp_async<Size>(&smem[1][t * W], src + (128 + t) * W);
+    }
+    cpa::commit();
+    cpa::wait_all();
+    out(t, &smem[0][t * W]);
+    out(128 + t, &smem[1][t * W]);
+  } else {
+    cpa::cp_async<Size>(&smem[0][t * W], src + t * W);
+    cpa::commit();
+    cpa::cp_async<Size>(&smem[1][t * W], src + (128 + t) * W);
+    cpa::commit();
+    cpa::wait_pending<1>(); // the first copy has landed, the second may fly
+    out(t, &smem[0][t * W]);
+    cpa::wait_all();
+    out(128 + t, &smem[1][t * W]);
+  }
+}
+
+// utils::cast<DST>(in[i]) for DST = half, bfloat16 (16-bit patterns out),
+// precision::tf32 and float (fp32 out).
+template <class DST>
+__global__ void __launch_bounds__(256)
+    cast_kernel(const float *const in, void *const out, const long long n) {
+  const long long i =
+      static_cast<long long>(blockIdx.x) * blockDim.x + threadIdx.x;
+  if (i >= n)
+    return;
+  const auto v = w::utils::cast<DST>(in[i]);
+  if constexpr (sizeof(v) == 2)
+    static_cast<unsigned short *>(out)[i] =
+        __builtin_bit_cast(unsigned short, v);
+  else
+    static_cast<float *>(out)[i] = v;
 }
 
 } // namespace wmmae_harness

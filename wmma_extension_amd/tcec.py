@@ -239,3 +239,21 @@ def mfma_probe(type_, m, n, k, a_bits, b_bits, c):
                                      _stream())
     _lib.check(st, "wmmae_mfma_probe")
     return d
+
+
+def utils_cp_async(size, mode, src):
+    """src: 256 elements of `size` bytes (any dtype, CUDA); returns the copy made through LDS."""
+    _need_cuda(src)
+    dst = torch.full_like(src, -1)
+    st = _lib.lib().wmmae_utils_cp_async(size, mode, _ptr(dst), _ptr(src), _stream())
+    _lib.check(st, "wmmae_utils_cp_async")
+    return dst
+
+
+def utils_cast(dst_type, x):
+    """x: fp32 CUDA tensor -> int16 bit patterns (dst_type 0 half, 1 bfloat16) or fp32 (2 tf32, 3 float)."""
+    _need_cuda(x)
+    out = torch.empty(x.shape, dtype=torch.int16 if dst_type in (0, 1) else torch.float32, device=x.device)
+    st = _lib.lib().wmmae_utils_cast(dst_type, _ptr(x), _ptr(out), x.numel(), _stream())
+    _lib.check(st, "wmmae_utils_cast")
+    return out
