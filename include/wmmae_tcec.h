@@ -224,6 +224,18 @@ int wmmae_tcec_api_gemm(int type, int ec, int m, int n, int k,
                         const float *B, int ldb, const float *beta, float *C,
                         int ldc, void *stream);
 
+/* One-wave complex TCEC product D = A*B (+C), m = n = k = 32, operands in
+ * tcec::fragment_complex (16x16x32 policy; 16x16x16 for type 3).  a, b, c, d:
+ * 32 x 32 interleaved (re, im) fp32 pairs, dense; *_col: memory layouts;
+ * c may be NULL; rounding as in wmmae_tcec_mma_tile.  mul != 1 (a power of
+ * two) routes A through load_matrix_sync_with_mul and D through the scaled
+ * store with 1/mul.
+ * Replaces: mma_kernel_abcd / mma_kernel_abd, test/tcec/mma_complex.cu:22-101. */
+int wmmae_tcec_mma_complex(int type, int ec, float *d, const float *a,
+                           const float *b, const float *c, int a_col, int b_col,
+                           int c_col, int d_col, int rounding, float mul,
+                           void *stream);
+
 /* utils::cp_async<size> (size 4, 8 or 16 bytes per lane): 128 threads move 256
  * elements from src to dst through LDS.  mode 0: lane-linear destinations
  * (the reference's test), 1: scattered destinations, 2: every third thread

@@ -44,6 +44,7 @@ EXPORTS = [
     "wmmae_tcec_frag_dump",
     "wmmae_tcec_elementwise",
     "wmmae_tcec_api_gemm",
+    "wmmae_tcec_mma_complex",
     "wmmae_utils_cp_async",
     "wmmae_utils_cast",
     "wmmae_mfma_probe",
@@ -94,6 +95,7 @@ _SIGNATURES = {
     "wmmae_tcec_frag_dump": (_i, [_i, _i, _i, _i, _vp, _vp, _i, _i, _vp]),
     "wmmae_tcec_elementwise": (_i, [_i, _i, _i, _vp, _c.c_float, _i, _i, _vp]),
     "wmmae_tcec_api_gemm": (_i, [_i, _i, _i, _i, _i, _fp, _vp, _i, _vp, _i, _fp, _vp, _i, _vp]),
+    "wmmae_tcec_mma_complex": (_i, [_i, _i, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _c.c_float, _vp]),
     "wmmae_utils_cp_async": (_i, [_i, _i, _vp, _vp, _vp]),
     "wmmae_utils_cast": (_i, [_i, _vp, _vp, _ll, _vp]),
     "wmmae_mfma_probe": (_i, [_i, _i, _i, _i, _vp, _vp, _vp, _vp, _vp]),

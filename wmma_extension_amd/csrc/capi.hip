@@ -1019,6 +1019,37 @@ int wmmae_tcec_api_gemm(const int type, const int ec, const int m, const int n,
   });
 }
 
+int wmmae_tcec_mma_complex(const int type, const int ec, float *const d,
+                           const float *const a, const float *const b,
+                           const float *const c, const int a_col,
+                           const int b_col, const int c_col, const int d_col,
+                           const int rounding, const float mul,
+                           void *const stream) {
+  if (!d || !a || !b)
+    return WMMAE_STATUS_NULL_POINTER;
+  if (rounding < 0 || rounding > 2 || mul == 0.f)
+    return WMMAE_STATUS_INVALID_VALUE;
+  if (!type_ec_supported(type, ec))
+    return WMMAE_STATUS_NOT_SUPPORTED;
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  using cplx = tcec::complex_t;
+  return with_type(type, [&](auto tt) {
+    using T = typename decltype(tt)::type;
+    return with_ec(ec, [&](auto te) {
+      using EC = typename decltype(te)::type;
+      using P = typename harness_policy<T, EC, 16, 16, 32>::type;
+      hipLaunchKernelGGL(
+          (wmmae_harness::tcec_mma_complex_kernel<32, T, P, w::row_major,
+                                                  w::col_major>),
+          dim3(1), dim3(64), 0, s, reinterpret_cast<cplx *>(d),
+          reinterpret_cast<const cplx *>(a), reinterpret_cast<const cplx *>(b),
+          reinterpret_cast<const cplx *>(c), a_col, b_col, c_col, d_col,
+          rounding, mul);
+      return launch_status();
+    });
+  });
+}
+
 int wmmae_utils_cp_async(const int size, const int mode, void *const dst,
                          const void *const src, void *const stream) {
   if (!dst || !src)

@@ -22,10 +22,13 @@
 //   tcec_api_gemm_kernel    : a tiled GEMM written against the public tcec:: API only
 //                             (reference: test/tcec/batch_gemm.cu:196-386)
 //   mfma_probe_kernel       : one raw MFMA on caller-supplied bit patterns
+//   tcec_mma_complex_kernel : one-wave complex D = A*B (+C) through fragment_complex
+//                             (reference: test/tcec/mma_complex.cu:22-101)
 //   cp_async_kernel         : utils::cp_async global -> LDS copies
 //                             (reference: test/utils/cp_async.cu:15-25)
 //   cast_kernel             : utils::cast (reference: test/utils/cast.cu)
 #pragma once
+#include <wmma_extension/tcec/complex.hpp>
 #include <wmma_extension/tcec/tcec.hpp>
 #include <wmma_extension/utils.hpp>
 #include <wmma_extension/wmma_mma.hpp>
@@ -435,6 +438,62 @@ __global__ void __launch_bounds__(64)
   w::load_matrix_sync(fc, c, N, w::mem_row_major);
   w::mma_sync(fc, fa, fb, fc);
   w::store_matrix_sync(d, fc, N, w::mem_row_major);
+}
+
+// --------------------------------------------------------------------------
+// One-wave complex product D = A*B (+C), N x N x N, every operand in one
+// tcec::fragment_complex; memory holds interleaved (re, im) pairs with dense
+// leading dimension N.  mul != 1 exercises the scaled load of A and the scaled
+// store (D = (mul*A)*B*(1/mul) + ..., exact for powers of two).
+// --------------------------------------------------------------------------
+template <int N, class T, class Policy, class AL, class BL>
+__global__ void __launch_bounds__(64)
+    tcec_mma_complex_kernel(tcec::complex_t *const d,
+                            const tcec::complex_t *const a,
+                            const tcec::complex_t *const b,
+                            const tcec::complex_t *const c, const int a_col,
+                            const int b_col, const int c_col, const int d_col,
+                            const int rounding, const float mul) {
+  tcec::fragment_complex<w::matrix_a, N, N, N, T, AL, Policy> fa;
+  tcec::fragment_complex<w::matrix_b, N, N, N, T, BL, Policy> fb;
+  tcec::fragment_complex<w::accumulator, N, N, N, T, void, Policy> fc, fd;
+  if (a_col)
+    tcec::load_matrix_sync_with_mul<w::col_major>(fa, a, N, mul);
+  else
+    tcec::load_matrix_sync_with_mul<w::row_major>(fa, a, N, mul);
+  if (b_col)
+    tcec::load_matrix_sync<w::col_major>(fb, b, N);
+  else
+    tcec::load_matrix_sync<w::row_major>(fb, b, N);
+  tcec::fill_fragment(fd, 0.0f);
+  if (c != nullptr) {
+    tcec::load_matrix_sync(fc, c, N, c_col ? w::mem_col_major : w::mem_row_major);
+    if (mul != 1.f) { // keep D = A*B + C after the scaled store
+      for (unsigned i = 0; i < fc.real.num_elements; i++) {
+        fc.real.x(i) *= mul;
+        fc.imag.x(i) *= mul;
+      }
+    }
+    if (rounding == 1)
+      tcec::mma_rn_sync(fd, fa, fb, fc);
+    else if (rounding == 2)
+      tcec::mma_rz_sync(fd, fa, fb, fc);
+    else
+      tcec::mma_sync(fd, fa, fb, fc);
+  } else {
+    if (rounding == 1)
+      tcec::mma_rn_sync(fd, fa, fb);
+    else if (rounding == 2)
+      tcec::mma_rz_sync(fd, fa, fb);
+    else
+      tcec::mma_sync(fd, fa, fb);
+  }
+  const w::layout_t dl = d_col ? w::mem_col_major : w::mem_row_major;
+  if (mul != 1.f)
+    tcec::store_matrix_sync(d, fd, N, 1.f / mul, dl);
+  else
+    tcec::store_matrix_sync(d, fd, N, dl);
+  tcec::fill_zero(fd);
 }
 
 // --------------------------------------------------------------------------

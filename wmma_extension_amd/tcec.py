@@ -257,3 +257,13 @@ def utils_cast(dst_type, x):
     st = _lib.lib().wmmae_utils_cast(dst_type, _ptr(x), _ptr(out), x.numel(), _stream())
     _lib.check(st, "wmmae_utils_cast")
     return out
+
+
+def mma_complex(type_, ec, a, b, c, a_col, b_col, c_col, d_col, rounding=0, mul=1.0):
+    """a, b, c: (32*32*2,) fp32 CUDA tensors of interleaved (re, im) pairs; returns d likewise."""
+    _need_cuda(a, b, c)
+    d = torch.full_like(a, float("nan"))
+    st = _lib.lib().wmmae_tcec_mma_complex(type_, ec, _ptr(d), _ptr(a), _ptr(b), _ptr(c), a_col, b_col,
+                                           c_col, d_col, rounding, float(mul), _stream())
+    _lib.check(st, "wmmae_tcec_mma_complex")
+    return d
