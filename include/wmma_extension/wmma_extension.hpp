@@ -287,5 +287,107 @@ print_fragment(const fragment<Use, M, N, K, T, Layout> &frag,
   }
 }
 
+// ------------------------------------------------------- identity matrices
+// frag += a * I (reference: wmma_extension.hpp:233-248; per-architecture
+// register lists in detail/sm_80.hpp:404-415).  Here the diagonal is found
+// through the layout model: the lane that owns (i, i) adds a.
+template <int M, int N, int K, class T, class FT>
+WMMAE_D void add_eye(fragment<accumulator, M, N, K, T> &frag, const FT a) {
+  detail::foreach_ij_core<fragment<accumulator, M, N, K, T>>(
+      [&](const unsigned *list, const unsigned, const unsigned i,
+          const unsigned j) {
+        if (i == j)
+          frag.x[list[0]] += detail::common::cast<T>(a);
+      });
+}
+template <int M, int N, int K, class T>
+WMMAE_D void make_identity_matrix(fragment<accumulator, M, N, K, T> &frag) {
+  fill_zero(frag);
+  add_eye(frag, detail::common::cast<T>(1.0f));
+}
+
+// -------------------------------------------------- direct (outer) products
+// Operand fragments whose single MMA gives the error-corrected outer product
+// u v^T of two fp32 vectors held as x = leading 16-bit part, dx = residual
+// (reference: wmma_extension.hpp:250-284, detail/sm_80.hpp:417-525,
+// docs/make_direct_product_fragments-en.svg):
+//   matrix_a: columns 0..3 = x, dx, x, dx      (column 3 only with 3 terms)
+//   matrix_b: rows    0..3 = x, x, dx, dx      (row 3 only with 3 terms)
+// so that A*B = x_a x_b^T + dx_a x_b^T + x_a dx_b^T (+ dx_a dx_b^T).  All other
+// elements are zeroed when `fill` is set and left alone otherwise.
+namespace detail {
+template <unsigned CORRECTION_TERMS, class Use, int M, int N, int K, class FT,
+          class Layout, class GetX, class GetDx>
+WMMAE_D void direct_product_core(fragment<Use, M, N, K, FT, Layout> &frag,
+                                 const bool fill, GetX x_of, GetDx dx_of) {
+  static_assert(!std::is_same<Use, accumulator>::value,
+                "direct products are operand fragments");
+  static_assert(K >= 4, "four k positions are used");
+  static_assert(CORRECTION_TERMS == 2 || CORRECTION_TERMS == 3,
+                "2 or 3 correction terms");
+  if (fill)
+    fill_zero(frag);
+  constexpr bool is_a = std::is_same<Use, matrix_a>::value;
+  foreach_ij_core<fragment<Use, M, N, K, FT, Layout>>(
+      [&](const unsigned *list, const unsigned, const unsigned i,
+          const unsigned j) {
+        const unsigned kk = is_a ? j : i; // position along k
+        const unsigned e = is_a ? i : j;  // vector element
+        if (kk >= 4 || (kk == 3 && CORRECTION_TERMS != 3))
+          return;
+        // matrix_a: x, dx, x, dx   matrix_b: x, x, dx, dx
+        const bool residual = is_a ? (kk & 1u) != 0 : kk >= 2;
+        frag.x[list[0]] = residual ? dx_of(e) : x_of(e);
+      });
+}
+} // namespace detail
+
+template <class MatrixType, int M, int N, int K, class MemMajor, class T,
+          class S, class FT>
+WMMAE_D void
+make_direct_product_fragment(fragment<MatrixType, M, N, K, FT, MemMajor> &frag_x,
+                             const T *const x, const S *const dx,
+                             const bool fill = true) {
+  detail::direct_product_core<2>(
+      frag_x, fill,
+      [&](const unsigned e) { return detail::common::cast<FT>(x[e]); },
+      [&](const unsigned e) { return detail::common::cast<FT>(dx[e]); });
+}
+template <class MatrixType, int M, int N, int K, class MemMajor, class T,
+          class S, class FT>
+WMMAE_D void make_direct_product_fragment_c3(
+    fragment<MatrixType, M, N, K, FT, MemMajor> &frag_x, const T *const x,
+    const S *const dx, const bool fill = true) {
+  detail::direct_product_core<3>(
+      frag_x, fill,
+      [&](const unsigned e) { return detail::common::cast<FT>(x[e]); },
+      [&](const unsigned e) { return detail::common::cast<FT>(dx[e]); });
+}
+// From the fp32 vector itself: dx = x - float(cast(x)), computed on the fly.
+template <class MatrixType, int M, int N, int K, class MemMajor, class FT>
+WMMAE_D void
+make_direct_product_fragment(fragment<MatrixType, M, N, K, FT, MemMajor> &frag_x,
+                             const float *const x, const bool fill = true) {
+  detail::direct_product_core<2>(
+      frag_x, fill,
+      [&](const unsigned e) { return detail::common::cast<FT>(x[e]); },
+      [&](const unsigned e) {
+        return detail::common::cast<FT>(
+            x[e] - static_cast<float>(detail::common::cast<FT>(x[e])));
+      });
+}
+template <class MatrixType, int M, int N, int K, class MemMajor, class FT>
+WMMAE_D void make_direct_product_fragment_c3(
+    fragment<MatrixType, M, N, K, FT, MemMajor> &frag_x, const float *const x,
+    const bool fill = true) {
+  detail::direct_product_core<3>(
+      frag_x, fill,
+      [&](const unsigned e) { return detail::common::cast<FT>(x[e]); },
+      [&](const unsigned e) {
+        return detail::common::cast<FT>(
+            x[e] - static_cast<float>(detail::common::cast<FT>(x[e])));
+      });
+}
+
 } // namespace wmma
 } // namespace mtk

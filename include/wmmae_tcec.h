@@ -236,6 +236,29 @@ int wmmae_tcec_mma_complex(int type, int ec, float *d, const float *a,
                            int c_col, int d_col, int rounding, float mul,
                            void *stream);
 
+/* Elementwise operators on 16x16x16 fragments: a, b are 16x16 row-major fp32
+ * tiles cast to the element type on the way in, out is the result fragment
+ * cast back.  op: 0 a+b, 1 a-b, 2 a*alpha, 3 a/alpha, 4 fma(alpha,a,b),
+ * 5 fma(a,alpha,b); use: 0 matrix_a, 1 matrix_b, 2 accumulator (elem 2 only);
+ * elem: 0 half, 1 bfloat16, 2 float.
+ * Replaces: test/primitive/operators.cu:14-57. */
+int wmmae_fragment_ops(int op, int use, int elem, float alpha, const float *a,
+                       const float *b, float *out, void *stream);
+
+/* An fp32 accumulator (shape 0: 16x16x16, 1: 32x32x8) filled with 1 plus
+ * add_eye(alpha) (identity == 0) or make_identity_matrix (identity != 0),
+ * stored column-major into out.
+ * Replaces: make_eye_kernel, test/primitive/add_eye.cu:24-30. */
+int wmmae_fragment_eye(int shape, int identity, float alpha, float *out,
+                       void *stream);
+
+/* h (16x16 column-major) = u v^T by one MMA on make_direct_product_fragment
+ * (terms 2) / _c3 (terms 3) operands; elem 0 half, 1 bfloat16; from_float != 0
+ * uses the fp32-vector overloads, else the (x, dx) ones.
+ * Replaces: direct_product_kernel, test/primitive/direct_product.cu:44-99. */
+int wmmae_direct_product(int elem, int terms, int from_float, const float *u,
+                         const float *v, float *h, void *stream);
+
 /* utils::cp_async<size> (size 4, 8 or 16 bytes per lane): 128 threads move 256
  * elements from src to dst through LDS.  mode 0: lane-linear destinations
  * (the reference's test), 1: scattered destinations, 2: every third thread

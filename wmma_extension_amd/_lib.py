@@ -45,6 +45,9 @@ EXPORTS = [
     "wmmae_tcec_elementwise",
     "wmmae_tcec_api_gemm",
     "wmmae_tcec_mma_complex",
+    "wmmae_fragment_ops",
+    "wmmae_fragment_eye",
+    "wmmae_direct_product",
     "wmmae_utils_cp_async",
     "wmmae_utils_cast",
     "wmmae_mfma_probe",
@@ -96,6 +99,9 @@ _SIGNATURES = {
     "wmmae_tcec_elementwise": (_i, [_i, _i, _i, _vp, _c.c_float, _i, _i, _vp]),
     "wmmae_tcec_api_gemm": (_i, [_i, _i, _i, _i, _i, _fp, _vp, _i, _vp, _i, _fp, _vp, _i, _vp]),
     "wmmae_tcec_mma_complex": (_i, [_i, _i, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _c.c_float, _vp]),
+    "wmmae_fragment_ops": (_i, [_i, _i, _i, _c.c_float, _vp, _vp, _vp, _vp]),
+    "wmmae_fragment_eye": (_i, [_i, _i, _c.c_float, _vp, _vp]),
+    "wmmae_direct_product": (_i, [_i, _i, _i, _vp, _vp, _vp, _vp]),
     "wmmae_utils_cp_async": (_i, [_i, _i, _vp, _vp, _vp]),
     "wmmae_utils_cast": (_i, [_i, _vp, _vp, _ll, _vp]),
     "wmmae_mfma_probe": (_i, [_i, _i, _i, _i, _vp, _vp, _vp, _vp, _vp]),

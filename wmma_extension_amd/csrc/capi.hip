@@ -1050,6 +1050,73 @@ int wmmae_tcec_mma_complex(const int type, const int ec, float *const d,
   });
 }
 
+int wmmae_fragment_ops(const int op, const int use, const int elem,
+                       const float alpha, const float *const a,
+                       const float *const b, float *const out,
+                       void *const stream) {
+  if (!a || !b || !out)
+    return WMMAE_STATUS_NULL_POINTER;
+  if (op < 0 || op > 5 || use < 0 || use > 2 || elem < 0 || elem > 2)
+    return WMMAE_STATUS_INVALID_VALUE;
+  if (use == 2 && elem != 2) // accumulators are fp32 on the matrix core
+    return WMMAE_STATUS_NOT_SUPPORTED;
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  auto go = [&](auto kernel) {
+    hipLaunchKernelGGL(kernel, dim3(1), dim3(64), 0, s, out, a, b, alpha, op);
+    return launch_status();
+  };
+  using R = w::row_major;
+  if (use == 2)
+    return go(wmmae_harness::fragment_ops_kernel<w::accumulator, float, void>);
+  if (use == 0) {
+    if (elem == 0)
+      return go(wmmae_harness::fragment_ops_kernel<w::matrix_a, w::half, R>);
+    if (elem == 1)
+      return go(wmmae_harness::fragment_ops_kernel<w::matrix_a, w::bfloat16, R>);
+    return go(wmmae_harness::fragment_ops_kernel<w::matrix_a, float, R>);
+  }
+  if (elem == 0)
+    return go(wmmae_harness::fragment_ops_kernel<w::matrix_b, w::half, R>);
+  if (elem == 1)
+    return go(wmmae_harness::fragment_ops_kernel<w::matrix_b, w::bfloat16, R>);
+  return go(wmmae_harness::fragment_ops_kernel<w::matrix_b, float, R>);
+}
+
+int wmmae_fragment_eye(const int shape, const int identity, const float alpha,
+                       float *const out, void *const stream) {
+  if (!out)
+    return WMMAE_STATUS_NULL_POINTER;
+  if (shape < 0 || shape > 1)
+    return WMMAE_STATUS_INVALID_VALUE;
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  if (shape == 0)
+    hipLaunchKernelGGL((wmmae_harness::fragment_eye_kernel<16, 16, 16>),
+                       dim3(1), dim3(64), 0, s, out, alpha, identity);
+  else
+    hipLaunchKernelGGL((wmmae_harness::fragment_eye_kernel<32, 32, 8>), dim3(1),
+                       dim3(64), 0, s, out, alpha, identity);
+  return launch_status();
+}
+
+int wmmae_direct_product(const int elem, const int terms, const int from_float,
+                         const float *const u, const float *const v,
+                         float *const h, void *const stream) {
+  if (!u || !v || !h)
+    return WMMAE_STATUS_NULL_POINTER;
+  if (elem < 0 || elem > 1 || (terms != 2 && terms != 3))
+    return WMMAE_STATUS_INVALID_VALUE;
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  auto go = [&](auto kernel) {
+    hipLaunchKernelGGL(kernel, dim3(1), dim3(64), 0, s, h, u, v, from_float);
+    return launch_status();
+  };
+  if (elem == 0)
+    return terms == 2 ? go(wmmae_harness::direct_product_kernel<w::half, 2>)
+                      : go(wmmae_harness::direct_product_kernel<w::half, 3>);
+  return terms == 2 ? go(wmmae_harness::direct_product_kernel<w::bfloat16, 2>)
+                    : go(wmmae_harness::direct_product_kernel<w::bfloat16, 3>);
+}
+
 int wmmae_utils_cp_async(const int size, const int mode, void *const dst,
                          const void *const src, void *const stream) {
   if (!dst || !src)

@@ -24,10 +24,17 @@
 //   mfma_probe_kernel       : one raw MFMA on caller-supplied bit patterns
 //   tcec_mma_complex_kernel : one-wave complex D = A*B (+C) through fragment_complex
 //                             (reference: test/tcec/mma_complex.cu:22-101)
+//   fragment_ops_kernel     : operators +, -, *, /, fma on fragments
+//                             (reference: test/primitive/operators.cu:14-57)
+//   fragment_eye_kernel     : add_eye / make_identity_matrix
+//                             (reference: test/primitive/add_eye.cu:24-30)
+//   direct_product_kernel   : make_direct_product_fragment(_c3) + one MMA
+//                             (reference: test/primitive/direct_product.cu:44-99)
 //   cp_async_kernel         : utils::cp_async global -> LDS copies
 //                             (reference: test/utils/cp_async.cu:15-25)
 //   cast_kernel             : utils::cast (reference: test/utils/cast.cu)
 #pragma once
+#include <wmma_extension/operators.hpp>
 #include <wmma_extension/tcec/complex.hpp>
 #include <wmma_extension/tcec/tcec.hpp>
 #include <wmma_extension/utils.hpp>
@@ -494,6 +501,116 @@ __global__ void __launch_bounds__(64)
   else
     tcec::store_matrix_sync(d, fd, N, dl);
   tcec::fill_zero(fd);
+}
+
+// --------------------------------------------------------------------------
+// Fragment operators.  a, b: 16x16 row-major fp32 tiles, cast to T on the way
+// in; out: the result fragment written back the same way.
+//   op 0: a + b   1: a - b   2: a * alpha   3: a / alpha
+//   op 4: fma(alpha, a, b)   5: fma(a, alpha, b)
+// --------------------------------------------------------------------------
+template <class Use, class T, class Layout>
+__global__ void __launch_bounds__(64)
+    fragment_ops_kernel(float *const out, const float *const a,
+                        const float *const b, const float alpha, const int op) {
+  using F = w::fragment<Use, 16, 16, 16, T, Layout>;
+  using S = typename F::storage_element_type;
+  F fa, fb, fr;
+  w::detail::foreach_ij_core<F>([&](const unsigned *list, const unsigned,
+                                    const unsigned i, const unsigned j) {
+    fa.x[list[0]] = w::detail::common::cast<T>(a[i * 16 + j]);
+    fb.x[list[0]] = w::detail::common::cast<T>(b[i * 16 + j]);
+  });
+  const S s = w::detail::common::cast<T>(alpha);
+  switch (op) {
+  case 0:
+    fr = fa + fb;
+    break;
+  case 1:
+    fr = fa - fb;
+    break;
+  case 2:
+    fr = fa * s;
+    break;
+  case 3:
+    fr = fa / s;
+    break;
+  case 4:
+    fr = w::fma(s, fa, fb);
+    break;
+  default:
+    fr = w::fma(fa, s, fb);
+    break;
+  }
+  w::detail::foreach_ij_core<F>([&](const unsigned *list, const unsigned,
+                                    const unsigned i, const unsigned j) {
+    out[i * 16 + j] = static_cast<float>(fr.x[list[0]]);
+  });
+}
+
+// fill(1) then add_eye(alpha), or make_identity_matrix; stored column-major.
+template <int M, int N, int K>
+__global__ void __launch_bounds__(64)
+    fragment_eye_kernel(float *const out, const float alpha,
+                        const int identity) {
+  w::fragment<w::accumulator, M, N, K, float> frag;
+  if (identity) {
+    w::fill_fragment(frag, 7.0f); // must be overwritten
+    w::make_identity_matrix(frag);
+  } else {
+    w::fill_fragment(frag, 1.0f);
+    w::add_eye(frag, alpha);
+  }
+  w::store_matrix_sync(out, frag, M, w::mem_col_major);
+}
+
+// h (16x16, column-major) = u v^T through one MMA on direct-product fragments.
+// from_float == 0: the 16-bit parts x, dx are prepared in LDS first and given
+// to the (x, dx) overload; otherwise the fp32 overload splits on the fly.
+template <class T, unsigned TERMS>
+__global__ void __launch_bounds__(64)
+    direct_product_kernel(float *const h, const float *const u,
+                          const float *const v, const int from_float) {
+  using S = typename w::detail::common::storage_t<T>::type;
+  w::fragment<w::matrix_a, 16, 16, 16, T, w::col_major> fa;
+  w::fragment<w::matrix_b, 16, 16, 16, T, w::row_major> fb;
+  w::fragment<w::accumulator, 16, 16, 16, float> fc;
+  __shared__ S su[16], sdu[16], sv[16], sdv[16];
+  if (threadIdx.x < 16) {
+    const float f = u[threadIdx.x];
+    const S hv = w::detail::common::cast<T>(f);
+    su[threadIdx.x] = hv;
+    sdu[threadIdx.x] = w::detail::common::cast<T>(f - static_cast<float>(hv));
+  } else if (threadIdx.x < 32) {
+    const float f = v[threadIdx.x - 16];
+    const S hv = w::detail::common::cast<T>(f);
+    sv[threadIdx.x - 16] = hv;
+    sdv[threadIdx.x - 16] = w::detail::common::cast<T>(f - static_cast<float>(hv));
+  }
+  __syncthreads();
+  // start from junk so that `fill` is seen to work
+  w::fill_fragment(fa, w::detail::common::cast<T>(3.0f));
+  w::fill_fragment(fb, w::detail::common::cast<T>(3.0f));
+  if (from_float) {
+    if constexpr (TERMS == 3) {
+      w::make_direct_product_fragment_c3(fa, u);
+      w::make_direct_product_fragment_c3(fb, v);
+    } else {
+      w::make_direct_product_fragment(fa, u);
+      w::make_direct_product_fragment(fb, v);
+    }
+  } else {
+    if constexpr (TERMS == 3) {
+      w::make_direct_product_fragment_c3(fa, su, sdu);
+      w::make_direct_product_fragment_c3(fb, sv, sdv);
+    } else {
+      w::make_direct_product_fragment(fa, su, sdu);
+      w::make_direct_product_fragment(fb, sv, sdv);
+    }
+  }
+  w::fill_zero(fc);
+  w::mma_sync(fc, fa, fb, fc);
+  w::store_matrix_sync(h, fc, 16, w::mem_col_major);
 }
 
 // --------------------------------------------------------------------------

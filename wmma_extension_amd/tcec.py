@@ -267,3 +267,29 @@ def mma_complex(type_, ec, a, b, c, a_col, b_col, c_col, d_col, rounding=0, mul=
                                            c_col, d_col, rounding, float(mul), _stream())
     _lib.check(st, "wmmae_tcec_mma_complex")
     return d
+
+
+def fragment_ops(op, use, elem, alpha, a, b):
+    """a, b: (16,16) fp32 CUDA tensors (row-major tiles); returns the (16,16) result."""
+    _need_cuda(a, b)
+    out = torch.full((16, 16), float("nan"), dtype=torch.float32, device=a.device)
+    st = _lib.lib().wmmae_fragment_ops(op, use, elem, float(alpha), _ptr(a), _ptr(b), _ptr(out), _stream())
+    _lib.check(st, "wmmae_fragment_ops")
+    return out
+
+
+def fragment_eye(shape, identity, alpha, device):
+    n = 16 if shape == 0 else 32
+    out = torch.full((n, n), float("nan"), dtype=torch.float32, device=device)
+    st = _lib.lib().wmmae_fragment_eye(shape, identity, float(alpha), _ptr(out), _stream())
+    _lib.check(st, "wmmae_fragment_eye")
+    return out
+
+
+def direct_product(elem, terms, from_float, u, v):
+    """u, v: (16,) fp32 CUDA tensors; returns h (16,16) with h[i, j] = u[i] v[j]."""
+    _need_cuda(u, v)
+    h = torch.full((16, 16), float("nan"), dtype=torch.float32, device=u.device)
+    st = _lib.lib().wmmae_direct_product(elem, terms, from_float, _ptr(u), _ptr(v), _ptr(h), _stream())
+    _lib.check(st, "wmmae_direct_product")
+    return h.t()            # stored column-major
