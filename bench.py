@@ -59,6 +59,8 @@ def make_inputs(torch, w, dev, seed):
     shape_b = (w["batch"], w["n"], w["k"])
 
     def draw(shape):
+        if w["dist"] == "zeros":
+            return torch.zeros(shape, device=dev, dtype=torch.float32)
         if w["dist"] == "uniform":
             return torch.rand(shape, generator=g, device=dev, dtype=torch.float32) * 2 - 1
         if w["dist"] == "normal":
@@ -216,6 +218,12 @@ def main():
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--no-accuracy", action="store_true")
     ap.add_argument("--flags", type=int, default=0)
+    ap.add_argument("--dist", default=None, choices=["uniform", "normal", "exp", "zeros"],
+                    help="override the workload's input distribution (zeros: what the kernel reaches "
+                         "when the matrix cores are not power limited; not a valid benchmark value)")
+    ap.add_argument("--clock-trace", action="store_true",
+                    help="sample the shader clock on a second stream during the timed region and add "
+                         "its statistics to the JSON line (the matrix cores are power limited)")
     ap.add_argument("--calibrate", action="store_true",
                     help="after the timed region run one 1 GiB read + 1 GiB write elementwise kernel "
                          "(the known-size copy that rocprofv3 FETCH_SIZE / WRITE_SIZE are scaled with)")
@@ -230,7 +238,9 @@ def main():
     _lib.lib()
     dev = torch.device("cuda:0")
     torch.cuda.set_device(dev)
-    w = WORKLOADS[args.workload]
+    w = dict(WORKLOADS[args.workload])
+    if args.dist is not None:
+        w["dist"] = args.dist
     if w.get("kind") == "prim":
         return bench_primitives(args, torch, tcec, dev, w)
     policy = tcec.Policy[w["policy"]]
@@ -268,12 +278,31 @@ def main():
     torch.cuda.synchronize()
     events = [(torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True))
               for _ in range(args.steps)]
-    torch.cuda.synchronize()
+    trace = None
+    if args.clock_trace:
+        # one more untimed step gives the length of the region to cover
+        t0 = time.perf_counter()
+        step()
+        torch.cuda.synchronize()
+        est_ms = (time.perf_counter() - t0) * 1e3 * args.steps
+        period = 10_000                                   # 100 us of the 100 MHz counter
+        nsamples = int(min(50_000, (est_ms * 1.5 + 30.0) / 0.1))
+        side = torch.cuda.Stream()
+        trace = tcec.clock_samples(nsamples, period, side)
+        time.sleep(0.005)                                 # a few idle samples first
+        mark0 = tcec.clock_samples(1, 0)                  # GPU time stamps of the region, main stream
+    if trace is None:
+        torch.cuda.synchronize()
     t0 = time.perf_counter()
     for i in range(args.steps):
         step(events[i])
-    torch.cuda.synchronize()
+    if trace is not None:
+        mark1 = tcec.clock_samples(1, 0)
+        torch.cuda.current_stream().synchronize()      # the sampler may run on for a while
+    else:
+        torch.cuda.synchronize()
     elapsed = time.perf_counter() - t0
+    torch.cuda.synchronize()
 
     if args.calibrate:
         calibration_copy(torch, dev)
@@ -324,6 +353,23 @@ def main():
         "gemm_only_effective_tflops": round(flops / (gemm_ms * 1e-3) / 1e12, 3),
         "fp32_vector_peak_tflops": 157.3,
     }
+    if trace is not None:
+        import numpy as np
+        tr = trace.cpu().numpy()
+        w0, w1 = int(mark0[0, 0]), int(mark1[0, 0])
+        tr = tr[tr[:, 0] > 0]
+        mhz = np.diff(tr[:, 1]) / np.maximum(np.diff(tr[:, 0]), 1) * 100.0
+        mid = (tr[1:, 0] + tr[:-1, 0]) / 2
+        busy = mhz[(mid >= w0) & (mid <= w1)]
+        idle = mhz[mid < w0]
+        out["shader_clock_mhz"] = {
+            "idle": round(float(idle.max()), 0) if idle.size else None,
+            "timed_region_mean": round(float(busy.mean()), 0) if busy.size else None,
+            "timed_region_min": round(float(busy.min()), 0) if busy.size else None,
+            "timed_region_max": round(float(busy.max()), 0) if busy.size else None,
+            "samples": int(busy.size), "sample_period_us": 100,
+            "note": "one extra wave on a second stream reads the shader cycle counter against the constant "
+                    "100 MHz counter; the timed region is delimited by two stamps on the work stream"}
     if not args.no_accuracy:
         from oracle import oracle as orc
         rows = 64 if k >= 8192 else 256

@@ -259,6 +259,14 @@ int wmmae_fragment_eye(int shape, int identity, float alpha, float *out,
 int wmmae_direct_product(int elem, int terms, int from_float, const float *u,
                          const float *v, float *h, void *stream);
 
+/* Measurement aid (no counterpart in the reference): one wave writes nsamples
+ * pairs out[2i] = constant-rate counter (100 MHz), out[2i+1] = shader cycle
+ * counter, one pair every period_ticks of the constant counter, then ends
+ * (nsamples * period_ticks <= 1e9, i.e. 10 s).  Launched on a second stream it
+ * records the shader clock while other kernels run. */
+int wmmae_clock_samples(unsigned long long *out, int nsamples,
+                        long long period_ticks, void *stream);
+
 /* utils::cp_async<size> (size 4, 8 or 16 bytes per lane): 128 threads move 256
  * elements from src to dst through LDS.  mode 0: lane-linear destinations
  * (the reference's test), 1: scattered destinations, 2: every third thread

@@ -48,6 +48,7 @@ EXPORTS = [
     "wmmae_fragment_ops",
     "wmmae_fragment_eye",
     "wmmae_direct_product",
+    "wmmae_clock_samples",
     "wmmae_utils_cp_async",
     "wmmae_utils_cast",
     "wmmae_mfma_probe",
@@ -102,6 +103,7 @@ _SIGNATURES = {
     "wmmae_fragment_ops": (_i, [_i, _i, _i, _c.c_float, _vp, _vp, _vp, _vp]),
     "wmmae_fragment_eye": (_i, [_i, _i, _c.c_float, _vp, _vp]),
     "wmmae_direct_product": (_i, [_i, _i, _i, _vp, _vp, _vp, _vp]),
+    "wmmae_clock_samples": (_i, [_vp, _i, _ll, _vp]),
     "wmmae_utils_cp_async": (_i, [_i, _i, _vp, _vp, _vp]),
     "wmmae_utils_cast": (_i, [_i, _vp, _vp, _ll, _vp]),
     "wmmae_mfma_probe": (_i, [_i, _i, _i, _i, _vp, _vp, _vp, _vp, _vp]),

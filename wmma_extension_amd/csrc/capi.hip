@@ -1117,6 +1117,20 @@ int wmmae_direct_product(const int elem, const int terms, const int from_float,
                     : go(wmmae_harness::direct_product_kernel<w::bfloat16, 3>);
 }
 
+int wmmae_clock_samples(unsigned long long *const out, const int nsamples,
+                        const long long period_ticks, void *const stream) {
+  if (!out)
+    return WMMAE_STATUS_NULL_POINTER;
+  // at most 10 s of sampling: the kernel must end on its own
+  if (nsamples < 1 || period_ticks < 0 ||
+      static_cast<long long>(nsamples) * period_ticks > 1000000000ll)
+    return WMMAE_STATUS_INVALID_VALUE;
+  hipLaunchKernelGGL(wmmae_harness::clock_samples_kernel, dim3(1), dim3(64), 0,
+                     static_cast<hipStream_t>(stream), out, nsamples,
+                     static_cast<unsigned long long>(period_ticks));
+  return launch_status();
+}
+
 int wmmae_utils_cp_async(const int size, const int mode, void *const dst,
                          const void *const src, void *const stream) {
   if (!dst || !src)

@@ -30,6 +30,7 @@
 //                             (reference: test/primitive/add_eye.cu:24-30)
 //   direct_product_kernel   : make_direct_product_fragment(_c3) + one MMA
 //                             (reference: test/primitive/direct_product.cu:44-99)
+//   clock_samples_kernel    : (constant-rate clock, shader clock) pairs over time
 //   cp_async_kernel         : utils::cp_async global -> LDS copies
 //                             (reference: test/utils/cp_async.cu:15-25)
 //   cast_kernel             : utils::cast (reference: test/utils/cast.cu)
@@ -611,6 +612,33 @@ __global__ void __launch_bounds__(64)
   w::fill_zero(fc);
   w::mma_sync(fc, fa, fb, fc);
   w::store_matrix_sync(h, fc, 16, w::mem_col_major);
+}
+
+// --------------------------------------------------------------------------
+// Shader-clock sampler: one lane records (constant 100 MHz counter, shader
+// cycle counter) pairs every `period` ticks of the constant counter, nsamples
+// times, then ends.  Run beside another kernel (on a second stream) it shows
+// how far the clock is pulled down while that kernel runs: on this chip the
+// matrix cores are power limited as soon as the operands are not constant.
+// The loop is bounded by the sample count and every wait by the constant
+// counter, so the kernel always ends.
+// --------------------------------------------------------------------------
+__global__ void __launch_bounds__(64)
+    clock_samples_kernel(unsigned long long *const out, const int nsamples,
+                         const unsigned long long period) {
+  if (threadIdx.x != 0)
+    return;
+  const unsigned long long t0 = wall_clock64();
+  for (int i = 0; i < nsamples; i++) {
+    const unsigned long long target = t0 + static_cast<unsigned long long>(i) * period;
+    unsigned long long now = wall_clock64();
+    while (now < target) {
+      __builtin_amdgcn_s_sleep(8);
+      now = wall_clock64();
+    }
+    out[2 * i] = now;
+    out[2 * i + 1] = clock64();
+  }
 }
 
 // --------------------------------------------------------------------------

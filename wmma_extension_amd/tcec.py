@@ -293,3 +293,13 @@ def direct_product(elem, terms, from_float, u, v):
     st = _lib.lib().wmmae_direct_product(elem, terms, from_float, _ptr(u), _ptr(v), _ptr(h), _stream())
     _lib.check(st, "wmmae_direct_product")
     return h.t()            # stored column-major
+
+
+def clock_samples(nsamples, period_ticks, stream=None, device="cuda:0"):
+    """Start the shader-clock sampler on `stream` (a torch.cuda.Stream; default: current).
+    Returns the (nsamples, 2) int64 CUDA tensor it fills: [:, 0] 100 MHz counter, [:, 1] shader cycles."""
+    out = torch.zeros((nsamples, 2), dtype=torch.int64, device=device)
+    s = ctypes.c_void_p(stream.cuda_stream) if stream is not None else _stream()
+    st = _lib.lib().wmmae_clock_samples(_ptr(out), nsamples, int(period_ticks), s)
+    _lib.check(st, "wmmae_clock_samples")
+    return out
