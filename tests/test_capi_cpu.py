@@ -120,3 +120,41 @@ def test_missing_library_fails_loudly(monkeypatch):
     monkeypatch.setattr(_lib, "LIB_PATH", "/nonexistent/libwmmae_tcec.so")
     with pytest.raises(RuntimeError, match="no CPU fallback"):
         _lib.lib()
+
+
+def test_harness_entries_reject_bad_arguments_on_the_host(h):
+    """The newer harness entry points return their status before any launch when
+    an argument is wrong (fake non-null pointers are never dereferenced)."""
+    p = ctypes.c_void_p(64)
+    f = ctypes.c_float
+    # complex one-wave product
+    assert h.wmmae_tcec_mma_complex(0, 1, None, p, p, p, 0, 0, 0, 0, 0, f(1.0), None) == -2
+    assert h.wmmae_tcec_mma_complex(0, 1, p, p, p, p, 0, 0, 0, 0, 5, f(1.0), None) == -1
+    assert h.wmmae_tcec_mma_complex(0, 1, p, p, p, p, 0, 0, 0, 0, 0, f(0.0), None) == -1
+    assert h.wmmae_tcec_mma_complex(3, 1, p, p, p, p, 0, 0, 0, 0, 0, f(1.0), None) == -4   # fp32 has no EC
+    assert h.wmmae_tcec_mma_complex(9, 0, p, p, p, p, 0, 0, 0, 0, 0, f(1.0), None) == -1
+    # fp32 policy on the real entry points
+    assert h.wmmae_tcec_mma_tile(0, 3, 1, 1, p, p, p, p, 0, 0, 0, 0, 0, None) == -4
+    assert h.wmmae_tcec_matvec(3, 1, p, p, p, 0, 0, None) == -4
+    assert h.wmmae_tcec_frag_dump(0, 3, 0, 0, p, p, 0, 0, None) == -4
+    # fragment operators, eye, direct product
+    assert h.wmmae_fragment_ops(6, 0, 0, f(1.0), p, p, p, None) == -1
+    assert h.wmmae_fragment_ops(0, 3, 0, f(1.0), p, p, p, None) == -1
+    assert h.wmmae_fragment_ops(0, 2, 0, f(1.0), p, p, p, None) == -4    # half accumulators do not exist
+    assert h.wmmae_fragment_ops(0, 0, 0, f(1.0), None, p, p, None) == -2
+    assert h.wmmae_fragment_eye(2, 0, f(1.0), p, None) == -1
+    assert h.wmmae_fragment_eye(0, 0, f(1.0), None, None) == -2
+    assert h.wmmae_direct_product(2, 2, 0, p, p, p, None) == -1
+    assert h.wmmae_direct_product(0, 4, 0, p, p, p, None) == -1
+    assert h.wmmae_direct_product(0, 2, 0, p, None, p, None) == -2
+    # utils
+    assert h.wmmae_utils_cp_async(12, 0, p, p, None) == -1
+    assert h.wmmae_utils_cp_async(4, 7, p, p, None) == -1
+    assert h.wmmae_utils_cp_async(16, 0, p, ctypes.c_void_p(72), None) == -7
+    assert h.wmmae_utils_cast(0, None, p, 4, None) == -2
+    assert h.wmmae_utils_cast(0, p, p, -1, None) == -1
+    assert h.wmmae_utils_cast(0, p, p, 0, None) == 0                       # nothing to do
+    # clock sampler: bounded by construction
+    assert h.wmmae_clock_samples(None, 10, 100, None) == -2
+    assert h.wmmae_clock_samples(p, 0, 100, None) == -1
+    assert h.wmmae_clock_samples(p, 100000, 100000, None) == -1            # would run for 100 s
