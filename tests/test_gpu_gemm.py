@@ -349,3 +349,35 @@ def test_api_level_gemm_fp32_policy(tc, orc, dev):
     with pytest.raises(WmmaeError) as e:
         tc.api_gemm(3, 1, m, n, k, 1.0, dA, k, dB, k, 0.0, dC, m)
     assert e.value.status == -4
+
+
+def test_pointer_array_entries_with_any_alignment(tc, orc, dev):
+    """Pointer-array entries that are only 4-byte aligned (matrices carved out of a
+    larger buffer at odd offsets): the fused kernel finds out by itself and falls back
+    to 4-byte requests; results equal the aligned call bit for bit."""
+    batch, m, n, k = 9, 72, 40, 96
+    rng = np.random.default_rng(123)
+    A = rng.standard_normal((batch, m, k)).astype(np.float32)
+    Bt = rng.standard_normal((batch, n, k)).astype(np.float32)
+    for offsets in ([1] * batch, [0, 1, 2, 3, 0, 5, 0, 7, 0]):
+        bufA = [torch.zeros(m * k + 8, dtype=torch.float32, device=dev) for _ in range(batch)]
+        bufB = [torch.zeros(n * k + 8, dtype=torch.float32, device=dev) for _ in range(batch)]
+        bufC = [torch.zeros(n * m + 8, dtype=torch.float32, device=dev) for _ in range(batch)]
+        As, Bs, Cs = [], [], []
+        for b, off in enumerate(offsets):
+            As.append(bufA[b][off:off + m * k].view(m, k)); As[-1].copy_(torch.from_numpy(A[b]))
+            Bs.append(bufB[b][off:off + n * k].view(n, k)); Bs[-1].copy_(torch.from_numpy(Bt[b]))
+            Cs.append(bufC[b][off:off + n * m].view(n, m))
+        pa = torch.tensor([t.data_ptr() for t in As], dtype=torch.int64, device=dev)
+        pb = torch.tensor([t.data_ptr() for t in Bs], dtype=torch.int64, device=dev)
+        pc = torch.tensor([t.data_ptr() for t in Cs], dtype=torch.int64, device=dev)
+        for policy in (0, 2):
+            tc.sgemm_batched("T", "N", m, n, k, 1.0, pa, k, pb, k, 0.0, pc, m, batch, policy)
+            torch.cuda.synchronize()
+            for b in range(batch):
+                single = _gemm(tc, dev, A[b], Bt[b].T, policy)
+                assert np.array_equal(Cs[b].cpu().numpy().T, single), (offsets[b], b, policy)
+                # nothing was written outside the matrix
+                off = offsets[b]
+                raw = bufC[b].cpu().numpy()
+                assert (raw[:off] == 0).all() and (raw[off + n * m:] == 0).all()
