@@ -37,6 +37,8 @@ WORKLOADS = {
     "c5b": dict(m=1024, n=1024, k=262144, batch=1, policy="F16_EC", dist="normal", mult=3,
                 desc="K-heavy TCEC SGEMM, M=N=1024, K=262144"),
 }
+# a timed region of a few milliseconds is measured while the power management still ramps
+DEFAULT_STEPS = {"c3": 200, "c5a": 400, "c5a_packed": 200, "c5b": 50, "c2": 100}
 PEAK_MFMA_TFLOPS = 2500.0      # dense fp16 / bf16 MFMA, MI355X
 PEAK_HBM_GBS = 8000.0
 # workloads whose dominant kernel is bound by HBM rather than by the matrix cores
@@ -212,8 +214,10 @@ def bench_primitives(args, torch, tcec, dev, w):
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
-    ap.add_argument("--steps", type=int, default=10)
-    ap.add_argument("--warmup", type=int, default=2)
+    ap.add_argument("--steps", type=int, default=None,
+                    help="timed steps; default 10 for the 16384^3 workloads and more for the short ones, so "
+                         "that the timed region lasts long enough for the clocks to settle")
+    ap.add_argument("--warmup", type=int, default=None, help="untimed steps; default 2 (20 for the short workloads)")
     ap.add_argument("--workload", default="c4", choices=sorted(WORKLOADS))
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--no-accuracy", action="store_true")
@@ -239,6 +243,10 @@ def main():
     dev = torch.device("cuda:0")
     torch.cuda.set_device(dev)
     w = dict(WORKLOADS[args.workload])
+    if args.warmup is None:
+        args.warmup = 20 if args.workload in DEFAULT_STEPS else 2
+    if args.steps is None:
+        args.steps = DEFAULT_STEPS.get(args.workload, 10)
     if args.dist is not None:
         w["dist"] = args.dist
     if w.get("kind") == "prim":

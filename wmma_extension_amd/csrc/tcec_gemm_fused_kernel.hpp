@@ -25,11 +25,19 @@
 // the tile.  With eight or more batch entries, an XCD (blockIdx % 8) takes
 // whole batch entries, so the tiles that share an operand panel share an L2.
 //
-// Raw layout of one 16-row block of a stage (2 KiB): when k is contiguous and
-// 16-byte aligned, two 16-byte requests per lane, lane l fetching row l%16,
-// k = 8*(l/16) + 4*h .. +3 for h = 0, 1 into slot [h][l]; otherwise eight
-// 4-byte requests, element e of the lane's eight into slot [e][l].  Either
-// way lane l later reads its own eight floats from consecutive-lane slots.
+// Raw layout of one 16-row block of a stage (2 KiB = 16 rows x 128 bytes).
+// When k is contiguous and 16-byte aligned, two 16-byte requests per lane:
+// request h covers rows 8h..8h+7, lane l fetching row 8h + l/8, so that eight
+// lanes take one whole 128-byte line (requests that touch half lines ran the
+// read stream at 4.1 instead of 5.2-6 TB/s).  Within its row, lane l fetches
+// 16-byte piece (l%8) ^ (2*((l/16)%4) + h): the pieces of a row are stored
+// permuted so that the conversion - where lane l needs the 32 bytes
+// k = 8*(l/16) .. +7 of row r = l%16, found as two 16-byte halves at byte
+// r*128 + 32*((l/16) ^ ((r/2)%4)), in swapped order for r >= 8 - does
+// not have the sixteen rows of a read start in the same LDS banks (each
+// ds_read_b128 of sixteen lanes covers all 64 banks once).  Otherwise (any
+// stride, any alignment) eight 4-byte requests per lane, element e of the
+// lane's eight into slot [e][l], read back from the same slots.
 // Rows past the matrix are clamped to the last row (their results are never
 // stored); k past K is clamped in the request and zeroed at the conversion.
 //
@@ -84,7 +92,8 @@ template <int N> __device__ __forceinline__ void wait_vmcnt_at_most() {
 
 // ABLATE (tuning only, 0 in the library): bit 0 drops the global->LDS requests,
 // bit 1 the conversion, bit 2 the MFMAs, bit 3 the per-stage barrier, bit 4 the
-// stores of C.
+// stores of C; bit 6 replaces the result by per-phase cycle counts (written
+// over C).
 template <class T, int TERMS, int BM, int BN, int ABLATE = 0,
           int NW = FusedConfig<TERMS, BM, BN>::NWAVES>
 __global__ void __launch_bounds__(64 * NW)
@@ -170,8 +179,8 @@ __global__ void __launch_bounds__(64 * NW)
 
   // ---- requests
   typedef const __attribute__((address_space(1))) float *gptr_t;
-  gptr_t rowptr[NQ];
-  auto set_rows = [&](const int i) __attribute__((always_inline)) {
+  gptr_t rowptr[NQ][2]; // [.][h]: row of request h (16-byte mode); [.][0] else
+  auto set_rows = [&](auto VEC, const int i) __attribute__((always_inline)) {
     int entry, tm, tn;
     decode(i, entry, tm, tn);
     // the pointer arrays are read with scalar loads (constant address space):
@@ -187,14 +196,19 @@ __global__ void __launch_bounds__(64 * NW)
 #pragma unroll
     for (int q = 0; q < NQ; q++) {
       const int rbl = wave + NW * q;
-      if (NW * q < RBA) {
-        int r = tm * BM + rbl * 16 + r16;
-        r = r < M ? r : M - 1;
-        rowptr[q] = (gptr_t)(Ab + static_cast<long long>(r) * p.a_rs);
-      } else {
-        int r = tn * BN + (rbl - RBA) * 16 + r16;
-        r = r < N ? r : N - 1;
-        rowptr[q] = (gptr_t)(Bb + static_cast<long long>(r) * p.b_rs);
+      const bool is_a = NW * q < RBA;
+      const int row0 = is_a ? tm * BM + rbl * 16 : tn * BN + (rbl - RBA) * 16;
+      const int last = is_a ? M - 1 : N - 1;
+      const float *const base = is_a ? Ab : Bb;
+      const long long rs = is_a ? p.a_rs : p.b_rs;
+#pragma unroll
+      for (int h = 0; h < 2; h++) {
+        // 16-byte mode: row 8h + lane/8; 4-byte mode: row lane%16
+        int r = row0 + (decltype(VEC)::value
+                            ? 8 * h + static_cast<int>(lane >> 3)
+                            : r16);
+        r = r < last ? r : last;
+        rowptr[q][h] = (gptr_t)(base + static_cast<long long>(r) * rs);
       }
     }
   };
@@ -208,12 +222,16 @@ __global__ void __launch_bounds__(64 * NW)
       unsigned char *const dst =
           lds_raw + slot * Cfg::RAW_STAGE_BYTES + rbl * 2048;
       if constexpr (decltype(VEC)::value) {
+        // K % 4 == 0 here: a piece is all in or all out
+        const int piece =
+            static_cast<int>((lane & 7u) ^ (2u * ((lane >> 4) & 3u)));
 #pragma unroll
         for (int h = 0; h < 2; h++) {
-          int k = ks * 32 + g8 + 4 * h;
-          k = k < K ? k : 0; // K % 4 == 0 here: a piece is all in or all out
+          int k = ks * 32 + 4 * (piece ^ h);
+          k = k < K ? k : 0;
           __builtin_amdgcn_global_load_lds(
-              (const __attribute__((address_space(1))) void *)(rowptr[q] + k),
+              (const __attribute__((address_space(1))) void *)(rowptr[q][h] +
+                                                                k),
               (__attribute__((address_space(3))) void *)(dst + h * 1024), 16, 0,
               0);
         }
@@ -224,7 +242,7 @@ __global__ void __launch_bounds__(64 * NW)
           int k = ks * 32 + g8 + e;
           k = k < K ? k : K - 1;
           __builtin_amdgcn_global_load_lds(
-              (const __attribute__((address_space(1))) void *)(rowptr[q] +
+              (const __attribute__((address_space(1))) void *)(rowptr[q][0] +
                                                                 k * kst),
               (__attribute__((address_space(3))) void *)(dst + e * 256), 4, 0,
               0);
@@ -237,35 +255,52 @@ __global__ void __launch_bounds__(64 * NW)
     constexpr int per_stage = NQ * (decltype(VEC)::value ? 2 : 8);
     wait_vmcnt_at_most<(NRAW - 1) * per_stage>();
   };
-  // raw slot -> split terms of fragment buffer `buf`
-  auto convert = [&](auto VEC, const int ks, const int slot, const int buf) __attribute__((always_inline)) {
-    if constexpr ((ABLATE & 2) != 0)
-      return;
+  // byte offset of this lane's eight floats inside a raw row block (16-byte mode)
+  const int vec_off =
+      r16 * 128 + 32 * static_cast<int>((lane >> 4) ^ ((lane >> 1) & 3u));
+  const int vec_off_lo = vec_off + 16 * (r16 >> 3);
+  const int vec_off_hi = vec_off + 16 * (1 - (r16 >> 3));
+  // conversion, first half: this lane's eight floats of each of the wave's
+  // row blocks, out of raw slot `slot`
+  auto load_raw = [&](auto VEC, const int slot, float (&v)[NQ][8]) __attribute__((always_inline)) {
 #pragma unroll
     for (int q = 0; q < NQ; q++) {
       const int rbl = wave + NW * q;
       const unsigned char *const src =
           lds_raw + slot * Cfg::RAW_STAGE_BYTES + rbl * 2048;
-      float v[8];
-      if constexpr (decltype(VEC)::value) {
-        const f32x4 lo = reinterpret_cast<const f32x4 *>(src)[lane];
-        const f32x4 hi = reinterpret_cast<const f32x4 *>(src)[64 + lane];
+      if constexpr ((ABLATE & 2) != 0) {
+#pragma unroll
+        for (int x = 0; x < 8; x++)
+          v[q][x] = 0.f;
+      } else if constexpr (decltype(VEC)::value) {
+        const f32x4 lo = *reinterpret_cast<const f32x4 *>(src + vec_off_lo);
+        const f32x4 hi = *reinterpret_cast<const f32x4 *>(src + vec_off_hi);
 #pragma unroll
         for (int x = 0; x < 4; x++) {
-          v[x] = lo[x];
-          v[4 + x] = hi[x];
+          v[q][x] = lo[x];
+          v[q][4 + x] = hi[x];
         }
       } else {
 #pragma unroll
         for (int e = 0; e < 8; e++)
-          v[e] = reinterpret_cast<const float *>(src)[e * 64 + lane];
+          v[q][e] = reinterpret_cast<const float *>(src)[e * 64 + lane];
       }
+    }
+  };
+  // conversion, second half: split and write the terms of k stage `ks` into
+  // fragment buffer `buf`
+  auto split_store = [&](const int ks, const int buf, float (&v)[NQ][8]) __attribute__((always_inline)) {
+    if constexpr ((ABLATE & 2) != 0)
+      return;
+#pragma unroll
+    for (int q = 0; q < NQ; q++) {
+      const int rbl = wave + NW * q;
       // k past K was clamped in the request: zero it (last stage only)
       if (ks * 32 + 32 > K) {
         const int left = K - (ks * 32 + g8);
 #pragma unroll
         for (int x = 0; x < 8; x++)
-          v[x] = x < left ? v[x] : 0.f;
+          v[q][x] = x < left ? v[q][x] : 0.f;
       }
       // the split of split_traits<T>, two elements at a time so that the
       // packed conversions are used: t0 = RN16(v), t1 = RN16((v - t0) * scale),
@@ -275,7 +310,7 @@ __global__ void __launch_bounds__(64 * NW)
       ab_vec t[3];
 #pragma unroll
       for (int x = 0; x < 8; x += 2) {
-        const f2_t vv = {v[x], v[x + 1]};
+        const f2_t vv = {v[q][x], v[q][x + 1]};
         const s2_t h0 = __builtin_convertvector(vv, s2_t);
         f2_t r = vv - __builtin_convertvector(h0, f2_t);
         if constexpr (traits::scale != 1.f)
@@ -364,8 +399,17 @@ __global__ void __launch_bounds__(64 * NW)
     }
   };
 
+  // Pipeline, per wave and stream stage s (one iteration of the k loop):
+  //   request stage s+1+NRAW into the raw slot that stage s+1 has left
+  //   wait until the wave's requests of stage s+2 have landed, read them
+  //   issue the MFMAs of stage s (fragments are in registers)
+  //   read the fragments of stage s+1 (converted last iteration) into the
+  //     same registers - the matrix core has fetched them by then
+  //   split stage s+2 and write its terms over the fragment buffer of stage s
+  //   barrier
+  // so the LDS latencies sit behind the MFMAs and the conversion arithmetic,
+  // and NRAW stages of requests are in flight while the wave computes.
   auto run = [&](auto VEC) __attribute__((always_inline)) {
-    // ---- prologue: fill the raw ring, convert stage 0
     int req_tile = 0, req_ks = 0; // next (tile, k stage) to request
     auto advance_request = [&]() __attribute__((always_inline)) {
       if (req_ks + 1 < num_k) {
@@ -373,56 +417,86 @@ __global__ void __launch_bounds__(64 * NW)
       } else if (req_tile + 1 < n_my) {
         req_tile++;
         req_ks = 0;
-        set_rows(req_tile);
+        set_rows(VEC, req_tile);
       } // else: stay on the last stage; the redundant requests land in free
         // slots and keep the in-flight count constant
     };
-    set_rows(0);
+    int conv_ks = 0; // k stage of the stream stage converted next
+    auto advance_conv = [&]() __attribute__((always_inline)) {
+      conv_ks = conv_ks + 1 == num_k ? 0 : conv_ks + 1;
+    };
+    ab_vec a[TERMS][MT_], b[TERMS][NT_];
+    auto read_frags = [&](const int buf) __attribute__((always_inline)) {
+      const u32x4 *const sa =
+          frag + ((buf * NRB + wm * MT_) * TERMS) * 64 + lane;
+      const u32x4 *const sb =
+          frag + ((buf * NRB + RBA + wn * NT_) * TERMS) * 64 + lane;
+#pragma unroll
+      for (int j = 0; j < NT_; j++)
+#pragma unroll
+        for (int t = 0; t < TERMS; t++)
+          b[t][j] = __builtin_bit_cast(ab_vec, sb[(j * TERMS + t) * 64]);
+#pragma unroll
+      for (int i = 0; i < MT_; i++)
+#pragma unroll
+        for (int t = 0; t < TERMS; t++)
+          a[t][i] = __builtin_bit_cast(ab_vec, sa[(i * TERMS + t) * 64]);
+    };
+    float v[NQ][8];
+
+    // ---- prologue: fill the raw ring, convert stages 0 and 1, load stage 0
+    set_rows(VEC, 0);
     for (int s = 0; s < NRAW; s++) {
       issue(VEC, req_ks, s);
       advance_request();
     }
-    wait_oldest_stage(VEC);
-    convert(VEC, 0, 0, 0);
-    clear_acc();
+    wait_oldest_stage(VEC); // stage 0
+    load_raw(VEC, 0, v);
+    split_store(conv_ks, 0, v);
+    advance_conv();
+    issue(VEC, req_ks, 0); // stage NRAW into the slot stage 0 has left
+    advance_request();
+    wait_oldest_stage(VEC); // stage 1
+    load_raw(VEC, 1 % NRAW, v);
+    split_store(conv_ks, 1, v);
+    advance_conv();
     asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");
+    read_frags(0);
+    // every wave has stage 0 in registers before anybody overwrites its buffer
+    asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");
+
+    // tuning only (ABLATE bit 6): shader-clock time spent per phase, written to C
+    unsigned long long prof[6] = {0, 0, 0, 0, 0, 0};
+    unsigned long long stamp = 0;
+    auto tick = [&](const int phase) __attribute__((always_inline)) {
+      if constexpr ((ABLATE & 64) != 0) {
+        __builtin_amdgcn_sched_barrier(0);
+        const unsigned long long now = __builtin_amdgcn_s_memtime();
+        if (phase >= 0)
+          prof[phase] += now - stamp;
+        stamp = now;
+        __builtin_amdgcn_sched_barrier(0);
+      }
+    };
 
     // The k loop of a tile is a loop of its own so that the accumulators are
     // touched by nothing but MFMAs inside it (they stay in AGPRs); the stream
     // of requests and conversions runs on across the tile boundary.
-    int slot_cur = 0; // raw slot of the stage being multiplied (converted, free)
-    int s = 0;        // its index in the stream
+    int slot_conv = 2 % NRAW; // raw slot of stage s+2
+    int s = 0;                // stream index of the stage being multiplied
     for (int cur_tile = 0; cur_tile < n_my; cur_tile++) {
       clear_acc();
       for (int cur_ks = 0; cur_ks < num_k; cur_ks++, s++) {
         const int buf = s & 1;
-        // refill the slot that stage s has left
-        issue(VEC, req_ks, slot_cur);
+        tick(-1);
+        // refill the slot that stage s+1 has left (it was converted last
+        // iteration): it is the one before slot_conv
+        issue(VEC, req_ks, slot_conv == 0 ? NRAW - 1 : slot_conv - 1);
         advance_request();
-
-        const u32x4 *const sa =
-            frag + ((buf * NRB + wm * MT_) * TERMS) * 64 + lane;
-        const u32x4 *const sb =
-            frag + ((buf * NRB + RBA + wn * NT_) * TERMS) * 64 + lane;
-        ab_vec a[TERMS][MT_], b[TERMS][NT_];
-#pragma unroll
-        for (int j = 0; j < NT_; j++)
-#pragma unroll
-          for (int t = 0; t < TERMS; t++)
-            b[t][j] = __builtin_bit_cast(ab_vec, sb[(j * TERMS + t) * 64]);
-#pragma unroll
-        for (int i = 0; i < MT_; i++)
-#pragma unroll
-          for (int t = 0; t < TERMS; t++)
-            a[t][i] = __builtin_bit_cast(ab_vec, sa[(i * TERMS + t) * 64]);
-
-        // next stage: raw -> terms, into the other fragment buffer.  After
-        // the last stage this converts a redundant tail request; nobody
-        // reads it.
-        const int slot_next = slot_cur + 1 == NRAW ? 0 : slot_cur + 1;
-        const int next_ks = cur_ks + 1 == num_k ? 0 : cur_ks + 1;
-        wait_oldest_stage(VEC);
-        convert(VEC, next_ks, slot_next, buf ^ 1);
+        tick(0);
+        wait_oldest_stage(VEC); // stage s+2 (past the end: a redundant tail stage)
+        tick(1);
+        load_raw(VEC, slot_conv, v);
 
         auto sweep = [&](f32x4(&acc)[MT_][NT_], const int ta, const int tb) __attribute__((always_inline)) {
 #pragma unroll
@@ -431,26 +505,53 @@ __global__ void __launch_bounds__(64 * NW)
             for (int j = 0; j < NT_; j++)
               acc[i][j] = mfma(a[ta][i], b[tb][j], acc[i][j]);
         };
-        // same products and order as tcec_gemm_kernel
-        if constexpr (TERMS >= 3) {
-          sweep(acc_err, 2, 0);
-          sweep(acc_err, 0, 2);
-          sweep(acc_err, 1, 1);
-        }
-        if constexpr (TERMS >= 2) {
-          sweep(acc_err, 1, 0);
-          sweep(acc_err, 0, 1);
-        }
-        sweep(acc_main, 0, 0);
-
-        slot_cur = slot_next;
+        auto multiply = [&]() __attribute__((always_inline)) {
+          // same products and order as tcec_gemm_kernel
+          if constexpr (TERMS >= 3) {
+            sweep(acc_err, 2, 0);
+            sweep(acc_err, 0, 2);
+            sweep(acc_err, 1, 1);
+          }
+          if constexpr (TERMS >= 2) {
+            sweep(acc_err, 1, 0);
+            sweep(acc_err, 0, 1);
+          }
+          sweep(acc_main, 0, 0);
+          // stage s+1 into the registers the MFMAs above have been fed from
+          read_frags(buf ^ 1);
+        };
+        // The two waves that share a SIMD run the matrix phase and the
+        // conversion phase in opposite order, so that one wave's MFMAs overlap
+        // the other's vector arithmetic instead of colliding with its MFMAs.
+        const bool matrix_first = NW < 8 || wave < NW / 2;
+        if (matrix_first)
+          multiply();
+        tick(2);
+        // stage s+2 over the buffer of stage s, which every wave took into
+        // registers before the last barrier
+        split_store(conv_ks, buf, v);
+        tick(3);
+        if (!matrix_first)
+          multiply();
+        advance_conv();
+        slot_conv = slot_conv + 1 == NRAW ? 0 : slot_conv + 1;
         if constexpr ((ABLATE & 8) == 0)
           asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");
+        tick(4);
       }
+      tick(-1);
       if constexpr ((ABLATE & 16) == 0)
         store_tile(cur_tile);
       else if (acc_main[0][0][0] == 123.456f) // keep the accumulators alive
         store_tile(cur_tile);
+      tick(5);
+    }
+    if constexpr ((ABLATE & 64) != 0) {
+      asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+      if (lane == 0)
+        for (int i = 0; i < 6; i++)
+          reinterpret_cast<unsigned long long *>(
+              p.C)[(blockIdx.x * NW + wave) * 8 + i] = prof[i];
     }
   };
   if (vec_a && vec_b)
