@@ -381,3 +381,29 @@ def test_pointer_array_entries_with_any_alignment(tc, orc, dev):
                 off = offsets[b]
                 raw = bufC[b].cpu().numpy()
                 assert (raw[:off] == 0).all() and (raw[off + n * m:] == 0).all()
+
+
+def test_sgemm_randomised_sweep(tc, orc, dev):
+    """Forty seeded random problems over both GEMM paths: shapes from 1 to ~900 (ragged),
+    all transposes, padded leading dimensions, random alpha/beta, all five policies."""
+    rng = np.random.default_rng(2024)
+    sizes = [1, 2, 7, 15, 16, 17, 31, 33, 63, 64, 65, 100, 127, 128, 129, 200, 255, 257, 300,
+             511, 512, 513, 640, 900]
+    for case in range(40):
+        m, n = (int(rng.choice(sizes)) for _ in range(2))
+        k = int(rng.choice([1, 3, 8, 31, 32, 33, 64, 100, 129, 256, 500]))
+        policy = int(rng.integers(0, 5))
+        ta, tb = rng.choice(["N", "T"]), rng.choice(["N", "T"])
+        alpha = float(rng.choice([1.0, -0.75, 2.5]))
+        beta = float(rng.choice([0.0, 0.0, 1.0, -1.5]))
+        ld_pad = int(rng.choice([0, 0, 1, 4]))
+        A = rng.uniform(-1, 1, (m, k)).astype(np.float32)
+        B = rng.uniform(-1, 1, (k, n)).astype(np.float32)
+        C = rng.uniform(-1, 1, (m, n)).astype(np.float32)
+        D = _gemm(tc, dev, A, B, policy, alpha=alpha, beta=beta, C=C, ta=ta, tb=tb, ld_pad=ld_pad)
+        kind, ec = POL_KIND[policy]
+        emu = orc.tcec_matmul(A, B, kind=kind, ec=ec, fk=32, main_outside=False)
+        expect = alpha * emu.astype(np.float64) + beta * C
+        tol = 32 * 2.0**-24 * max(1.0, np.abs(expect).max())
+        assert np.abs(D - expect).max() <= tol, (case, m, n, k, policy, ta, tb, alpha, beta, ld_pad)
+        _check(orc, D, A, B, policy, C=C, alpha=alpha, beta=beta)
