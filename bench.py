@@ -234,7 +234,7 @@ def main():
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py: this build measures one GPU only; --gpus must be 1 "
-              "(the path shards by C blocks / batch with no exchange, see DESIGN.md)", file=sys.stderr)
+              "(the path would shard by blocks of C or by batch entry, with no exchange)", file=sys.stderr)
         sys.exit(2)
 
     import torch
