@@ -236,6 +236,26 @@ int wmmae_tcec_mma_complex(int type, int ec, float *d, const float *a,
                            int c_col, int d_col, int rounding, float mul,
                            void *stream);
 
+/* One MMA D = A*B (+C) through mtk::wmma::mma::load_matrix_sync / mma_sync /
+ * store_matrix_sync.  elem: 0 half, 1 bfloat16, 2 float; shape: 0 16x16x16,
+ * 1 16x16x32, 2 32x32x8, 3 32x32x16 (float: shapes 0 and 2); a (M x K),
+ * b (K x N), c, d (M x N): fp32 images, dense, *_col = 1 for column major;
+ * c may be NULL.  Replaces: test/primitive/mma.cu:11-45. */
+int wmmae_primitive_mma(int elem, int shape, float *d, const float *a,
+                        const float *b, const float *c, int a_col, int b_col,
+                        int c_col, int d_col, void *stream);
+
+/* Error-corrected 16x16x16 half product built with foreach only (A, dA, B, dB
+ * fragments filled from the callback's mem_index, three MMAs).  a: 16x16
+ * column-major, b: 16x16 row-major, d: column-major.
+ * Replaces: test/primitive/foreach.cu:24-80. */
+int wmmae_foreach_ec(float *d, const float *a, const float *b, void *stream);
+
+/* y^T = x^T * E, 16 elements, E 16x16 column-major: load_vector into a
+ * row_major matrix_a fragment, one MMA, store_vector of the first row.
+ * Replaces: test/primitive/gevm.cu:22-43. */
+int wmmae_gevm(float *y, const float *x, const float *e, void *stream);
+
 /* Elementwise operators on 16x16x16 fragments: a, b are 16x16 row-major fp32
  * tiles cast to the element type on the way in, out is the result fragment
  * cast back.  op: 0 a+b, 1 a-b, 2 a*alpha, 3 a/alpha, 4 fma(alpha,a,b),

@@ -158,3 +158,13 @@ def test_harness_entries_reject_bad_arguments_on_the_host(h):
     assert h.wmmae_clock_samples(None, 10, 100, None) == -2
     assert h.wmmae_clock_samples(p, 0, 100, None) == -1
     assert h.wmmae_clock_samples(p, 100000, 100000, None) == -1            # would run for 100 s
+
+
+def test_primitive_entries_reject_bad_arguments_on_the_host(h):
+    p = ctypes.c_void_p(64)
+    assert h.wmmae_primitive_mma(3, 0, p, p, p, p, 0, 0, 0, 0, None) == -1
+    assert h.wmmae_primitive_mma(0, 4, p, p, p, p, 0, 0, 0, 0, None) == -1
+    assert h.wmmae_primitive_mma(2, 1, p, p, p, p, 0, 0, 0, 0, None) == -4     # fp32 has no 16x16x32
+    assert h.wmmae_primitive_mma(0, 0, None, p, p, p, 0, 0, 0, 0, None) == -2
+    assert h.wmmae_foreach_ec(p, None, p, None) == -2
+    assert h.wmmae_gevm(None, p, p, None) == -2

@@ -112,3 +112,69 @@ def test_layout_model_matches_silicon(tc, orc, dev, type_, shape):
                       torch.from_numpy(bbits).to(dev), torch.from_numpy(c).to(dev))
     torch.cuda.synchronize()
     assert np.array_equal(d.cpu().numpy(), a @ b + c)
+
+
+# ---------------------------------------------------------------- the reference's MMA-and-compare tests
+def _img(x, col):
+    return np.ascontiguousarray(x.T if col else x).reshape(-1).astype(np.float32)
+
+
+@pytest.mark.parametrize("elem", [0, 1, 2])
+@pytest.mark.parametrize("shape", [0, 1, 2, 3])
+def test_primitive_mma_all_shapes(tc, orc, dev, elem, shape):
+    """mma::load_matrix_sync -> mma_sync -> mma::store_matrix_sync on uniform[-1,1] inputs:
+    max|diff|/max|ref| below 16 eps of the operand type (test/primitive/mma.cu:103-105),
+    for every layout combination, with and without C."""
+    import itertools
+    from wmma_extension_amd import tcec as T
+    from wmma_extension_amd._lib import WmmaeError
+    m, n, k = T.PRIMITIVE_SHAPES[shape]
+    if elem == 2 and shape in (1, 3):
+        with pytest.raises(WmmaeError) as e:
+            z = torch.zeros(m * k, device=dev)
+            tc.primitive_mma(elem, shape, z, torch.zeros(k * n, device=dev), None, 0, 0, 0, 0)
+        assert e.value.status == -4
+        return
+    eps = {0: 2.0**-10, 1: 2.0**-7, 2: 2.0**-23}[elem]
+    rng = np.random.default_rng(17 + 4 * elem + shape)
+    for a_col, b_col, c_col, d_col, with_c in itertools.product((0, 1), repeat=5):
+        A = rng.uniform(-1, 1, (m, k)).astype(np.float32)
+        B = rng.uniform(-1, 1, (k, n)).astype(np.float32)
+        C = rng.uniform(-1, 1, (m, n)).astype(np.float32) if with_c else None
+        d = tc.primitive_mma(elem, shape, torch.from_numpy(_img(A, a_col)).to(dev),
+                             torch.from_numpy(_img(B, b_col)).to(dev),
+                             None if C is None else torch.from_numpy(_img(C, c_col)).to(dev),
+                             a_col, b_col, c_col, d_col).cpu().numpy()
+        D = d.reshape(n, m).T if d_col else d.reshape(m, n)
+        ref = orc.gemm_f64(A, B) + (C if with_c else 0)
+        assert orc.max_rel_err(D, ref) < 16 * eps, (a_col, b_col, c_col, d_col, with_c)
+
+
+def test_foreach_error_corrected_product(tc, orc, dev):
+    """A, dA, B, dB filled through foreach's mem_index, three MMAs: error below 1e-6
+    against FP64 on uniform[-1,1] inputs (test/primitive/foreach.cu:24-80, :120)."""
+    rng = np.random.default_rng(1)
+    A = rng.uniform(-1, 1, (16, 16)).astype(np.float32)
+    B = rng.uniform(-1, 1, (16, 16)).astype(np.float32)
+    d = tc.foreach_ec(torch.from_numpy(_img(A, 1)).to(dev), torch.from_numpy(_img(B, 0)).to(dev)).cpu().numpy()
+    D = d.reshape(16, 16).T
+    assert np.abs(D - orc.gemm_f64(A, B)).max() < 1e-6
+    # without the two correction products the error is a thousand times larger
+    h = lambda x: x.astype(np.float16).astype(np.float64)
+    assert np.abs(h(A) @ h(B) - orc.gemm_f64(A, B)).max() > 1e-4
+
+
+def test_gevm_identity_and_general(tc, orc, dev):
+    """Identity times a load_vector fragment returns the (fp16-rounded) vector through
+    store_vector (test/primitive/gevm.cu:22-43, eye at i%17==0); a general matrix gives
+    the row-vector product."""
+    rng = np.random.default_rng(2)
+    x = rng.uniform(-1, 1, 16).astype(np.float32)
+    eye = np.zeros(256, dtype=np.float32)
+    eye[np.arange(256) % 17 == 0] = 1.0
+    y = tc.gevm(torch.from_numpy(x).to(dev), torch.from_numpy(eye).to(dev)).cpu().numpy()
+    assert np.array_equal(y, x.astype(np.float16).astype(np.float32))
+    E = rng.uniform(-1, 1, (16, 16)).astype(np.float32)
+    y = tc.gevm(torch.from_numpy(x).to(dev), torch.from_numpy(_img(E, 1)).to(dev)).cpu().numpy()
+    h = lambda v: v.astype(np.float16).astype(np.float64)
+    assert np.abs(y - h(x) @ h(E)).max() < 1e-6

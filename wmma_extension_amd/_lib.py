@@ -45,6 +45,9 @@ EXPORTS = [
     "wmmae_tcec_elementwise",
     "wmmae_tcec_api_gemm",
     "wmmae_tcec_mma_complex",
+    "wmmae_primitive_mma",
+    "wmmae_foreach_ec",
+    "wmmae_gevm",
     "wmmae_fragment_ops",
     "wmmae_fragment_eye",
     "wmmae_direct_product",
@@ -100,6 +103,9 @@ _SIGNATURES = {
     "wmmae_tcec_elementwise": (_i, [_i, _i, _i, _vp, _c.c_float, _i, _i, _vp]),
     "wmmae_tcec_api_gemm": (_i, [_i, _i, _i, _i, _i, _fp, _vp, _i, _vp, _i, _fp, _vp, _i, _vp]),
     "wmmae_tcec_mma_complex": (_i, [_i, _i, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _c.c_float, _vp]),
+    "wmmae_primitive_mma": (_i, [_i, _i, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _vp]),
+    "wmmae_foreach_ec": (_i, [_vp, _vp, _vp, _vp]),
+    "wmmae_gevm": (_i, [_vp, _vp, _vp, _vp]),
     "wmmae_fragment_ops": (_i, [_i, _i, _i, _c.c_float, _vp, _vp, _vp, _vp]),
     "wmmae_fragment_eye": (_i, [_i, _i, _c.c_float, _vp, _vp]),
     "wmmae_direct_product": (_i, [_i, _i, _i, _vp, _vp, _vp, _vp]),

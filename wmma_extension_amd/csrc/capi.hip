@@ -1059,6 +1059,73 @@ int wmmae_tcec_mma_complex(const int type, const int ec, float *const d,
   });
 }
 
+int wmmae_primitive_mma(const int elem, const int shape, float *const d,
+                        const float *const a, const float *const b,
+                        const float *const c, const int a_col, const int b_col,
+                        const int c_col, const int d_col, void *const stream) {
+  if (!d || !a || !b)
+    return WMMAE_STATUS_NULL_POINTER;
+  if (elem < 0 || elem > 2 || shape < 0 || shape > 3)
+    return WMMAE_STATUS_INVALID_VALUE;
+  if (elem == 2 && shape != 0 && shape != 2)
+    return WMMAE_STATUS_NOT_SUPPORTED; // fp32 operands: 16x16x16 and 32x32x8
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  auto go = [&](auto kernel) {
+    hipLaunchKernelGGL(kernel, dim3(1), dim3(64), 0, s, d, a, b, c, c_col,
+                       d_col);
+    return launch_status();
+  };
+  return with_layout(a_col, [&](auto la) {
+    using AL = typename decltype(la)::type;
+    return with_layout(b_col, [&](auto lb) {
+      using BL = typename decltype(lb)::type;
+      auto by_shape = [&](auto tt) {
+        using T = typename decltype(tt)::type;
+        switch (shape) {
+        case 0:
+          return go(wmmae_harness::primitive_mma_kernel<T, 16, 16, 16, AL, BL>);
+        case 1:
+          if constexpr (!std::is_same<T, float>::value)
+            return go(
+                wmmae_harness::primitive_mma_kernel<T, 16, 16, 32, AL, BL>);
+          break;
+        case 2:
+          return go(wmmae_harness::primitive_mma_kernel<T, 32, 32, 8, AL, BL>);
+        default:
+          if constexpr (!std::is_same<T, float>::value)
+            return go(
+                wmmae_harness::primitive_mma_kernel<T, 32, 32, 16, AL, BL>);
+          break;
+        }
+        return static_cast<int>(WMMAE_STATUS_NOT_SUPPORTED);
+      };
+      if (elem == 0)
+        return by_shape(tag<w::half>{});
+      if (elem == 1)
+        return by_shape(tag<w::bfloat16>{});
+      return by_shape(tag<float>{});
+    });
+  });
+}
+
+int wmmae_foreach_ec(float *const d, const float *const a, const float *const b,
+                     void *const stream) {
+  if (!d || !a || !b)
+    return WMMAE_STATUS_NULL_POINTER;
+  hipLaunchKernelGGL(wmmae_harness::foreach_ec_kernel, dim3(1), dim3(64), 0,
+                     static_cast<hipStream_t>(stream), d, a, b);
+  return launch_status();
+}
+
+int wmmae_gevm(float *const y, const float *const x, const float *const e,
+               void *const stream) {
+  if (!y || !x || !e)
+    return WMMAE_STATUS_NULL_POINTER;
+  hipLaunchKernelGGL(wmmae_harness::gevm_kernel, dim3(1), dim3(64), 0,
+                     static_cast<hipStream_t>(stream), y, x, e);
+  return launch_status();
+}
+
 int wmmae_fragment_ops(const int op, const int use, const int elem,
                        const float alpha, const float *const a,
                        const float *const b, float *const out,

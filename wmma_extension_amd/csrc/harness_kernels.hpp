@@ -24,6 +24,12 @@
 //   mfma_probe_kernel       : one raw MFMA on caller-supplied bit patterns
 //   tcec_mma_complex_kernel : one-wave complex D = A*B (+C) through fragment_complex
 //                             (reference: test/tcec/mma_complex.cu:22-101)
+//   primitive_mma_kernel    : mma::load_matrix_sync -> mma_sync -> mma::store_matrix_sync
+//                             (reference: test/primitive/mma.cu:11-45)
+//   foreach_ec_kernel       : A, dA, B, dB built through foreach, three MMAs
+//                             (reference: test/primitive/foreach.cu:24-80)
+//   gevm_kernel             : identity times a load_vector fragment, store_vector
+//                             (reference: test/primitive/gevm.cu:22-43)
 //   fragment_ops_kernel     : operators +, -, *, /, fma on fragments
 //                             (reference: test/primitive/operators.cu:14-57)
 //   fragment_eye_kernel     : add_eye / make_identity_matrix
@@ -502,6 +508,98 @@ __global__ void __launch_bounds__(64)
   else
     tcec::store_matrix_sync(d, fd, N, dl);
   tcec::fill_zero(fd);
+}
+
+// --------------------------------------------------------------------------
+// One MMA through the mtk::wmma::mma spelling of the primitives.  a: M x K,
+// b: K x N, c/d: M x N fp32 images in the given layouts (dense leading
+// dimensions); operands are cast to T while loading.
+// --------------------------------------------------------------------------
+template <class T, int M, int N, int K, class AL, class BL>
+__global__ void __launch_bounds__(64)
+    primitive_mma_kernel(float *const d, const float *const a,
+                         const float *const b, const float *const c,
+                         const int c_col, const int d_col) {
+  namespace mma = w::mma;
+  mma::fragment<w::matrix_a, M, N, K, T, AL> fa;
+  mma::fragment<w::matrix_b, M, N, K, T, BL> fb;
+  mma::fragment<w::accumulator, M, N, K, float> fc, fd;
+  mma::load_matrix_sync(fa, a, std::is_same<AL, w::col_major>::value ? M : K);
+  mma::load_matrix_sync(fb, b, std::is_same<BL, w::col_major>::value ? K : N);
+  if (c != nullptr)
+    mma::load_matrix_sync(fc, c, c_col ? M : N,
+                          c_col ? w::mem_col_major : w::mem_row_major);
+  else
+    mma::fill_zero(fc);
+  mma::mma_sync(fd, fa, fb, fc);
+  mma::store_matrix_sync(d, fd, d_col ? M : N,
+                         d_col ? w::mem_col_major : w::mem_row_major);
+}
+
+// --------------------------------------------------------------------------
+// Error-corrected 16x16x16 product written with foreach only: the callback's
+// mem_index addresses the dense tile, the fragment registers receive the
+// leading half and the residual half of every element, and three MMAs follow.
+// a, b: 16x16 fp32, column-major for A and row-major for B as in the
+// reference's test; d column-major.
+// --------------------------------------------------------------------------
+__global__ void __launch_bounds__(64)
+    foreach_ec_kernel(float *const d, const float *const a,
+                      const float *const b) {
+  using FA = w::fragment<w::matrix_a, 16, 16, 16, w::half, w::col_major>;
+  using FB = w::fragment<w::matrix_b, 16, 16, 16, w::half, w::row_major>;
+  FA fa, fda;
+  FB fb, fdb;
+  w::fragment<w::accumulator, 16, 16, 16, float> fc;
+  w::foreach<FA>([&](const unsigned *list, const unsigned count,
+                     const unsigned mem_index) {
+    const float v = a[mem_index];
+    const w::half hv = w::detail::common::cast<w::half>(v);
+    const w::half dv =
+        w::detail::common::cast<w::half>(v - static_cast<float>(hv));
+    for (unsigned f = 0; f < count; f++) {
+      fa.x[list[f]] = hv;
+      fda.x[list[f]] = dv;
+    }
+  });
+  w::foreach<FB>([&](const unsigned *list, const unsigned count,
+                     const unsigned mem_index) {
+    const float v = b[mem_index];
+    const w::half hv = w::detail::common::cast<w::half>(v);
+    const w::half dv =
+        w::detail::common::cast<w::half>(v - static_cast<float>(hv));
+    for (unsigned f = 0; f < count; f++) {
+      fb.x[list[f]] = hv;
+      fdb.x[list[f]] = dv;
+    }
+  });
+  w::fill_zero(fc);
+  w::mma_sync(fc, fa, fdb, fc);
+  w::mma_sync(fc, fda, fb, fc);
+  w::mma_sync(fc, fa, fb, fc);
+  w::foreach<decltype(fc)>(w::mem_col_major,
+                           [&](const unsigned *list, const unsigned count,
+                               const unsigned mem_index) {
+                             for (unsigned f = 0; f < count; f++)
+                               d[mem_index] = fc.x[list[f]];
+                           });
+}
+
+// --------------------------------------------------------------------------
+// y^T = x^T * E for a 16x16 matrix E (the reference uses the identity): x goes
+// into the first row of a row_major matrix_a fragment through load_vector, the
+// product's first row comes back through store_vector.
+// --------------------------------------------------------------------------
+__global__ void __launch_bounds__(64)
+    gevm_kernel(float *const y, const float *const x, const float *const e) {
+  w::fragment<w::matrix_a, 16, 16, 16, w::half, w::row_major> fa;
+  w::fragment<w::matrix_b, 16, 16, 16, w::half, w::col_major> fb;
+  w::fragment<w::accumulator, 16, 16, 16, float> fc;
+  w::load_vector(fa, x);
+  w::load_matrix_sync(fb, e, 16);
+  w::fill_zero(fc);
+  w::mma_sync(fc, fa, fb, fc);
+  w::store_vector(y, fc, w::mem_row_major);
 }
 
 // --------------------------------------------------------------------------

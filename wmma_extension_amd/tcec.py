@@ -303,3 +303,31 @@ def clock_samples(nsamples, period_ticks, stream=None, device="cuda:0"):
     st = _lib.lib().wmmae_clock_samples(_ptr(out), nsamples, int(period_ticks), s)
     _lib.check(st, "wmmae_clock_samples")
     return out
+
+
+PRIMITIVE_SHAPES = {0: (16, 16, 16), 1: (16, 16, 32), 2: (32, 32, 8), 3: (32, 32, 16)}
+
+
+def primitive_mma(elem, shape, a, b, c, a_col, b_col, c_col, d_col):
+    """a, b, c: flat fp32 CUDA images of the operands in the given layouts; returns flat d."""
+    _need_cuda(a, b, c)
+    m, n, _ = PRIMITIVE_SHAPES[shape]
+    d = torch.full((m * n,), float("nan"), dtype=torch.float32, device=a.device)
+    st = _lib.lib().wmmae_primitive_mma(elem, shape, _ptr(d), _ptr(a), _ptr(b), _ptr(c), a_col, b_col,
+                                        c_col, d_col, _stream())
+    _lib.check(st, "wmmae_primitive_mma")
+    return d
+
+
+def foreach_ec(a, b):
+    _need_cuda(a, b)
+    d = torch.full((256,), float("nan"), dtype=torch.float32, device=a.device)
+    _lib.check(_lib.lib().wmmae_foreach_ec(_ptr(d), _ptr(a), _ptr(b), _stream()), "wmmae_foreach_ec")
+    return d
+
+
+def gevm(x, e):
+    _need_cuda(x, e)
+    y = torch.full((16,), float("nan"), dtype=torch.float32, device=x.device)
+    _lib.check(_lib.lib().wmmae_gevm(_ptr(y), _ptr(x), _ptr(e), _stream()), "wmmae_gevm")
+    return y
