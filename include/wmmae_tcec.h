@@ -82,10 +82,11 @@ int wmmae_query(int what, long long *out);
  * workspace holds the split operands (and K slices for K-heavy shapes); size
  * from wmmae_tcec_sgemm_workspace_bytes.  workspace == NULL lets the library
  * take it from the stream-ordered allocator (hipMallocAsync / hipFreeAsync on
- * `stream`).  Products with m, n <= 512 that need no K slices (flags == 0) are
- * split inside the GEMM kernel (as the reference's bgemm_kernel splits at
- * fragment load, batch_gemm.cu:196-386): they use no workspace, allocate
- * nothing and ignore the workspace arguments.  Both paths give the same bits. */
+ * `stream`).  Products whose operands are reused by few tiles (m, n <= 512, or
+ * larger with a short k; flags == 0, no K slices) are split inside the GEMM
+ * kernel (as the reference's bgemm_kernel splits at fragment load,
+ * batch_gemm.cu:196-386): they use no workspace, allocate nothing and ignore
+ * the workspace arguments.  Both paths give the same bits. */
 int wmmae_tcec_sgemm_workspace_bytes(int m, int n, int k, int batch, int policy,
                                      size_t *bytes);
 

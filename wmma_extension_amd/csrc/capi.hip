@@ -6,6 +6,7 @@
 #include "tcec_gemm_kernels.hpp"
 #include <wmmae_tcec.h>
 
+#include <algorithm>
 #include <hip/hip_runtime.h>
 
 namespace {
@@ -186,15 +187,26 @@ int launch_gemm(const GemmArgs &g) {
   const int splits = g.partial != nullptr ? g.splits : 1;
   const int split_stages = static_cast<int>(ceil_div(KT, splits));
   const int zdim = static_cast<int>(ceil_div(KT, split_stages));
-  hipLaunchKernelGGL(kernel, dim3(tiles_m * tiles_n, g.batch, zdim),
-                     dim3(Cfg::NTHREADS), Cfg::LDS_BYTES, g.stream, g.a, g.b,
+  // persistent workgroups: as many as are resident at once (the large tiles
+  // take most of a compute unit's LDS, so one per unit), each walking its
+  // share of the (tile, batch, slice) items
+  const long long items =
+      static_cast<long long>(tiles_m) * tiles_n * g.batch * zdim;
+  if (items >= (1ll << 31)) // the kernel counts items in 32 bits
+    return WMMAE_STATUS_INVALID_VALUE;
+  constexpr int per_cu =
+      (160 * 1024) / Cfg::LDS_BYTES > 4 ? 4 : (160 * 1024) / Cfg::LDS_BYTES;
+  const int grid = static_cast<int>(std::min<long long>(
+      items, static_cast<long long>(device_cus()) * per_cu));
+  hipLaunchKernelGGL(kernel, dim3(grid), dim3(Cfg::NTHREADS), Cfg::LDS_BYTES,
+                     g.stream, g.a, g.b,
                      g.c, g.m, g.n, KT, rb_a, rb_b, g.ldc, g.alpha, g.beta,
                      g.inv_scale, tiles_m, tiles_n, vec_store,
                      static_cast<long long>(rb_a) * KT * TERMS * 64,
                      static_cast<long long>(rb_b) * KT * TERMS * 64,
                      g.stride_c, split_stages,
                      zdim > 1 ? g.partial : static_cast<float *>(nullptr),
-                     g.c_ptrs);
+                     g.c_ptrs, g.batch, zdim);
   int st = launch_status();
   if (st == WMMAE_STATUS_SUCCESS && zdim > 1) {
     const long long blocks = ceil_div(static_cast<long long>(g.m) * g.n, 256);
@@ -311,13 +323,33 @@ int fused_dispatch(const int policy, const FusedArgs &f) {
   }
 }
 
-// Products this small are bound by HBM: every operand element is needed by at
-// most four blocks, and a separate split pass would double the traffic.
-// K-heavy single products that want K slices stay on the packed path.
+// Fused (split inside the GEMM kernel) or packed (split pass + MFMA kernel)?
+// The fused kernel does the same conversion and matrix work per 128x128x32
+// tile step whatever the shape, about 220 effective TFLOP/s with two terms, and
+// moves only the fp32 operands and C.  The packed path multiplies twice as
+// fast but first writes and re-reads the split operands, which pays off only
+// when every operand element is used by many tiles.  Both times are estimated
+// from rates measured on MI355X; K-heavy single products that want K slices
+// stay on the packed path.
 inline bool use_fused(const int m, const int n, const int k, const int batch,
-                      const int flags) {
-  return m <= 512 && n <= 512 && k > 0 && (flags & WMMAE_FLAG_RN_MAIN) == 0 &&
-         choose_splits(m, n, k, batch) == 1;
+                      const int flags, const int terms) {
+  if (k <= 0 || (flags & WMMAE_FLAG_RN_MAIN) != 0 ||
+      choose_splits(m, n, k, batch) != 1)
+    return false;
+  if (m <= 512 && n <= 512)
+    return true;
+  const double ab = (static_cast<double>(m) + n) * k * batch; // operand elements
+  const double c_bytes = 4.0 * m * n * batch;
+  const double flops = 2.0 * m * n * k * batch;
+  const double hbm = 4.5e12, hbm_stream = 5.5e12; // bytes/s: mixed, streaming
+  const double fused_rate = terms == 1 ? 250e12 : terms == 2 ? 220e12 : 155e12;
+  const double issued = terms == 1 ? 1.0 : terms == 2 ? 3.0 : 6.0;
+  const double t_fused =
+      std::max(flops / fused_rate, (4.0 * ab + c_bytes) / hbm);
+  const double t_packed =
+      (4.0 + 2.0 * terms) * ab / hbm_stream +
+      std::max(flops * issued / 1.4e15, (2.0 * terms * ab + c_bytes) / hbm);
+  return t_fused < t_packed;
 }
 
 inline bool is_n(const char t) { return t == 'N' || t == 'n'; }
@@ -510,7 +542,7 @@ int sgemm_impl(const char transa, const char transb, const int m, const int n,
       ldc < m)
     return WMMAE_STATUS_BAD_LEADING_DIM;
 
-  if (use_fused(m, n, k, batch, flags)) {
+  if (use_fused(m, n, k, batch, flags, p.terms)) {
     if (batch > (1 << 26)) // tile indices are 32-bit
       return WMMAE_STATUS_NOT_SUPPORTED;
     FusedArgs f;

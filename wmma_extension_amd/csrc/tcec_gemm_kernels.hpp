@@ -241,7 +241,8 @@ __global__ void __launch_bounds__(WGM *WGN * 64)
                      const long long batch_stride_b,
                      const long long batch_stride_c, const int split_stages,
                      float *__restrict__ partial,
-                     float *const *__restrict__ c_ptrs) {
+                     float *const *__restrict__ c_ptrs, const int batches,
+                     const int splits) {
   using Cfg = GemmConfig<MT, TERMS, BM, BN, WGM, WGN, NSTAGE, RN_MAIN>;
   typedef MT ab_vec __attribute__((ext_vector_type(8)));
   constexpr int NCH = Cfg::NCH, CH_A = Cfg::CH_A, CPW = Cfg::CPW;
@@ -256,95 +257,151 @@ __global__ void __launch_bounds__(WGM *WGN * 64)
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
   const int wm = wave % WGM, wn = wave / WGM;
 
-  // ---- block -> tile: spread consecutive ids over the 8 XCDs, then walk the
-  // tile grid in groups of GROUP tile rows so that the blocks resident on one
-  // XCD share A row panels and B column panels in that XCD's L2.
-  const int num_tiles = tiles_m * tiles_n;
-  int pid = blockIdx.x;
-  {
-    constexpr int XCDS = 8;
-    const int per = (num_tiles + XCDS - 1) / XCDS;
-    const int tall = (num_tiles % XCDS == 0) ? XCDS : (num_tiles % XCDS);
-    const int xcd = pid % XCDS, local = pid / XCDS;
-    pid = xcd < tall ? xcd * per + local
-                     : tall * per + (xcd - tall) * (per - 1) + local;
-  }
-  int tm, tn;
-  {
-    // 32 blocks run on one XCD at a time: a GROUP x (32/GROUP) patch of
-    // tiles that is close to square in elements needs the fewest L2 fills
-    constexpr int GROUP = BM > BN ? 4 : 8;
-    const int width = GROUP * tiles_n;
-    const int group = pid / width;
-    const int first_m = group * GROUP;
-    const int gsz = (tiles_m - first_m) < GROUP ? (tiles_m - first_m) : GROUP;
-    const int in_group = pid - group * width;
-    tm = first_m + in_group % gsz;
-    tn = in_group / gsz;
-  }
-  if constexpr ((ABLATE & 32) != 0)
-    tm = tn = 0;
-  const long long batch = blockIdx.y;
+  // ---- work items.  One item is one output tile of one batch entry (and one
+  // K slice under split-K); item ids run over tiles first, then batch entries,
+  // then slices.  The grid holds at most one workgroup per compute unit and a
+  // workgroup takes items blockIdx.x, blockIdx.x + gridDim.x, ...: the global
+  // -> LDS requests then run on across the item boundary, so that the next
+  // tile's first stages are already in LDS when the current tile is stored.
+  // Within the tile grid, consecutive ids are spread over the 8 XCDs and then
+  // walk the grid in groups of GROUP tile rows, so that the workgroups
+  // resident on one XCD share A row panels and B column panels in its L2.
+  // (the host keeps the item count below 2^31: 32-bit divisions only)
+  const unsigned num_tiles = static_cast<unsigned>(tiles_m * tiles_n);
+  const unsigned num_items = num_tiles * batches * splits;
+  const int n_my = static_cast<int>(
+      (num_items - blockIdx.x + gridDim.x - 1) / gridDim.x);
+  struct Item {
+    int tm, tn, batch, z;
+  };
+  auto decode = [&](const int i) {
+    const unsigned v = blockIdx.x + static_cast<unsigned>(i) * gridDim.x;
+    Item it;
+    const unsigned rest = v / num_tiles;
+    unsigned pid = v - rest * num_tiles;
+    it.z = static_cast<int>(rest / batches);
+    it.batch = static_cast<int>(rest - it.z * batches);
+    {
+      constexpr unsigned XCDS = 8;
+      const unsigned per = (num_tiles + XCDS - 1) / XCDS;
+      const unsigned tall =
+          (num_tiles % XCDS == 0) ? XCDS : (num_tiles % XCDS);
+      const unsigned xcd = pid % XCDS, local = pid / XCDS;
+      pid = xcd < tall ? xcd * per + local
+                       : tall * per + (xcd - tall) * (per - 1) + local;
+    }
+    {
+      // 32 workgroups run on one XCD at a time: a GROUP x (32/GROUP) patch of
+      // tiles that is close to square in elements needs the fewest L2 fills
+      constexpr unsigned GROUP = BM > BN ? 4 : 8;
+      const unsigned width = GROUP * tiles_n;
+      const unsigned group = pid / width;
+      const unsigned first_m = group * GROUP;
+      const unsigned gsz =
+          (tiles_m - first_m) < GROUP ? (tiles_m - first_m) : GROUP;
+      const unsigned in_group = pid - group * width;
+      const unsigned col = in_group / gsz;
+      it.tm = static_cast<int>(first_m + in_group - col * gsz);
+      it.tn = static_cast<int>(col);
+    }
+    if constexpr ((ABLATE & 32) != 0)
+      it.tm = it.tn = 0;
+    return it;
+  };
+  // Split-K: with `partial` set, slice z covers split_stages k stages from
+  // z*split_stages on and the workgroup writes its raw sum (no alpha / beta)
+  // to partial[z][batch] as a dense column-major M x N matrix;
+  // reduce_splits_kernel adds the slices.  Used when there are too few output
+  // tiles to fill the chip.
+  auto stages_of = [&](const Item &it) {
+    if (partial == nullptr)
+      return KT;
+    const int begin = it.z * split_stages;
+    return KT - begin < split_stages ? KT - begin : split_stages;
+  };
 
-  // ---- global sources of the chunks this wave requests every stage.
+  // ---- request cursor: the item and stage requested next, and the global
+  // sources of the chunks this wave requests every stage of that item.
   // Row blocks past the end of a packed operand are clamped to the last real
   // one: the rows / columns computed from them are never stored.
-  const u32x4 *gsrc[CPW];
+  // The sources are wave-uniform byte addresses kept in scalar registers (the
+  // empty asm statements pin them there); a lane adds its own 16-byte offset
+  // in the request instruction.
+  // Wave w requests chunks w*CPW .. w*CPW+CPW-1 of a stage, i.e. all terms of
+  // CPW/TERMS row blocks; the terms of one row block and stage are adjacent in
+  // the packed operand, so one address per row block serves them through the
+  // instruction's immediate offset.
+  constexpr unsigned STAGE_BYTES = CH_PER_RB * 1024u; // one stage of a row block
+  constexpr int RPW = CPW / CH_PER_RB;                // row blocks per wave
+  static_assert(CPW % CH_PER_RB == 0, "a wave requests whole row blocks");
+  unsigned long long gsrc[RPW];
+  const unsigned lane_off = lane * 16u;
+  int req_item = 0, req_st = 0, req_stages = 0;
+  auto set_sources = [&](const int i) {
+    const Item it = decode(i);
+    req_stages = stages_of(it);
+    const long long first_stage =
+        partial != nullptr ? static_cast<long long>(it.z) * split_stages : 0;
 #pragma unroll
-  for (int q = 0; q < CPW; q++) {
-    const int c = wave + Cfg::NW * q; // chunk index inside the stage
-    if (c < CH_A) {
-      const int rbl = c / CH_PER_RB, j = c % CH_PER_RB;
-      int rb = tm * RBM + rbl;
-      rb = rb < rb_a ? rb : rb_a - 1;
-      gsrc[q] = Ap + batch * batch_stride_a +
-                (static_cast<long long>(rb) * KT * CH_PER_RB + j) * 64;
-    } else {
-      const int cb = c - CH_A;
-      const int rbl = cb / CH_PER_RB, j = cb % CH_PER_RB;
-      int rb = tn * RBN + rbl;
-      rb = rb < rb_b ? rb : rb_b - 1;
-      gsrc[q] = Bp + batch * batch_stride_b +
-                (static_cast<long long>(rb) * KT * CH_PER_RB + j) * 64;
+    for (int g = 0; g < RPW; g++) {
+      const int r = wave * RPW + g; // row block inside the stage: A's, then B's
+      const bool is_a = r < RBM;
+      int rb = is_a ? it.tm * RBM + r : it.tn * RBN + (r - RBM);
+      const int rb_end = is_a ? rb_a : rb_b;
+      rb = rb < rb_end ? rb : rb_end - 1;
+      const u32x4 *const base = is_a ? Ap + it.batch * batch_stride_a
+                                     : Bp + it.batch * batch_stride_b;
+      gsrc[g] = reinterpret_cast<unsigned long long>(
+          base +
+          (static_cast<long long>(rb) * KT + first_stage) * (CH_PER_RB * 64));
+      asm volatile("" : "+s"(gsrc[g]));
     }
-  }
+  };
+  // after the last stage of the last item the cursor stays where it is: the
+  // few redundant requests keep the in-flight count constant, so one
+  // s_waitcnt immediate serves the whole loop
+  auto advance_request = [&]() {
+    if (req_st + 1 < req_stages) {
+      req_st++;
+#pragma unroll
+      for (int g = 0; g < RPW; g++) {
+        gsrc[g] += STAGE_BYTES;
+        asm volatile("" : "+s"(gsrc[g]));
+      }
+    } else if (req_item + 1 < n_my) {
+      req_item++;
+      req_st = 0;
+      set_sources(req_item);
+    }
+  };
 
   f32x4 acc_main[MT_][NT_], acc_err[MT_][NT_];
+  auto clear_acc = [&]() {
 #pragma unroll
-  for (int i = 0; i < MT_; i++)
+    for (int i = 0; i < MT_; i++)
 #pragma unroll
-    for (int j = 0; j < NT_; j++) {
-      acc_main[i][j] = f32x4{0.f, 0.f, 0.f, 0.f};
-      acc_err[i][j] = f32x4{0.f, 0.f, 0.f, 0.f};
-    }
+      for (int j = 0; j < NT_; j++) {
+        acc_main[i][j] = f32x4{0.f, 0.f, 0.f, 0.f};
+        acc_err[i][j] = f32x4{0.f, 0.f, 0.f, 0.f};
+      }
+  };
 
-  // Split-K: with `partial` set, blockIdx.z selects a range of split_stages
-  // k stages and the block writes its raw sum (no alpha / beta) to
-  // partial[z][batch] as a dense column-major M x N matrix; reduce_splits_kernel
-  // adds the slices.  Used when there are too few output tiles to fill the chip.
-  const int st_begin = partial != nullptr ? blockIdx.z * split_stages : 0;
-  const int num_stages =
-      partial != nullptr
-          ? (KT - st_begin < split_stages ? KT - st_begin : split_stages)
-          : KT;
-#pragma unroll
-  for (int q = 0; q < CPW; q++)
-    gsrc[q] += static_cast<long long>(st_begin) * (CH_PER_RB * 64);
-
-  // Request chunk Q (of this wave's CPW chunks) of stage `st` into LDS buffer
-  // `buf`.  The stage is clamped to the last one: the few redundant loads at
-  // the tail keep the in-flight count constant, so one s_waitcnt immediate
-  // serves the whole loop.
-  auto issue_chunk = [&](int st, const int buf, auto Q) {
+  // Request chunk Q (of this wave's CPW chunks) of the cursor's stage into
+  // LDS buffer `buf`.
+  auto issue_chunk = [&](const int buf, auto Q) {
     constexpr int q = decltype(Q)::value;
-    st = st < num_stages ? st : num_stages - 1;
-    const long long off = static_cast<long long>(st) * (CH_PER_RB * 64) + lane;
-    const int c = wave + Cfg::NW * q;
+    // first chunk of the row block; the immediate offset of the instruction
+    // moves the global and the LDS address alike to the chunk of term q%TERMS
+    const int c0 = wave * CPW + q - q % CH_PER_RB;
+    unsigned long long b = gsrc[q / CH_PER_RB];
+    unsigned vo = lane_off;
+    asm volatile("" : "+s"(b), "+v"(vo)); // scalar base + 32-bit lane offset
     __builtin_amdgcn_global_load_lds(
-        (const __attribute__((address_space(1))) void *)(gsrc[q] + off),
+        reinterpret_cast<const __attribute__((address_space(1))) char *>(b) +
+            vo,
         (__attribute__((address_space(3))) void *)(lds_raw +
-                                                   (buf * NCH + c) * 1024),
-        16, 0, 0);
+                                                   (buf * NCH + c0) * 1024),
+        16, (q % CH_PER_RB) * 1024, 0);
   };
 
   // In-place accumulate, written as inline assembly so that every accumulator
@@ -420,13 +477,23 @@ __global__ void __launch_bounds__(WGM *WGN * 64)
   // stage st in registers, so its LDS buffer is free for the new request.
   // Memory instructions are spread between the MFMAs so that the single wave
   // of a SIMD never sits on a full memory queue while the matrix core idles.
-  auto step = [&](const Frags &cur, Frags &nxt, const int st, const int wbuf,
+  // `skip_waits` > 0: the requests this step depends on were awaited before
+  // the previous tile's stores went out (see the epilogue), only the barrier
+  // is needed.
+  int skip_waits = 0;
+  auto step = [&](const Frags &cur, Frags &nxt, const int wbuf,
                   const int rbuf) {
-    // own loads of stage st+1 landed; own LDS reads of stage st finished
-    if constexpr ((ABLATE & 4) == 0)
-      asm volatile("s_waitcnt vmcnt(%0) lgkmcnt(0)\n\ts_barrier" ::"n"(
-                       (ABLATE & 8) ? 63 : CPW * (NSTAGE - 2))
-                   : "memory");
+    // own loads of the next stage landed; own LDS reads of this stage finished
+    if constexpr ((ABLATE & 4) == 0) {
+      if (skip_waits > 0) {
+        skip_waits--;
+        asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");
+      } else {
+        asm volatile("s_waitcnt vmcnt(%0) lgkmcnt(0)\n\ts_barrier" ::"n"(
+                         (ABLATE & 8) ? 63 : CPW * (NSTAGE - 2))
+                     : "memory");
+      }
+    }
 
     static_for<0, NMFMA>([&](auto N_) {
       constexpr int n = decltype(N_)::value;
@@ -462,7 +529,7 @@ __global__ void __launch_bounds__(WGM *WGN * 64)
       constexpr int qhi = ((n + 1) * CPW + NMFMA - 1) / NMFMA;
       static_for<qlo, (qhi < CPW ? qhi : CPW)>([&](auto Q) {
         if constexpr ((ABLATE & 1) == 0)
-          issue_chunk(st + NSTAGE, wbuf, Q);
+          issue_chunk(wbuf, Q);
         __builtin_amdgcn_sched_barrier(0);
       });
       // LDS reads due after this MFMA
@@ -474,85 +541,111 @@ __global__ void __launch_bounds__(WGM *WGN * 64)
         __builtin_amdgcn_sched_barrier(0);
       });
     });
+    advance_request();
   };
 
-  // ---- prologue: request the first NSTAGE stages, fetch stage 0's fragments
+  // ---- epilogue of one item: recombine, scale, store
+  auto store_item = [&](const Item &it) {
+    const bool to_partial = partial != nullptr;
+    float *const Cb =
+        to_partial
+            ? partial + (static_cast<long long>(it.z) * batches + it.batch) *
+                            (static_cast<long long>(M) * N)
+            : (c_ptrs != nullptr ? c_ptrs[it.batch]
+                                 : C + it.batch * batch_stride_c);
+    const long long ld_out = to_partial ? M : ldc;
+    const float a_out = to_partial ? 1.f : alpha;
+    const float b_out = to_partial ? 0.f : beta;
+    const int vec_out =
+        to_partial ? (M % 4 == 0)
+                   : (vec_store && (reinterpret_cast<uintptr_t>(Cb) & 15u) == 0);
+    const int row_base =
+        it.tm * BM + wm * Cfg::WM + 4 * static_cast<int>(lane >> 4);
+    const int col_base = it.tn * BN + wn * Cfg::WN + static_cast<int>(lane & 15u);
 #pragma unroll
-  for (int s = 0; s < NSTAGE; s++)
-    static_for<0, CPW>([&](auto Q) { issue_chunk(s, s, Q); });
+    for (int j = 0; j < NT_; j++) {
+      const int col = col_base + 16 * j;
+      if (col >= N)
+        continue;
+#pragma unroll
+      for (int i = 0; i < MT_; i++) {
+        const int row = row_base + 16 * i;
+        if (row >= M)
+          continue;
+        f32x4 v = acc_main[i][j];
+        if constexpr (TERMS >= 2)
+          v += acc_err[i][j] * inv_scale;
+        v *= a_out;
+        float *const dst = Cb + row + static_cast<long long>(col) * ld_out;
+        if (vec_out && row + 3 < M) {
+          if (b_out != 0.f)
+            v += b_out * *reinterpret_cast<const f32x4 *>(dst);
+          *reinterpret_cast<f32x4 *>(dst) = v;
+        } else {
+#pragma unroll
+          for (int x = 0; x < 4; x++) {
+            if (row + x < M) {
+              float o = v[x];
+              if (b_out != 0.f)
+                o += b_out * dst[x];
+              dst[x] = o;
+            }
+          }
+        }
+      }
+    }
+  };
+
+  // ---- prologue: request the first NSTAGE stages of the stream, fetch the
+  // first stage's fragments
+  set_sources(0);
+#pragma unroll
+  for (int s = 0; s < NSTAGE; s++) {
+    static_for<0, CPW>([&](auto Q) { issue_chunk(s, Q); });
+    advance_request();
+  }
   Frags f0, f1;
   asm volatile("s_waitcnt vmcnt(%0)\n\ts_barrier" ::"n"(CPW * (NSTAGE - 1))
                : "memory");
   static_for<0, NFRAG>([&](auto R_) { read_frag(f0, 0, R_); });
 
-  // ---- main loop, unrolled by two so that the fragment sets swap by name
+  // ---- items; the stage loop is unrolled by two so that the fragment sets
+  // swap by name.  Every step reads the fragments of the stream's next stage,
+  // which after an item's last stage is the first stage of the next item.
   int wbuf = 0; // buffer of the stage being multiplied == next to be refilled
   auto next_buf = [](const int b2) { return b2 + 1 == NSTAGE ? 0 : b2 + 1; };
-  int st = 0;
-  for (; st + 1 < num_stages; st += 2) {
-    const int b1 = next_buf(wbuf);
-    step(f0, f1, st, wbuf, b1);
-    const int b2 = next_buf(b1);
-    step(f1, f0, st + 1, b1, b2);
-    wbuf = b2;
-  }
-  if (st < num_stages)
-    step(f0, f1, st, wbuf, next_buf(wbuf));
-
-  // the redundant tail loads must not outlive the workgroup's LDS allocation;
-  // the no-ops cover the matrix core's write-to-VALU-read distance for the
-  // last accumulate instructions, which the compiler cannot see
-  asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)\n\ts_nop 15\n\ts_nop 15" ::
-                   : "memory");
-
-  // ---- epilogue: recombine, scale, store
-  const bool to_partial = partial != nullptr;
-  float *const Cb =
-      to_partial ? partial + (static_cast<long long>(blockIdx.z) * gridDim.y +
-                              batch) *
-                                 (static_cast<long long>(M) * N)
-                 : (c_ptrs != nullptr ? c_ptrs[batch]
-                                      : C + batch * batch_stride_c);
-  const long long ld_out = to_partial ? M : ldc;
-  const float a_out = to_partial ? 1.f : alpha;
-  const float b_out = to_partial ? 0.f : beta;
-  const int vec_out =
-      to_partial ? (M % 4 == 0)
-                 : (vec_store && (reinterpret_cast<uintptr_t>(Cb) & 15u) == 0);
-  const int row_base = tm * BM + wm * Cfg::WM + 4 * static_cast<int>(lane >> 4);
-  const int col_base = tn * BN + wn * Cfg::WN + static_cast<int>(lane & 15u);
-#pragma unroll
-  for (int j = 0; j < NT_; j++) {
-    const int col = col_base + 16 * j;
-    if (col >= N)
-      continue;
-#pragma unroll
-    for (int i = 0; i < MT_; i++) {
-      const int row = row_base + 16 * i;
-      if (row >= M)
-        continue;
-      f32x4 v = acc_main[i][j];
-      if constexpr (TERMS >= 2)
-        v += acc_err[i][j] * inv_scale;
-      v *= a_out;
-      float *const dst = Cb + row + static_cast<long long>(col) * ld_out;
-      if (vec_out && row + 3 < M) {
-        if (b_out != 0.f)
-          v += b_out * *reinterpret_cast<const f32x4 *>(dst);
-        *reinterpret_cast<f32x4 *>(dst) = v;
-      } else {
-#pragma unroll
-        for (int x = 0; x < 4; x++) {
-          if (row + x < M) {
-            float o = v[x];
-            if (b_out != 0.f)
-              o += b_out * dst[x];
-            dst[x] = o;
-          }
-        }
-      }
+  for (int item = 0; item < n_my; item++) {
+    const Item it = decode(item);
+    const int num_stages = stages_of(it);
+    clear_acc();
+    int st = 0;
+    for (; st + 1 < num_stages; st += 2) {
+      const int b1 = next_buf(wbuf);
+      step(f0, f1, wbuf, b1);
+      const int b2 = next_buf(b1);
+      step(f1, f0, b1, b2);
+      wbuf = b2;
     }
+    if (st < num_stages) {
+      // odd stage count: the next item's first fragments arrive in f1
+      const int b1 = next_buf(wbuf);
+      step(f0, f1, wbuf, b1);
+      wbuf = b1;
+      f0 = f1;
+    }
+    // The stores of C share the memory counter with the requests, and loads
+    // and stores need not complete in issue order, so a counted wait behind
+    // the stores would have to sit them out.  Everything requested so far is
+    // awaited here instead, before the stores go out; the steps that only
+    // depend on those requests skip their counted wait.  The no-ops cover the
+    // matrix core's write-to-VALU-read distance for the last accumulate
+    // instructions, which the compiler cannot see.
+    asm volatile("s_waitcnt vmcnt(0)\n\ts_nop 15\n\ts_nop 15" ::: "memory");
+    skip_waits = NSTAGE - 1;
+    store_item(it);
   }
+  // the redundant tail requests must not outlive the workgroup's LDS allocation
+  asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)" ::: "memory");
 }
 
 } // namespace wmmae_gemm
