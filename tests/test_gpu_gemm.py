@@ -116,15 +116,16 @@ def test_sgemm_k_zero_and_workspace(tc, orc, dev):
     B = rng.uniform(-1, 1, (64, 64)).astype(np.float32)
     ws = torch.empty(tc.workspace_bytes(64, 64, 64), dtype=torch.uint8, device=dev)
     assert np.array_equal(_gemm(tc, dev, A, B, 0, workspace=ws), _gemm(tc, dev, A, B, 0))
-    # a product large enough to go through the packed operands needs room for them
+    # a product that goes through the packed operands (the round-to-nearest flag always
+    # does) needs room for them
     A = rng.uniform(-1, 1, (1536, 1024)).astype(np.float32)
     B = rng.uniform(-1, 1, (1024, 1024)).astype(np.float32)
     ws = torch.empty(tc.workspace_bytes(1536, 1024, 1024), dtype=torch.uint8, device=dev)
-    assert np.array_equal(_gemm(tc, dev, A, B, 0, workspace=ws), _gemm(tc, dev, A, B, 0))
+    assert np.array_equal(_gemm(tc, dev, A, B, 0, flags=1, workspace=ws), _gemm(tc, dev, A, B, 0, flags=1))
     small = torch.empty(16, dtype=torch.uint8, device=dev)
     from wmma_extension_amd._lib import WmmaeError
     with pytest.raises(WmmaeError) as e:
-        _gemm(tc, dev, A, B, 0, workspace=small)
+        _gemm(tc, dev, A, B, 0, flags=1, workspace=small)
     assert e.value.status == -5
 
 

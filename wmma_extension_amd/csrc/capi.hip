@@ -187,17 +187,32 @@ int launch_gemm(const GemmArgs &g) {
   const int splits = g.partial != nullptr ? g.splits : 1;
   const int split_stages = static_cast<int>(ceil_div(KT, splits));
   const int zdim = static_cast<int>(ceil_div(KT, split_stages));
-  // persistent workgroups: as many as are resident at once (the large tiles
-  // take most of a compute unit's LDS, so one per unit), each walking its
-  // share of the (tile, batch, slice) items
   const long long items =
       static_cast<long long>(tiles_m) * tiles_n * g.batch * zdim;
   if (items >= (1ll << 31)) // the kernel counts items in 32 bits
     return WMMAE_STATUS_INVALID_VALUE;
+  // More items than resident workgroups (the large tiles take most of a
+  // compute unit's LDS, so one per unit):
+  //  * 8 or more batch entries: persistent workgroups, an XCD owns whole
+  //    entries, so that an entry's operands are read into one L2 only
+  //    (batch 256 of 1024x1024x256: 196 -> 256 effective TFLOPS);
+  //  * short K loops: persistent workgroups walking one shared list, their
+  //    requests running ahead into the next item;
+  //  * long K loops (64 stages = 2048 of k or more per item) of few entries:
+  //    one workgroup per item, handed out by the hardware as compute units
+  //    become free, which evens out compute units of unequal speed over many
+  //    rounds (a fixed share per workgroup measured 7 % slower at 16384^3).
   constexpr int per_cu =
       (160 * 1024) / Cfg::LDS_BYTES > 4 ? 4 : (160 * 1024) / Cfg::LDS_BYTES;
-  const int grid = static_cast<int>(std::min<long long>(
-      items, static_cast<long long>(device_cus()) * per_cu));
+  const long long resident = static_cast<long long>(device_cus()) * per_cu;
+  int grid = static_cast<int>(std::min(items, resident));
+  int entry_per_xcd = 0;
+  if (items > resident) {
+    if (g.batch >= 8 && zdim == 1 && resident % 8 == 0)
+      entry_per_xcd = 1;
+    else if (split_stages >= 64)
+      grid = static_cast<int>(items);
+  }
   hipLaunchKernelGGL(kernel, dim3(grid), dim3(Cfg::NTHREADS), Cfg::LDS_BYTES,
                      g.stream, g.a, g.b,
                      g.c, g.m, g.n, KT, rb_a, rb_b, g.ldc, g.alpha, g.beta,
@@ -206,7 +221,7 @@ int launch_gemm(const GemmArgs &g) {
                      static_cast<long long>(rb_b) * KT * TERMS * 64,
                      g.stride_c, split_stages,
                      zdim > 1 ? g.partial : static_cast<float *>(nullptr),
-                     g.c_ptrs, g.batch, zdim);
+                     g.c_ptrs, g.batch, zdim, entry_per_xcd);
   int st = launch_status();
   if (st == WMMAE_STATUS_SUCCESS && zdim > 1) {
     const long long blocks = ceil_div(static_cast<long long>(g.m) * g.n, 256);
@@ -338,17 +353,22 @@ inline bool use_fused(const int m, const int n, const int k, const int batch,
     return false;
   if (m <= 512 && n <= 512)
     return true;
+  // Times of both paths, linear fits to measurements on MI355X (batched
+  // products, m = n = 512 .. 2048, k = 64 .. 2048).  Fused kernel: C stored
+  // at 7.5 TB/s (two waves per SIMD, one stores while the other multiplies),
+  // then 250 / 242 / 166 effective TFLOPS for 1 / 2 / 3 terms.  Packed path:
+  // two split launches moving 4 + 2*terms bytes per operand element at
+  // 6.6 TB/s, C stored at 5.3 (4.0 with the 128x128 tile of three terms) TB/s
+  // while the single wave per SIMD does nothing else, then 700 / 460 / 252.
   const double ab = (static_cast<double>(m) + n) * k * batch; // operand elements
   const double c_bytes = 4.0 * m * n * batch;
   const double flops = 2.0 * m * n * k * batch;
-  const double hbm = 4.5e12, hbm_stream = 5.5e12; // bytes/s: mixed, streaming
-  const double fused_rate = terms == 1 ? 250e12 : terms == 2 ? 220e12 : 155e12;
-  const double issued = terms == 1 ? 1.0 : terms == 2 ? 3.0 : 6.0;
-  const double t_fused =
-      std::max(flops / fused_rate, (4.0 * ab + c_bytes) / hbm);
-  const double t_packed =
-      (4.0 + 2.0 * terms) * ab / hbm_stream +
-      std::max(flops * issued / 1.4e15, (2.0 * terms * ab + c_bytes) / hbm);
+  const double fused_rate = terms == 1 ? 250e12 : terms == 2 ? 242e12 : 166e12;
+  const double packed_rate = terms == 1 ? 700e12 : terms == 2 ? 460e12 : 252e12;
+  const double t_fused = c_bytes / 7.5e12 + flops / fused_rate;
+  const double t_packed = 12e-6 + (4.0 + 2.0 * terms) * ab / 6.6e12 +
+                          c_bytes / (terms == 3 ? 4.0e12 : 5.3e12) +
+                          flops / packed_rate;
   return t_fused < t_packed;
 }
 

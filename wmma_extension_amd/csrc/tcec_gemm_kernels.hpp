@@ -242,7 +242,7 @@ __global__ void __launch_bounds__(WGM *WGN * 64)
                      const long long batch_stride_c, const int split_stages,
                      float *__restrict__ partial,
                      float *const *__restrict__ c_ptrs, const int batches,
-                     const int splits) {
+                     const int splits, const int entry_per_xcd) {
   using Cfg = GemmConfig<MT, TERMS, BM, BN, WGM, WGN, NSTAGE, RN_MAIN>;
   typedef MT ab_vec __attribute__((ext_vector_type(8)));
   constexpr int NCH = Cfg::NCH, CH_A = Cfg::CH_A, CPW = Cfg::CPW;
@@ -258,31 +258,48 @@ __global__ void __launch_bounds__(WGM *WGN * 64)
   const int wm = wave % WGM, wn = wave / WGM;
 
   // ---- work items.  One item is one output tile of one batch entry (and one
-  // K slice under split-K); item ids run over tiles first, then batch entries,
-  // then slices.  The grid holds at most one workgroup per compute unit and a
-  // workgroup takes items blockIdx.x, blockIdx.x + gridDim.x, ...: the global
-  // -> LDS requests then run on across the item boundary, so that the next
-  // tile's first stages are already in LDS when the current tile is stored.
-  // Within the tile grid, consecutive ids are spread over the 8 XCDs and then
-  // walk the grid in groups of GROUP tile rows, so that the workgroups
-  // resident on one XCD share A row panels and B column panels in its L2.
+  // K slice under split-K).  A workgroup takes the items my_first,
+  // my_first + my_step, ... of a list: the global -> LDS requests run on
+  // across the item boundary, so that the next tile's first stages are
+  // already in LDS when the current tile is stored.
+  //   entry_per_xcd == 0: one list, tiles first, then batch entries, then
+  //     slices, shared by all workgroups.  Within the tile grid, consecutive
+  //     ids are spread over the 8 XCDs and then walk the grid in groups of
+  //     GROUP tile rows, so that the workgroups resident on one XCD share A
+  //     row panels and B column panels in its L2.
+  //   entry_per_xcd != 0 (no split-K, gridDim.x a multiple of 8): XCD x, i.e.
+  //     the workgroups with blockIdx.x % 8 == x, owns batch entries x, x+8,
+  //     ...: the operands of an entry are then read into one L2 only.
   // (the host keeps the item count below 2^31: 32-bit divisions only)
+  constexpr unsigned XCDS = 8;
   const unsigned num_tiles = static_cast<unsigned>(tiles_m * tiles_n);
-  const unsigned num_items = num_tiles * batches * splits;
-  const int n_my = static_cast<int>(
-      (num_items - blockIdx.x + gridDim.x - 1) / gridDim.x);
+  const unsigned my_xcd = blockIdx.x % XCDS;
+  const unsigned my_first = entry_per_xcd ? blockIdx.x / XCDS : blockIdx.x;
+  const unsigned my_step = entry_per_xcd ? gridDim.x / XCDS : gridDim.x;
+  const unsigned list_items =
+      entry_per_xcd
+          ? num_tiles * ((batches - my_xcd + XCDS - 1) / XCDS)
+          : num_tiles * batches * splits;
+  if (my_first >= list_items)
+    return; // nothing for this workgroup (before any barrier)
+  const int n_my =
+      static_cast<int>((list_items - my_first + my_step - 1) / my_step);
   struct Item {
     int tm, tn, batch, z;
   };
   auto decode = [&](const int i) {
-    const unsigned v = blockIdx.x + static_cast<unsigned>(i) * gridDim.x;
+    const unsigned v = my_first + static_cast<unsigned>(i) * my_step;
     Item it;
     const unsigned rest = v / num_tiles;
     unsigned pid = v - rest * num_tiles;
-    it.z = static_cast<int>(rest / batches);
-    it.batch = static_cast<int>(rest - it.z * batches);
-    {
-      constexpr unsigned XCDS = 8;
+    if (entry_per_xcd) {
+      it.z = 0;
+      it.batch = static_cast<int>(my_xcd + XCDS * rest);
+    } else {
+      it.z = static_cast<int>(rest / batches);
+      it.batch = static_cast<int>(rest - it.z * batches);
+    }
+    if (!entry_per_xcd) {
       const unsigned per = (num_tiles + XCDS - 1) / XCDS;
       const unsigned tall =
           (num_tiles % XCDS == 0) ? XCDS : (num_tiles % XCDS);
@@ -327,15 +344,20 @@ __global__ void __launch_bounds__(WGM *WGN * 64)
   // The sources are wave-uniform byte addresses kept in scalar registers (the
   // empty asm statements pin them there); a lane adds its own 16-byte offset
   // in the request instruction.
-  // Wave w requests chunks w*CPW .. w*CPW+CPW-1 of a stage, i.e. all terms of
-  // CPW/TERMS row blocks; the terms of one row block and stage are adjacent in
-  // the packed operand, so one address per row block serves them through the
-  // instruction's immediate offset.
+  // A wave requests all terms of RPW row blocks per stage; the terms of one
+  // row block and stage are adjacent in the packed operand, so one address
+  // per row block serves them through the instruction's immediate offset.
+  // Which row blocks: w, w + NW, w + 2 NW, ... with one or two terms (the
+  // waves then ask for neighbouring row blocks at the same time; batched
+  // 1024x1024x256 measured 276 against 258 effective TFLOPS), w*RPW ..
+  // w*RPW + RPW-1 with three terms (16384^3: 240 against 219).
   constexpr unsigned STAGE_BYTES = CH_PER_RB * 1024u; // one stage of a row block
   constexpr int RPW = CPW / CH_PER_RB;                // row blocks per wave
+  constexpr bool STRIDED_RB = TERMS <= 2;
+  constexpr int RB_STEP = STRIDED_RB ? Cfg::NW : 1; // between a wave's row blocks
   static_assert(CPW % CH_PER_RB == 0, "a wave requests whole row blocks");
   unsigned long long gsrc[RPW];
-  const unsigned lane_off = lane * 16u;
+  unsigned lane_off = lane * 16u;
   int req_item = 0, req_st = 0, req_stages = 0;
   auto set_sources = [&](const int i) {
     const Item it = decode(i);
@@ -344,7 +366,8 @@ __global__ void __launch_bounds__(WGM *WGN * 64)
         partial != nullptr ? static_cast<long long>(it.z) * split_stages : 0;
 #pragma unroll
     for (int g = 0; g < RPW; g++) {
-      const int r = wave * RPW + g; // row block inside the stage: A's, then B's
+      // row block inside the stage: A's, then B's
+      const int r = STRIDED_RB ? wave + Cfg::NW * g : wave * RPW + g;
       const bool is_a = r < RBM;
       int rb = is_a ? it.tm * RBM + r : it.tn * RBN + (r - RBM);
       const int rb_end = is_a ? rb_a : rb_b;
@@ -386,21 +409,26 @@ __global__ void __launch_bounds__(WGM *WGN * 64)
       }
   };
 
-  // Request chunk Q (of this wave's CPW chunks) of the cursor's stage into
-  // LDS buffer `buf`.
-  auto issue_chunk = [&](const int buf, auto Q) {
+  // Request chunk Q (of this wave's CPW chunks) of the cursor's stage; w_base
+  // is the LDS byte offset of the wave's first chunk in the target buffer.
+  auto wave_base = [&](const int buf) {
+    return (buf * NCH + wave * (STRIDED_RB ? CH_PER_RB : CPW)) * 1024;
+  };
+  auto issue_chunk = [&](const int w_base, auto Q) {
     constexpr int q = decltype(Q)::value;
     // first chunk of the row block; the immediate offset of the instruction
     // moves the global and the LDS address alike to the chunk of term q%TERMS
-    const int c0 = wave * CPW + q - q % CH_PER_RB;
-    unsigned long long b = gsrc[q / CH_PER_RB];
-    unsigned vo = lane_off;
-    asm volatile("" : "+s"(b), "+v"(vo)); // scalar base + 32-bit lane offset
+    // (redefined in place: the address is then formed here, as the
+    // instruction's scalar base + 32-bit lane offset, and not hoisted into
+    // vector registers)
+    asm volatile("" : "+s"(gsrc[q / CH_PER_RB]), "+v"(lane_off));
     __builtin_amdgcn_global_load_lds(
-        reinterpret_cast<const __attribute__((address_space(1))) char *>(b) +
-            vo,
-        (__attribute__((address_space(3))) void *)(lds_raw +
-                                                   (buf * NCH + c0) * 1024),
+        reinterpret_cast<const __attribute__((address_space(1))) char *>(
+            gsrc[q / CH_PER_RB]) +
+            lane_off,
+        (__attribute__((address_space(3))) void *)(lds_raw + w_base +
+                                                   (q / CH_PER_RB) * RB_STEP *
+                                                       CH_PER_RB * 1024),
         16, (q % CH_PER_RB) * 1024, 0);
   };
 
@@ -438,17 +466,17 @@ __global__ void __launch_bounds__(WGM *WGN * 64)
   constexpr int NFRAG = TERMS * (MT_ + NT_);
   // fragment IDX of a stage (compile-time index, so that every fragment is a
   // fixed register): B fragments first, then A
-  auto read_frag = [&](Frags &f, const int buf, auto IDX) {
+  auto read_frag = [&](Frags &f, const int r_base, auto IDX) {
     constexpr int r = decltype(IDX)::value;
+    const u32x4 *const stage =
+        reinterpret_cast<const u32x4 *>(lds_raw + r_base) + lane;
     if constexpr (r < TERMS * NT_) {
       constexpr int j = r / TERMS, t = r % TERMS;
-      const u32x4 *const sb =
-          lds + (buf * NCH + CH_A + wn * NT_ * CH_PER_RB) * 64 + lane;
+      const u32x4 *const sb = stage + (CH_A + wn * NT_ * CH_PER_RB) * 64;
       f.b[t][j] = __builtin_bit_cast(ab_vec, sb[(j * CH_PER_RB + t) * 64]);
     } else {
       constexpr int i = (r - TERMS * NT_) / TERMS, t = (r - TERMS * NT_) % TERMS;
-      const u32x4 *const sa =
-          lds + (buf * NCH + wm * MT_ * CH_PER_RB) * 64 + lane;
+      const u32x4 *const sa = stage + (wm * MT_ * CH_PER_RB) * 64;
       f.a[t][i] = __builtin_bit_cast(ab_vec, sa[(i * CH_PER_RB + t) * 64]);
     }
   };
@@ -466,6 +494,8 @@ __global__ void __launch_bounds__(WGM *WGN * 64)
 #define WMMAE_TUNE_SPAN_NUM 3
 #define WMMAE_TUNE_SPAN_DEN 4
 #endif
+  // MFMA after which the last request of a step goes out
+  constexpr int N_ADVANCE = (NMFMA * (CPW - 1)) / CPW;
   constexpr int SPAN =
       (NMFMA * WMMAE_TUNE_SPAN_NUM) / WMMAE_TUNE_SPAN_DEN > 0
           ? (NMFMA * WMMAE_TUNE_SPAN_NUM) / WMMAE_TUNE_SPAN_DEN
@@ -483,16 +513,22 @@ __global__ void __launch_bounds__(WGM *WGN * 64)
   int skip_waits = 0;
   auto step = [&](const Frags &cur, Frags &nxt, const int wbuf,
                   const int rbuf) {
+    // LDS offsets of this step, worked out before the barrier so that nothing
+    // stands between it and the first MFMA
+    int w_base = wave_base(wbuf);
+    int r_base = rbuf * (NCH * 1024);
+    asm volatile("" : "+s"(w_base), "+s"(r_base));
     // own loads of the next stage landed; own LDS reads of this stage finished
     if constexpr ((ABLATE & 4) == 0) {
-      if (skip_waits > 0) {
+      // the branch sits before the barrier, where the wave waits anyway
+      if (skip_waits > 0)
         skip_waits--;
-        asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");
-      } else {
-        asm volatile("s_waitcnt vmcnt(%0) lgkmcnt(0)\n\ts_barrier" ::"n"(
-                         (ABLATE & 8) ? 63 : CPW * (NSTAGE - 2))
+      else
+        asm volatile("s_waitcnt vmcnt(%0)" ::"n"((ABLATE & 8)
+                                                     ? 63
+                                                     : CPW * (NSTAGE - 2))
                      : "memory");
-      }
+      asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");
     }
 
     static_for<0, NMFMA>([&](auto N_) {
@@ -529,19 +565,24 @@ __global__ void __launch_bounds__(WGM *WGN * 64)
       constexpr int qhi = ((n + 1) * CPW + NMFMA - 1) / NMFMA;
       static_for<qlo, (qhi < CPW ? qhi : CPW)>([&](auto Q) {
         if constexpr ((ABLATE & 1) == 0)
-          issue_chunk(wbuf, Q);
+          issue_chunk(w_base, Q);
         __builtin_amdgcn_sched_barrier(0);
       });
+      // all requests of this step are out: move the cursor on while the
+      // remaining MFMAs run
+      if constexpr (n == N_ADVANCE) {
+        advance_request();
+        __builtin_amdgcn_sched_barrier(0);
+      }
       // LDS reads due after this MFMA
       constexpr int lo = n == 0 ? 0 : reads_due(n, SPAN, NFRAG);
       constexpr int hi = n + 1 == NMFMA ? NFRAG : reads_due(n + 1, SPAN, NFRAG);
       static_for<lo, hi>([&](auto R_) {
         if constexpr ((ABLATE & 2) == 0)
-          read_frag(nxt, rbuf, R_);
+          read_frag(nxt, r_base, R_);
         __builtin_amdgcn_sched_barrier(0);
       });
     });
-    advance_request();
   };
 
   // ---- epilogue of one item: recombine, scale, store
@@ -601,7 +642,7 @@ __global__ void __launch_bounds__(WGM *WGN * 64)
   set_sources(0);
 #pragma unroll
   for (int s = 0; s < NSTAGE; s++) {
-    static_for<0, CPW>([&](auto Q) { issue_chunk(s, Q); });
+    static_for<0, CPW>([&](auto Q) { issue_chunk(wave_base(s), Q); });
     advance_request();
   }
   Frags f0, f1;
