@@ -534,7 +534,12 @@ __global__ void __launch_bounds__(WGM *WGN * 64)
     static_for<0, NMFMA>([&](auto N_) {
       constexpr int n = decltype(N_)::value;
       constexpr int p = n / NTILE;
-      constexpr int i = (n % NTILE) / NT_, j = n % NT_;
+      // tiles in serpentine order: consecutive MFMAs share the A fragment
+      // along a row of tiles and the B fragment at the turn (fewer operand
+      // bits change between instructions; measured 1 % faster under the
+      // power limit)
+      constexpr int i = (n % NTILE) / NT_;
+      constexpr int j = (i % 2) ? NT_ - 1 - n % NT_ : n % NT_;
       // (term of A, term of B) of product p
       constexpr int ta =
           TERMS == 1   ? 0
