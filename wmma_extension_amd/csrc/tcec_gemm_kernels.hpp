@@ -300,12 +300,25 @@ __global__ void __launch_bounds__(WGM *WGN * 64)
       it.batch = static_cast<int>(rest - it.z * batches);
     }
     if (!entry_per_xcd) {
-      const unsigned per = (num_tiles + XCDS - 1) / XCDS;
-      const unsigned tall =
-          (num_tiles % XCDS == 0) ? XCDS : (num_tiles % XCDS);
-      const unsigned xcd = pid % XCDS, local = pid / XCDS;
-      pid = xcd < tall ? xcd * per + local
-                       : tall * per + (xcd - tall) * (per - 1) + local;
+      // Ids x, x+8, x+16, ... run on XCD x, 32 of them at a time: these 32
+      // get one patch of the walk below, and the eight XCDs get eight
+      // neighbouring patches, which share the patches' A row panels: what
+      // misses in one XCD's L2 is then in flight to, or already in, the
+      // memory-side cache for the others.  The ids beyond the last full
+      // round of 8 x 32 are cut into eight runs, one per XCD.
+      constexpr unsigned PATCH = 32;
+      const unsigned full = num_tiles / (XCDS * PATCH) * (XCDS * PATCH);
+      if (pid < full) {
+        const unsigned xcd = pid % XCDS, local = pid / XCDS;
+        pid = ((local / PATCH) * XCDS + xcd) * PATCH + local % PATCH;
+      } else {
+        const unsigned rem = num_tiles - full, t = pid - full;
+        const unsigned per = (rem + XCDS - 1) / XCDS;
+        const unsigned tall = (rem % XCDS == 0) ? XCDS : (rem % XCDS);
+        const unsigned xcd = t % XCDS, local = t / XCDS;
+        pid = full + (xcd < tall ? xcd * per + local
+                                 : tall * per + (xcd - tall) * (per - 1) + local);
+      }
     }
     {
       // 32 workgroups run on one XCD at a time: a GROUP x (32/GROUP) patch of
@@ -520,7 +533,9 @@ __global__ void __launch_bounds__(WGM *WGN * 64)
     asm volatile("" : "+s"(w_base), "+s"(r_base));
     // own loads of the next stage landed; own LDS reads of this stage finished
     if constexpr ((ABLATE & 4) == 0) {
-      // the branch sits before the barrier, where the wave waits anyway
+      // the requests of the stage read next are older than those of the
+      // NSTAGE-2 stages after it (the branch sits before the barrier, where
+      // the wave waits anyway)
       if (skip_waits > 0)
         skip_waits--;
       else
