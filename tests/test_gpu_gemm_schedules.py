@@ -1,0 +1,112 @@
+"""The packed GEMM kernel hands its (tile, batch entry, K slice) items to workgroups in
+three ways (persistent workgroups with XCD-owned batch entries, persistent workgroups on
+one shared list, one workgroup per item).  Which one runs depends only on the shape, and
+none of them may change a single bit of the result: every case below computes the same
+product twice, once in a shape that takes the schedule under test and once cut into
+pieces small enough for one workgroup per item, and compares the bytes.  One piece is also
+checked against FP64 to the driver's accuracy bound."""
+import numpy as np
+import pytest
+import torch
+
+pytestmark = pytest.mark.gpu
+
+TERMS = {0: 2, 1: 1, 2: 3}
+
+
+def _uniform(shape, seed, dev):
+    g = torch.Generator(device="cpu").manual_seed(seed)
+    return (torch.rand(shape, generator=g, dtype=torch.float32) * 2 - 1).to(dev)
+
+
+def _pack(tc, policy, X, dev):
+    """X: (batch, rows, k) fp32 on the device -> packed bytes, bytes per entry."""
+    batch, rows, k = X.shape
+    per = tc.pack_bytes(rows, k, 1, policy)
+    assert tc.pack_bytes(rows, k, batch, policy) == per * batch
+    p = torch.empty(per * batch, dtype=torch.uint8, device=dev)
+    tc.pack(policy, rows, k, X, k, 1, p, batch, rows * k)
+    return p, per
+
+
+def _fp64_check(orc, A, B, C, policy):
+    ref = orc.gemm_f64(A.cpu().numpy(), B.cpu().numpy().T)
+    got = C.cpu().numpy().T
+    assert orc.max_rel_err(got, ref) < (4e-6 if policy != 1 else 2e-2)
+
+
+@pytest.mark.parametrize("policy", [0, 2])
+@pytest.mark.parametrize("shape", [(1024, 1024, 160, 9), (520, 1000, 64, 21), (1024, 1024, 32, 9),
+                                   (512, 512, 2080, 36)])
+def test_xcd_owned_batch_entries_equal_single_entry_calls(tc, orc, dev, policy, shape):
+    """8 or more entries and more items than resident workgroups: an XCD walks whole entries,
+    requests run on into the next item (1, 2, 5 and 65 stages per item, odd and even)."""
+    m, n, k, batch = shape
+    A = _uniform((batch, m, k), 100 + k, dev)
+    B = _uniform((batch, n, k), 200 + k, dev)
+    C0 = _uniform((batch, n, m), 300 + k, dev)
+    pa, per_a = _pack(tc, policy, A, dev)
+    pb, per_b = _pack(tc, policy, B, dev)
+    C = C0.clone()
+    tc.gemm_packed(policy, m, n, k, 1.25, pa, pb, -0.5, C, m, batch, m * n)
+    ref = C0.clone()
+    for e in range(batch):
+        tc.gemm_packed(policy, m, n, k, 1.25, pa[e * per_a:(e + 1) * per_a],
+                       pb[e * per_b:(e + 1) * per_b], -0.5, ref[e], m)
+    torch.cuda.synchronize()
+    assert torch.equal(C, ref)
+    e = batch - 1
+    plain = torch.zeros((n, m), dtype=torch.float32, device=dev)
+    tc.gemm_packed(policy, m, n, k, 1.0, pa[e * per_a:(e + 1) * per_a],
+                   pb[e * per_b:(e + 1) * per_b], 0.0, plain, m)
+    _fp64_check(orc, A[e], B[e], plain, policy)
+
+
+@pytest.mark.parametrize("policy", [0, 2])
+@pytest.mark.parametrize("shape", [(4096, 4096, 96, 1), (2048, 3000, 40, 3), (4096, 2048, 1024, 2)])
+def test_persistent_shared_list_equals_column_blocks(tc, orc, dev, policy, shape):
+    """Few entries, short K loops, more tiles than resident workgroups: persistent
+    workgroups on one list.  The same product from column blocks of 512 columns of B
+    (few enough tiles for one workgroup each) has to agree bit for bit."""
+    m, n, k, batch = shape
+    A = _uniform((batch, m, k), 400 + k, dev)
+    B = _uniform((batch, n, k), 500 + k, dev)
+    pa, per_a = _pack(tc, policy, A, dev)
+    pb, per_b = _pack(tc, policy, B, dev)
+    C = torch.full((batch, n, m), 7.0, dtype=torch.float32, device=dev)
+    tc.gemm_packed(policy, m, n, k, 1.0, pa, pb, 0.0, C, m, batch, m * n)
+    ref = torch.full((batch, n, m), 7.0, dtype=torch.float32, device=dev)
+    kt = (k + 31) // 32
+    rb_bytes = kt * TERMS[policy] * 1024            # one 16-row block of a packed operand
+    blk = 512
+    for e in range(batch):
+        for c0 in range(0, n, blk):
+            cols = min(blk, n - c0)
+            pbe = pb[e * per_b + (c0 // 16) * rb_bytes:(e + 1) * per_b]
+            tc.gemm_packed(policy, m, cols, k, 1.0, pa[e * per_a:(e + 1) * per_a], pbe, 0.0,
+                           ref[e, c0:c0 + cols], m)
+    torch.cuda.synchronize()
+    assert torch.equal(C, ref)
+    if m * n * k <= 4096 * 4096 * 96:
+        _fp64_check(orc, A[0], B[0], C[0], policy)
+
+
+def test_one_workgroup_per_item_for_long_k(tc, orc, dev):
+    """Many tiles with 64 or more stages each and a single entry: one workgroup per item.
+    Rows of A in two halves give the same bits."""
+    m, n, k = 4096, 4096, 2048 + 32
+    A = _uniform((1, m, k), 7, dev)
+    B = _uniform((1, n, k), 8, dev)
+    pa, _ = _pack(tc, 0, A, dev)
+    pb, _ = _pack(tc, 0, B, dev)
+    C = torch.zeros((n, m), dtype=torch.float32, device=dev)
+    tc.gemm_packed(0, m, n, k, 1.0, pa, pb, 0.0, C, m)
+    ref = torch.zeros((n, m), dtype=torch.float32, device=dev)
+    half = m // 2
+    rb_bytes = ((k + 31) // 32) * 2 * 1024
+    for r0 in (0, half):
+        # rows r0 .. r0+half of C: the column-major slab starts at element r0 of every column
+        tc.gemm_packed(0, half, n, k, 1.0, pa[(r0 // 16) * rb_bytes:], pb, 0.0,
+                       ref.view(-1)[r0:], m)
+    torch.cuda.synchronize()
+    assert torch.equal(C, ref)
