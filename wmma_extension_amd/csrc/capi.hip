@@ -247,7 +247,9 @@ template <class MT, int TERMS, bool RN> int gemm_by_size(const GemmArgs &g) {
       ceil_div(g.m, 256) * ceil_div(g.n, 128) * g.batch * z;
   const long long mid =
       ceil_div(g.m, 128) * ceil_div(g.n, 128) * g.batch * z;
-  if constexpr (TERMS <= 2) {
+  // (not with the separate fp32 adds of RN: their temporaries do not fit the
+  // register file next to the large tile's accumulators)
+  if constexpr (TERMS <= 2 && !RN) {
     if (big >= cus) {
       // time in units of one 128x128 tile: rounds * tile cost
       const double t_big = static_cast<double>(ceil_div(big, cus)) * 2.0;
