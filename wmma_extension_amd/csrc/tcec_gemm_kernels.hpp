@@ -205,7 +205,8 @@ __global__ void __launch_bounds__(256)
 //
 // ABLATE (tuning only, 0 in the library): bit 0 drops the global->LDS requests
 // of the main loop, bit 1 its LDS reads, bit 2 its barriers, bit 3 the wait
-// for the requests, bit 4 the MFMAs, bit 5 makes every block read tile (0,0).
+// for the requests, bit 4 the MFMAs, bit 5 makes every block read tile (0,0),
+// bit 7 drops every fourth request, bit 8 every fourth LDS read.
 // Results are then wrong; the variants exist to time the remaining parts.
 // --------------------------------------------------------------------------
 template <class MT, int TERMS, int BM, int BN, int WGM, int WGN, int NSTAGE,
@@ -584,7 +585,8 @@ __global__ void __launch_bounds__(WGM *WGN * 64)
       constexpr int qlo = (n * CPW + NMFMA - 1) / NMFMA;
       constexpr int qhi = ((n + 1) * CPW + NMFMA - 1) / NMFMA;
       static_for<qlo, (qhi < CPW ? qhi : CPW)>([&](auto Q) {
-        if constexpr ((ABLATE & 1) == 0)
+        if constexpr ((ABLATE & 1) == 0 &&
+                      !((ABLATE & 128) != 0 && decltype(Q)::value % 4 == 3))
           issue_chunk(w_base, Q);
         __builtin_amdgcn_sched_barrier(0);
       });
@@ -598,7 +600,8 @@ __global__ void __launch_bounds__(WGM *WGN * 64)
       constexpr int lo = n == 0 ? 0 : reads_due(n, SPAN, NFRAG);
       constexpr int hi = n + 1 == NMFMA ? NFRAG : reads_due(n + 1, SPAN, NFRAG);
       static_for<lo, hi>([&](auto R_) {
-        if constexpr ((ABLATE & 2) == 0)
+        if constexpr ((ABLATE & 2) == 0 &&
+                      !((ABLATE & 256) != 0 && decltype(R_)::value % 4 == 3))
           read_frag(nxt, r_base, R_);
         __builtin_amdgcn_sched_barrier(0);
       });
