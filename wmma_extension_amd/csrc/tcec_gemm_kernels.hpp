@@ -432,10 +432,11 @@ __global__ void __launch_bounds__(WGM *WGN * 64)
     constexpr int q = decltype(Q)::value;
     // first chunk of the row block; the immediate offset of the instruction
     // moves the global and the LDS address alike to the chunk of term q%TERMS
-    // (redefined in place: the address is then formed here, as the
-    // instruction's scalar base + 32-bit lane offset, and not hoisted into
-    // vector registers)
-    asm volatile("" : "+s"(gsrc[q / CH_PER_RB]), "+v"(lane_off));
+    // (the lane offset is redefined in place once per row block: the address
+    // is then formed here, as the instruction's scalar base + 32-bit lane
+    // offset, and not hoisted into vector register pairs)
+    if constexpr (q % CH_PER_RB == 0)
+      asm volatile("" : "+v"(lane_off));
     __builtin_amdgcn_global_load_lds(
         reinterpret_cast<const __attribute__((address_space(1))) char *>(
             gsrc[q / CH_PER_RB]) +
