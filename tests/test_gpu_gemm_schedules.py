@@ -110,3 +110,32 @@ def test_one_workgroup_per_item_for_long_k(tc, orc, dev):
                        ref.view(-1)[r0:], m)
     torch.cuda.synchronize()
     assert torch.equal(C, ref)
+
+
+@pytest.mark.parametrize("policy", [0, 2])
+def test_pointer_arrays_through_packed_operands_and_xcd_owned_entries(tc, orc, dev, policy):
+    """wmmae_tcec_sgemm_batched (device arrays of matrix pointers, test/tcec/batch_gemm.cu:433-443)
+    on a batch that goes through packed operands (the round-to-nearest flag always does) with
+    more items than resident workgroups: same bits as the strided call on a copy of the same
+    matrices, FP64 agreement on one entry."""
+    batch, m, n, k = 10, 1024, 896, 96
+    A = _uniform((batch, m, k), 31, dev)
+    B = _uniform((batch, n, k), 32, dev)
+    # entries scattered in memory, in another order than the strided copy
+    As = [A[e].clone() for e in reversed(range(batch))][::-1]
+    Bs = [B[e].clone() for e in range(batch)]
+    Cs = [torch.full((n, m), 2.0, dtype=torch.float32, device=dev) for _ in range(batch)]
+    pa = torch.tensor([t.data_ptr() for t in As], dtype=torch.int64, device=dev)
+    pb = torch.tensor([t.data_ptr() for t in Bs], dtype=torch.int64, device=dev)
+    pc = torch.tensor([t.data_ptr() for t in Cs], dtype=torch.int64, device=dev)
+    ws = torch.empty(tc.workspace_bytes(m, n, k, batch, policy), dtype=torch.uint8, device=dev)
+    tc.sgemm_batched("T", "N", m, n, k, 0.5, pa, k, pb, k, 1.5, pc, m, batch, policy, 1, ws)
+    C = torch.full((batch, n, m), 2.0, dtype=torch.float32, device=dev)
+    tc.sgemm_strided_batched("T", "N", m, n, k, 0.5, A, k, m * k, B, k, n * k, 1.5, C, m, m * n,
+                             batch, policy, 1, ws)
+    torch.cuda.synchronize()
+    for e in range(batch):
+        assert torch.equal(Cs[e], C[e]), e
+    e = 7
+    ref = 0.5 * orc.gemm_f64(A[e].cpu().numpy(), B[e].cpu().numpy().T) + 3.0
+    assert orc.max_rel_err(C[e].cpu().numpy().T, ref) < 4e-6
