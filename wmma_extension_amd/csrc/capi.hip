@@ -234,12 +234,11 @@ int launch_gemm(const GemmArgs &g) {
   return st;
 }
 
-// Tile choice: the large tile when it still gives every compute unit work,
-// otherwise smaller tiles so that more blocks exist.
-// Tile configuration: the 256x128 tile moves the fewest operand bytes per flop
-// and is the choice whenever its tiles fill the chip evenly; the grid runs in
-// rounds of one tile per compute unit, so when the last round would be mostly
-// empty the 128x128 tile (about 5 % slower per flop) can still finish sooner.
+// Tile choice: the 256x128 tile moves the fewest operand bytes per flop and is
+// the choice whenever its tiles fill the chip evenly; the tiles run in rounds
+// of one per compute unit, so when the last round would be mostly empty the
+// 128x128 tile (about 5 % slower per flop) can still finish sooner; 64x64
+// tiles for problems too small to give the larger ones work.
 template <class MT, int TERMS, bool RN> int gemm_by_size(const GemmArgs &g) {
   const int cus = device_cus();
   const long long z = g.partial != nullptr ? g.splits : 1;
