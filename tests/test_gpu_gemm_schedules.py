@@ -139,3 +139,37 @@ def test_pointer_arrays_through_packed_operands_and_xcd_owned_entries(tc, orc, d
     e = 7
     ref = 0.5 * orc.gemm_f64(A[e].cpu().numpy(), B[e].cpu().numpy().T) + 3.0
     assert orc.max_rel_err(C[e].cpu().numpy().T, ref) < 4e-6
+
+
+def test_random_shapes_packed_path_and_driver_choice_agree(tc, orc, dev):
+    """120 seeded problems (1..5000 rows and columns, 1..3000 of k, 1..40 entries, all five
+    policies): pack + gemm_packed and the driver's own choice of path give the same bits,
+    and both stay within the policy's error bound of an FP64 product computed on the GPU."""
+    import random
+    rnd = random.Random(20240)
+    bound = {0: 4e-6, 2: 4e-6, 1: 3e-3, 3: 3e-4, 4: 3e-2}
+    for case in range(120):
+        policy = rnd.choice([0, 0, 2, 2, 1, 3, 4])
+        batch = rnd.choice([1, 1, 1, 2, 3, 9, 17, 40])
+        big = rnd.random() < 0.5
+        m = rnd.randint(1, 5000 if big else 700)
+        n = rnd.randint(1, 5000 if big else 700)
+        k = rnd.randint(1, 700 if batch * m * n > 4e6 else 3000)
+        while batch * (m * k + n * k + m * n) * 4 > 1.0e9:
+            batch = max(1, batch // 2)
+            m = max(1, m // 2)
+        A = _uniform((batch, m, k), 1000 + case, dev)
+        B = _uniform((batch, n, k), 2000 + case, dev)
+        ref = torch.matmul(A.double(), B.double().transpose(1, 2))
+        scale = ref.abs().amax(dim=(1, 2)).clamp_min(1e-30)
+        pa, _ = _pack(tc, policy, A, dev)
+        pb, _ = _pack(tc, policy, B, dev)
+        C = torch.full((batch, n, m), float("nan"), device=dev)
+        tc.gemm_packed(policy, m, n, k, 1.0, pa, pb, 0.0, C, m, batch, m * n)
+        C2 = torch.full((batch, n, m), float("nan"), device=dev)
+        tc.sgemm_strided_batched("T", "N", m, n, k, 1.0, A, k, m * k, B, k, n * k, 0.0, C2, m, m * n,
+                                 batch, policy)
+        err = ((C.transpose(1, 2).double() - ref).abs().amax(dim=(1, 2)) / scale).max().item()
+        tag = (case, policy, batch, m, n, k)
+        assert err < bound[policy], tag
+        assert torch.equal(C, C2), tag
