@@ -104,3 +104,22 @@ def test_config5b_k_heavy(tc, orc, dev):
     assert err <= 2 * e32, (err, e32)
     # the sequential fp32 loop loses ~sqrt(K) ulps here; TCEC stays well below it
     assert err < e32
+
+
+def test_reference_harness_command_prints_the_reference_csv(tc, orc, dev):
+    """python -m wmma_extension_amd.batch_gemm: the reference harness's loop, inputs, residual
+    and output line (test/tcec/batch_gemm.cu:505-520, 559-575, 604, 657) on a small grid."""
+    import io
+    from wmma_extension_amd import batch_gemm
+    out = io.StringIO()
+    batch_gemm.main(["--m", "512", "--k", "128", "1024", "--batch", "6", "--count", "3"], out)
+    lines = out.getvalue().strip().split("\n")
+    assert lines[0] == "mode,m,n,k,batch_size,residual,throughput"
+    assert len(lines) == 3
+    for line, k in zip(lines[1:], (128, 1024)):
+        f = line.split(",")
+        assert f[:5] == ["wmmae", "512", "512", str(k), "6"]
+        # all-positive ramps: the fp32 accumulators' error grows with k (1e-7 at k=128,
+        # 6e-7 at k=1024 measured; plain fp32 accumulation is no better)
+        assert 0.0 <= float(f[5]) < 2e-6
+        assert float(f[6]) > 0.0
