@@ -83,12 +83,20 @@ int wmmae_query(int what, long long *out);
  * from wmmae_tcec_sgemm_workspace_bytes.  workspace == NULL lets the library
  * take it from the stream-ordered allocator (hipMallocAsync / hipFreeAsync on
  * `stream`).  Products whose operands are reused by few tiles (m, n <= 512, or
- * larger with a short k; flags == 0, no K slices) are split inside the GEMM
+ * larger with a short k; no K slices) are split inside the GEMM
  * kernel (as the reference's bgemm_kernel splits at fragment load,
  * batch_gemm.cu:196-386): they use no workspace, allocate nothing and ignore
  * the workspace arguments.  Both paths give the same bits. */
 int wmmae_tcec_sgemm_workspace_bytes(int m, int n, int k, int batch, int policy,
                                      size_t *bytes);
+
+/* Which of these the GEMM entry points take for a shape (no counterpart in the
+ * reference, whose harness fixes one kernel configuration at compile time,
+ * batch_gemm.cu:408-431, 659): *path = 0 the single kernel that splits the
+ * operands on the fly (no workspace), 1 packed operands in the workspace,
+ * 2 packed operands and K slices (when the workspace has room for them). */
+int wmmae_tcec_sgemm_path(int m, int n, int k, int batch, int policy, int flags,
+                          int *path);
 
 int wmmae_tcec_sgemm(char transa, char transb, int m, int n, int k,
                      const float *alpha, const float *A, int lda,

@@ -168,3 +168,22 @@ def test_primitive_entries_reject_bad_arguments_on_the_host(h):
     assert h.wmmae_primitive_mma(0, 0, None, p, p, p, 0, 0, 0, 0, None) == -2
     assert h.wmmae_foreach_ec(p, None, p, None) == -2
     assert h.wmmae_gevm(None, p, p, None) == -2
+
+
+def test_sgemm_path_query_on_the_baseline_workloads():
+    """wmmae_tcec_sgemm_path needs no GPU: the batched 256^3 products take the single kernel,
+    4096^3 and 16384^3 packed operands, the K-heavy product K slices; bad arguments are
+    turned down."""
+    import ctypes
+    from wmma_extension_amd import _lib
+    h = _lib.lib()
+    out = ctypes.c_int(-1)
+    for args, want in (((256, 256, 256, 1024, 0, 0), 0), ((4096, 4096, 4096, 1, 0, 0), 1),
+                       ((16384, 16384, 16384, 1, 2, 0), 1), ((1024, 1024, 262144, 1, 0, 0), 2),
+                       ((512, 512, 1024, 256, 0, 1), 0), ((512, 512, 1024, 256, 1, 1), 1)):
+        assert h.wmmae_tcec_sgemm_path(*args, ctypes.byref(out)) == 0
+        assert out.value == want, args
+    assert h.wmmae_tcec_sgemm_path(16, 16, 16, 1, 0, 0, None) == -2
+    assert h.wmmae_tcec_sgemm_path(-1, 16, 16, 1, 0, 0, ctypes.byref(out)) == -1
+    assert h.wmmae_tcec_sgemm_path(16, 16, 16, 1, 9, 0, ctypes.byref(out)) == -1
+    assert h.wmmae_tcec_sgemm_path(16, 16, 16, 1, 0, 2, ctypes.byref(out)) == -1

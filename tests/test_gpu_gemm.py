@@ -116,17 +116,19 @@ def test_sgemm_k_zero_and_workspace(tc, orc, dev):
     B = rng.uniform(-1, 1, (64, 64)).astype(np.float32)
     ws = torch.empty(tc.workspace_bytes(64, 64, 64), dtype=torch.uint8, device=dev)
     assert np.array_equal(_gemm(tc, dev, A, B, 0, workspace=ws), _gemm(tc, dev, A, B, 0))
-    # a product that goes through the packed operands (the round-to-nearest flag always
-    # does) needs room for them
-    A = rng.uniform(-1, 1, (1536, 1024)).astype(np.float32)
-    B = rng.uniform(-1, 1, (1024, 1024)).astype(np.float32)
-    ws = torch.empty(tc.workspace_bytes(1536, 1024, 1024), dtype=torch.uint8, device=dev)
-    assert np.array_equal(_gemm(tc, dev, A, B, 0, flags=1, workspace=ws), _gemm(tc, dev, A, B, 0, flags=1))
-    small = torch.empty(16, dtype=torch.uint8, device=dev)
+    # products that go through packed operands (a K-heavy one with K slices, a large one
+    # without) need room for them
     from wmma_extension_amd._lib import WmmaeError
-    with pytest.raises(WmmaeError) as e:
-        _gemm(tc, dev, A, B, 0, flags=1, workspace=small)
-    assert e.value.status == -5
+    small = torch.empty(16, dtype=torch.uint8, device=dev)
+    for (m, n, k), path in (((128, 128, 8192), tc.PATH_PACKED_SPLIT_K), ((3072, 2048, 2048), tc.PATH_PACKED)):
+        assert tc.sgemm_path(m, n, k) == path
+        A = rng.uniform(-1, 1, (m, k)).astype(np.float32)
+        B = rng.uniform(-1, 1, (k, n)).astype(np.float32)
+        ws = torch.empty(tc.workspace_bytes(m, n, k), dtype=torch.uint8, device=dev)
+        assert np.array_equal(_gemm(tc, dev, A, B, 0, workspace=ws), _gemm(tc, dev, A, B, 0))
+        with pytest.raises(WmmaeError) as e:
+            _gemm(tc, dev, A, B, 0, workspace=small)
+        assert e.value.status == -5
 
 
 @pytest.mark.parametrize("policy", [0, 2])
@@ -221,15 +223,18 @@ def test_pack_then_gemm_reuses_operands(tc, orc, dev):
 @pytest.mark.parametrize("trans", ["TN", "NT"])
 def test_small_products_split_in_kernel_match_packed_path(tc, orc, dev, policy, trans):
     """Products up to 512 x 512 are split inside the GEMM kernel (no packed copy in
-    memory); the result is bit for bit that of pack + gemm_packed."""
+    memory); the result is bit for bit that of pack + gemm_packed, also with the leading
+    product accumulated outside the matrix core (policies that have that variant)."""
     rng = np.random.default_rng(91 + policy)
+    flags = 1 if policy in (0, 2) and trans == "NT" else 0
     for m, n, k in ((64, 64, 64), (40, 24, 50), (256, 256, 256), (500, 130, 77), (512, 512, 33)):
+        assert tc.sgemm_path(m, n, k, 1, policy, flags) == tc.PATH_FUSED
         A = rng.standard_normal((m, k)).astype(np.float32)
         B = rng.standard_normal((k, n)).astype(np.float32)
         C0 = rng.standard_normal((m, n)).astype(np.float32)
         for ld_pad in (0, 1):
             fused = _gemm(tc, dev, A, B, policy, alpha=1.25, beta=-0.5, C=C0, ta=trans[0], tb=trans[1],
-                          ld_pad=ld_pad)
+                          ld_pad=ld_pad, flags=flags)
             dA = torch.from_numpy(A).to(dev)
             dB = torch.from_numpy(np.ascontiguousarray(B.T)).to(dev)
             pa = torch.empty(tc.pack_bytes(m, k, 1, policy), dtype=torch.uint8, device=dev)
@@ -237,7 +242,7 @@ def test_small_products_split_in_kernel_match_packed_path(tc, orc, dev, policy, 
             tc.pack(policy, m, k, dA, k, 1, pa)
             tc.pack(policy, n, k, dB, k, 1, pb)
             dC = torch.from_numpy(np.ascontiguousarray(C0.T)).to(dev)
-            tc.gemm_packed(policy, m, n, k, 1.25, pa, pb, -0.5, dC, m)
+            tc.gemm_packed(policy, m, n, k, 1.25, pa, pb, -0.5, dC, m, flags=flags)
             torch.cuda.synchronize()
             assert np.array_equal(dC.cpu().numpy().T, fused), (m, n, k, ld_pad)
         _check(orc, fused, A, B, policy, C=C0, alpha=1.25, beta=-0.5)

@@ -115,10 +115,11 @@ def test_one_workgroup_per_item_for_long_k(tc, orc, dev):
 @pytest.mark.parametrize("policy", [0, 2])
 def test_pointer_arrays_through_packed_operands_and_xcd_owned_entries(tc, orc, dev, policy):
     """wmmae_tcec_sgemm_batched (device arrays of matrix pointers, test/tcec/batch_gemm.cu:433-443)
-    on a batch that goes through packed operands (the round-to-nearest flag always does) with
-    more items than resident workgroups: same bits as the strided call on a copy of the same
-    matrices, FP64 agreement on one entry."""
-    batch, m, n, k = 10, 1024, 896, 96
+    on a batch that goes through packed operands with more items than resident workgroups,
+    leading product accumulated outside the matrix core: same bits as the strided call on a
+    copy of the same matrices, FP64 agreement on one entry."""
+    batch, m, n, k = 10, 2048, 1792, 512
+    assert tc.sgemm_path(m, n, k, batch, policy, 1) == tc.PATH_PACKED
     A = _uniform((batch, m, k), 31, dev)
     B = _uniform((batch, n, k), 32, dev)
     # entries scattered in memory, in another order than the strided copy

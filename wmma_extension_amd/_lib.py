@@ -29,6 +29,7 @@ EXPORTS = [
     "wmmae_status_string",
     "wmmae_query",
     "wmmae_tcec_sgemm_workspace_bytes",
+    "wmmae_tcec_sgemm_path",
     "wmmae_tcec_sgemm",
     "wmmae_tcec_sgemm_strided_batched",
     "wmmae_tcec_sgemm_batched",
@@ -82,6 +83,7 @@ _SIGNATURES = {
     "wmmae_status_string": (_c.c_char_p, [_i]),
     "wmmae_query": (_i, [_i, _c.POINTER(_ll)]),
     "wmmae_tcec_sgemm_workspace_bytes": (_i, [_i, _i, _i, _i, _i, _c.POINTER(_sz)]),
+    "wmmae_tcec_sgemm_path": (_i, [_i, _i, _i, _i, _i, _i, _c.POINTER(_i)]),
     "wmmae_tcec_sgemm": (_i, [_c.c_char, _c.c_char, _i, _i, _i, _fp, _vp, _i, _vp, _i, _fp,
                               _vp, _i, _i, _i, _vp, _sz, _vp]),
     "wmmae_tcec_sgemm_strided_batched": (_i, [_c.c_char, _c.c_char, _i, _i, _i, _fp, _vp, _i, _ll,

@@ -348,9 +348,13 @@ int fused_dispatch(const int policy, const FusedArgs &f) {
 // from rates measured on MI355X; K-heavy single products that want K slices
 // stay on the packed path.
 inline bool use_fused(const int m, const int n, const int k, const int batch,
-                      const int flags, const int terms) {
-  if (k <= 0 || (flags & WMMAE_FLAG_RN_MAIN) != 0 ||
-      choose_splits(m, n, k, batch) != 1)
+                      const int flags, const int terms, const int policy) {
+  // (the round-to-nearest flag with a policy that has no such variant is
+  // turned down by the packed path's dispatch)
+  const bool rn_unsupported =
+      (flags & WMMAE_FLAG_RN_MAIN) != 0 && policy != WMMAE_POLICY_F16_EC &&
+      policy != WMMAE_POLICY_BF16X3_EC;
+  if (k <= 0 || rn_unsupported || choose_splits(m, n, k, batch) != 1)
     return false;
   if (m <= 512 && n <= 512)
     return true;
@@ -563,7 +567,7 @@ int sgemm_impl(const char transa, const char transb, const int m, const int n,
       ldc < m)
     return WMMAE_STATUS_BAD_LEADING_DIM;
 
-  if (use_fused(m, n, k, batch, flags, p.terms)) {
+  if (use_fused(m, n, k, batch, flags, p.terms, policy)) {
     if (batch > (1 << 26)) // tile indices are 32-bit
       return WMMAE_STATUS_NOT_SUPPORTED;
     FusedArgs f;
@@ -595,6 +599,7 @@ int sgemm_impl(const char transa, const char transb, const int m, const int n,
               (b_ptrs != nullptr || (aligned16(B) && stride_b % 4 == 0));
     q.vec_store = (ldc % 4 == 0) &&
                   (c_ptrs != nullptr || (aligned16(C) && stride_c % 4 == 0));
+    q.rn_main = (flags & WMMAE_FLAG_RN_MAIN) != 0;
     q.alpha = *alpha;
     q.beta = *beta;
     q.inv_scale = p.inv_scale;
@@ -687,6 +692,25 @@ int wmmae_tcec_gemm_packed_workspace_bytes(const int policy, const int m,
                          ? 1
                          : choose_splits(m, n, k, batch);
   *bytes = splits > 1 ? static_cast<size_t>(splits) * batch * m * n * 4u : 0;
+  return WMMAE_STATUS_SUCCESS;
+}
+
+int wmmae_tcec_sgemm_path(const int m, const int n, const int k,
+                          const int batch, const int policy, const int flags,
+                          int *const path) {
+  PolicyInfo p;
+  if (path == nullptr)
+    return WMMAE_STATUS_NULL_POINTER;
+  if (m < 0 || n < 0 || k < 0 || batch < 0 || !policy_info(policy, p) ||
+      (flags & ~WMMAE_FLAG_RN_MAIN) != 0)
+    return WMMAE_STATUS_INVALID_VALUE;
+  if (use_fused(m, n, k, batch, flags, p.terms, policy))
+    *path = 0;
+  else
+    *path = (m > 0 && n > 0 && k > 0 && batch > 0 &&
+             choose_splits(m, n, k, batch) > 1)
+                ? 2
+                : 1;
   return WMMAE_STATUS_SUCCESS;
 }
 

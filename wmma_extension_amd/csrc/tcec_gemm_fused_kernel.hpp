@@ -67,6 +67,9 @@ struct FusedParams {
   // entries are checked by the kernel)
   int vec_a, vec_b;
   int vec_store;
+  // accumulate the leading product with fp32 adds outside the matrix core
+  // (tcec_gemm_kernel's RN_MAIN; the reference's mma_rn_sync)
+  int rn_main;
   float alpha, beta, inv_scale;
 };
 
@@ -516,7 +519,16 @@ __global__ void __launch_bounds__(64 * NW)
             sweep(acc_err, 1, 0);
             sweep(acc_err, 0, 1);
           }
-          sweep(acc_main, 0, 0);
+          if (p.rn_main) {
+#pragma unroll
+            for (int i = 0; i < MT_; i++)
+#pragma unroll
+              for (int j = 0; j < NT_; j++)
+                acc_main[i][j] +=
+                    mfma(a[0][i], b[0][j], f32x4{0.f, 0.f, 0.f, 0.f});
+          } else {
+            sweep(acc_main, 0, 0);
+          }
           // stage s+1 into the registers the MFMAs above have been fed from
           read_frags(buf ^ 1);
         };

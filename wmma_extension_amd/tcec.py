@@ -61,6 +61,17 @@ def workspace_bytes(m, n, k, batch=1, policy=Policy.F16_EC):
     return out.value
 
 
+PATH_FUSED, PATH_PACKED, PATH_PACKED_SPLIT_K = 0, 1, 2
+
+
+def sgemm_path(m, n, k, batch=1, policy=Policy.F16_EC, flags=0):
+    """Which path the GEMM entry points take for this shape (PATH_* above)."""
+    out = ctypes.c_int(-1)
+    _lib.check(_lib.lib().wmmae_tcec_sgemm_path(m, n, k, batch, int(policy), flags,
+                                                ctypes.byref(out)), "wmmae_tcec_sgemm_path")
+    return out.value
+
+
 def pack_bytes(rows, k, batch=1, policy=Policy.F16_EC):
     out = ctypes.c_size_t(0)
     _lib.check(_lib.lib().wmmae_tcec_pack_bytes(rows, k, batch, int(policy), ctypes.byref(out)),
