@@ -7,6 +7,7 @@
 #include <wmmae_tcec.h>
 
 #include <algorithm>
+#include <atomic>
 #include <hip/hip_runtime.h>
 
 namespace {
@@ -139,6 +140,26 @@ inline int device_cus() {
   return cached;
 }
 
+// A kernel that wants more dynamic LDS than the default limit has to be told
+// so once per device; `done` is the calling site's own bit mask of devices
+// (one static per kernel instantiation), so later launches skip the driver
+// call.
+inline hipError_t allow_dynamic_lds(const void *const kernel, const int bytes,
+                                    std::atomic<unsigned long long> &done) {
+  int dev = 0;
+  hipError_t e = hipGetDevice(&dev);
+  if (e != hipSuccess)
+    return e;
+  const bool tracked = dev >= 0 && dev < 64;
+  if (tracked && ((done.load(std::memory_order_relaxed) >> dev) & 1ull) != 0)
+    return hipSuccess;
+  e = hipFuncSetAttribute(kernel, hipFuncAttributeMaxDynamicSharedMemorySize,
+                          bytes);
+  if (e == hipSuccess && tracked)
+    done.fetch_or(1ull << dev, std::memory_order_relaxed);
+  return e;
+}
+
 // Number of K slices: only when the output tiles cannot fill the chip and
 // every slice still has a long K loop.
 inline int choose_splits(const int m, const int n, const int k,
@@ -170,9 +191,9 @@ int launch_gemm(const GemmArgs &g) {
   using Cfg = wmmae_gemm::GemmConfig<MT, TERMS, BM, BN, WGM, WGN, NSTAGE, RN>;
   auto kernel =
       wmmae_gemm::tcec_gemm_kernel<MT, TERMS, BM, BN, WGM, WGN, NSTAGE, RN>;
-  WMMAE_HIP_TRY(hipFuncSetAttribute(reinterpret_cast<const void *>(kernel),
-                                    hipFuncAttributeMaxDynamicSharedMemorySize,
-                                    Cfg::LDS_BYTES));
+  static std::atomic<unsigned long long> lds_allowed{0};
+  WMMAE_HIP_TRY(allow_dynamic_lds(reinterpret_cast<const void *>(kernel),
+                                  Cfg::LDS_BYTES, lds_allowed));
   const int tiles_m = static_cast<int>(ceil_div(g.m, BM));
   const int tiles_n = static_cast<int>(ceil_div(g.n, BN));
   const int KT = packed_k_tiles(g.k);
@@ -293,9 +314,9 @@ struct FusedArgs {
 template <class T, int TERMS, int BM, int BN> int launch_fused(FusedArgs f) {
   using Cfg = wmmae_gemm::FusedConfig<TERMS, BM, BN>;
   auto kernel = wmmae_gemm::tcec_gemm_fused_kernel<T, TERMS, BM, BN>;
-  WMMAE_HIP_TRY(hipFuncSetAttribute(reinterpret_cast<const void *>(kernel),
-                                    hipFuncAttributeMaxDynamicSharedMemorySize,
-                                    Cfg::LDS_BYTES));
+  static std::atomic<unsigned long long> lds_allowed{0};
+  WMMAE_HIP_TRY(allow_dynamic_lds(reinterpret_cast<const void *>(kernel),
+                                  Cfg::LDS_BYTES, lds_allowed));
   wmmae_gemm::FusedParams &p = f.p;
   p.tiles_m = static_cast<int>(ceil_div(p.M, BM));
   p.tiles_per_batch = p.tiles_m * static_cast<int>(ceil_div(p.N, BN));
