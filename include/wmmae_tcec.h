@@ -138,10 +138,12 @@ int wmmae_tcec_pack(int policy, int rows, int k, const float *X,
                     long long row_stride, long long k_stride,
                     long long batch_stride, int batch, void *packed,
                     size_t packed_bytes, void *stream);
-/* workspace (optional, may be NULL): room for split-K slices, used when the
- * output has too few tiles to fill the chip (K-heavy shapes); size from
- * wmmae_tcec_gemm_packed_workspace_bytes (0 when no split would be made).
- * Without it the product runs unsplit. */
+/* workspace (optional, may be NULL): room for K slices, used when the output
+ * has too few tiles to fill the chip (K-heavy shapes: every tile is cut), or
+ * when its tiles leave the last round over the compute units mostly empty
+ * (single large products: only that round's tiles are cut); size from
+ * wmmae_tcec_gemm_packed_workspace_bytes (0 when no cut would be made).
+ * Without it the product runs uncut. */
 int wmmae_tcec_gemm_packed_workspace_bytes(int policy, int m, int n, int k,
                                            int batch, size_t *bytes);
 int wmmae_tcec_gemm_packed(int policy, int m, int n, int k, const float *alpha,

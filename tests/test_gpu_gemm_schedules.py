@@ -174,3 +174,36 @@ def test_random_shapes_packed_path_and_driver_choice_agree(tc, orc, dev):
         tag = (case, policy, batch, m, n, k)
         assert err < bound[policy], tag
         assert torch.equal(C, C2), tag
+
+
+@pytest.mark.parametrize("policy", [0, 2])
+@pytest.mark.parametrize("shape", [(5120, 5120, 2304), (2304, 2304, 4096), (4000, 4500, 2100)])
+def test_k_slices_for_the_last_round_of_tiles(tc, orc, dev, policy, shape):
+    """Tile counts that leave the last round over the compute units mostly empty: with room
+    in the workspace the tiles of that round are cut along K and folded afterwards.  The
+    tiles of the whole rounds keep their bits, the cut ones agree with the uncut run to
+    rounding of the partial sums, and both agree with FP64."""
+    m, n, k = shape
+    assert tc.gemm_packed_workspace_bytes(policy, m, n, k) > 0
+    A = _uniform((1, m, k), 61, dev)
+    B = _uniform((1, n, k), 62, dev)
+    C0 = _uniform((n, m), 63, dev)
+    pa, _ = _pack(tc, policy, A, dev)
+    pb, _ = _pack(tc, policy, B, dev)
+    plain = C0.clone()
+    tc.gemm_packed(policy, m, n, k, 0.75, pa, pb, 0.5, plain, m)              # no workspace: uncut
+    ws = torch.empty(tc.gemm_packed_workspace_bytes(policy, m, n, k), dtype=torch.uint8, device=dev)
+    cut = C0.clone()
+    tc.gemm_packed(policy, m, n, k, 0.75, pa, pb, 0.5, cut, m, workspace=ws)
+    again = C0.clone()
+    tc.gemm_packed(policy, m, n, k, 0.75, pa, pb, 0.5, again, m, workspace=ws)
+    torch.cuda.synchronize()
+    assert torch.equal(cut, again)                                            # deterministic
+    differ = (cut != plain)
+    frac = differ.float().mean().item()
+    assert 0.0 < frac < 0.5                      # only the last round's tiles were cut
+    ref = 0.75 * torch.matmul(A[0].double(), B[0].double().T).T + 0.5 * C0.double()
+    scale = ref.abs().max()
+    assert ((cut.double() - ref).abs().max() / scale).item() < 4e-6
+    assert ((plain.double() - ref).abs().max() / scale).item() < 4e-6
+    assert ((cut - plain).abs().max().double() / scale).item() < 1e-6

@@ -124,6 +124,10 @@ struct GemmArgs {
   float *const *c_ptrs; // device array of C pointers, or nullptr
   float *partial;  // split-K slices, or nullptr
   int splits;      // >= 1
+  // room for the K slices of the tiles of a partly empty last round (used
+  // only without split-K), or nullptr
+  float *tail_ws;
+  size_t tail_ws_bytes;
   hipStream_t stream;
 };
 
@@ -178,6 +182,41 @@ inline int choose_splits(const int m, const int n, const int k,
   return s < 1 ? 1 : static_cast<int>(s);
 }
 
+// K slices for the tiles of the last round only.  `tiles` output tiles run in
+// rounds of `resident` (one workgroup per item, long K loops); when the last
+// round is less than half full its tiles are cut into `slices` K slices of at
+// least 32 stages each, so that the round takes about 1/slices of a tile's
+// time (plus the pass that folds the slices).  slices == 1: not worth it.
+struct TailPlan {
+  long long full = 0, tail = 0; // tiles in whole rounds, tiles in the last
+  int slices = 1, stages = 0;   // K slices of a tail tile, stages per slice
+};
+inline TailPlan plan_tail(const long long tiles, const long long resident,
+                          const int KT) {
+  TailPlan t;
+  t.full = tiles / resident * resident;
+  t.tail = tiles - t.full;
+  if (t.full == 0 || t.tail == 0 || t.tail * 2 > resident || KT < 64)
+    return t;
+  long long s = std::min<long long>({resident / t.tail, KT / 32, 16});
+  if (s < 2)
+    return t;
+  t.stages = static_cast<int>(ceil_div(KT, s));
+  t.slices = static_cast<int>(ceil_div(KT, t.stages));
+  return t;
+}
+// Time of `tiles` tiles in units of one tile, with and without that plan.
+inline double rounds_cost(const long long tiles, const long long resident,
+                          const int KT, const bool tail_allowed) {
+  const TailPlan t = plan_tail(tiles, resident, KT);
+  const double full_rounds = static_cast<double>(t.full / resident);
+  if (t.tail == 0)
+    return full_rounds;
+  if (!tail_allowed || t.slices < 2)
+    return full_rounds + 1.0;
+  return full_rounds + 1.0 / t.slices + 0.2; // slices, pipeline refills, fold
+}
+
 // Deepest LDS ring (at most 4 stages) that fits the 160 KiB of a compute unit.
 constexpr int ring_depth(const int bm, const int bn, const int terms) {
   const int stage_bytes = (bm / 16 + bn / 16) * terms * 1024;
@@ -228,11 +267,28 @@ int launch_gemm(const GemmArgs &g) {
   const long long resident = static_cast<long long>(device_cus()) * per_cu;
   int grid = static_cast<int>(std::min(items, resident));
   int entry_per_xcd = 0;
+  unsigned tail_begin = 0xffffffffu; // no tail slices
+  TailPlan tail;
   if (items > resident) {
-    if (g.batch >= 8 && zdim == 1 && resident % 8 == 0)
+    if (g.batch >= 8 && zdim == 1 && resident % 8 == 0) {
       entry_per_xcd = 1;
-    else if (split_stages >= 64)
+    } else if (split_stages >= 64) {
       grid = static_cast<int>(items);
+      // one entry, no split-K, room for the slices: the tiles of a partly
+      // empty last round are cut along K
+      if (g.batch == 1 && zdim == 1 && g.c_ptrs == nullptr &&
+          g.tail_ws != nullptr) {
+        tail = plan_tail(items, resident, KT);
+        const size_t need =
+            static_cast<size_t>(tail.slices) * tail.tail * BM * BN * 4u;
+        if (tail.slices >= 2 && need <= g.tail_ws_bytes) {
+          tail_begin = static_cast<unsigned>(tail.full);
+          grid = static_cast<int>(tail.full + tail.tail * tail.slices);
+        } else {
+          tail.slices = 1;
+        }
+      }
+    }
   }
   hipLaunchKernelGGL(kernel, dim3(grid), dim3(Cfg::NTHREADS), Cfg::LDS_BYTES,
                      g.stream, g.a, g.b,
@@ -242,8 +298,17 @@ int launch_gemm(const GemmArgs &g) {
                      static_cast<long long>(rb_b) * KT * TERMS * 64,
                      g.stride_c, split_stages,
                      zdim > 1 ? g.partial : static_cast<float *>(nullptr),
-                     g.c_ptrs, g.batch, zdim, entry_per_xcd);
+                     g.c_ptrs, g.batch, zdim, entry_per_xcd, tail_begin,
+                     tail.stages, g.tail_ws);
   int st = launch_status();
+  if (st == WMMAE_STATUS_SUCCESS && tail_begin != 0xffffffffu) {
+    hipLaunchKernelGGL((wmmae_gemm::reduce_tail_kernel<BM, BN>),
+                       dim3(static_cast<unsigned>(tail.tail), BM * BN / 1024),
+                       dim3(256), 0, g.stream, g.tail_ws, tail.slices,
+                       tail_begin, static_cast<unsigned>(tiles_m * tiles_n),
+                       tiles_m, tiles_n, g.c, g.m, g.n, g.ldc, g.alpha, g.beta);
+    st = launch_status();
+  }
   if (st == WMMAE_STATUS_SUCCESS && zdim > 1) {
     const long long blocks = ceil_div(static_cast<long long>(g.m) * g.n, 256);
     hipLaunchKernelGGL(wmmae_gemm::reduce_splits_kernel,
@@ -258,7 +323,7 @@ int launch_gemm(const GemmArgs &g) {
 // Tile choice: the 256x128 tile moves the fewest operand bytes per flop and is
 // the choice whenever its tiles fill the chip evenly; the tiles run in rounds
 // of one per compute unit, so when the last round would be mostly empty the
-// 128x128 tile (about 5 % slower per flop) can still finish sooner; 64x64
+// 128x128 tile (5 to 25 % slower per flop) can still finish sooner; 64x64
 // tiles for problems too small to give the larger ones work.
 template <class MT, int TERMS, bool RN> int gemm_by_size(const GemmArgs &g) {
   const int cus = device_cus();
@@ -272,8 +337,13 @@ template <class MT, int TERMS, bool RN> int gemm_by_size(const GemmArgs &g) {
   if constexpr (TERMS <= 2 && !RN) {
     if (big >= cus) {
       // time in units of one 128x128 tile: rounds * tile cost
-      const double t_big = static_cast<double>(ceil_div(big, cus)) * 2.0;
-      const double t_mid = static_cast<double>(ceil_div(mid, cus)) * 1.05;
+      const int KT = packed_k_tiles(g.k);
+      const bool tail_ok = g.batch == 1 && z == 1 && g.c_ptrs == nullptr &&
+                           g.tail_ws != nullptr;
+      const double t_big = rounds_cost(big, cus, KT, tail_ok) * 2.0;
+      // (a 128x128 tile measured at 1.2 to 1.25 times half a 256x128 tile in
+      // runs of two to eight rounds, 1.05 in long ones)
+      const double t_mid = rounds_cost(mid, cus, KT, tail_ok) * 1.2;
       if (t_big <= t_mid)
         return launch_gemm<MT, TERMS, 256, 128, 2, 2, RN>(g);
     }
@@ -550,12 +620,20 @@ int gemm_packed_impl(const int policy, const int m, const int n, const int k,
   // split-K only when the caller supplied room for the slices
   g.splits = choose_splits(m, n, k, batch);
   g.partial = nullptr;
-  if (g.splits > 1 && workspace != nullptr &&
-      reinterpret_cast<uintptr_t>(workspace) % 16 == 0 &&
-      workspace_bytes >= static_cast<size_t>(g.splits) * batch * m * n * 4u)
+  g.tail_ws = nullptr;
+  g.tail_ws_bytes = 0;
+  const bool ws_usable =
+      workspace != nullptr && reinterpret_cast<uintptr_t>(workspace) % 16 == 0;
+  if (g.splits > 1 && ws_usable &&
+      workspace_bytes >= static_cast<size_t>(g.splits) * batch * m * n * 4u) {
     g.partial = static_cast<float *>(workspace);
-  else
+  } else {
     g.splits = 1;
+    if (ws_usable) {
+      g.tail_ws = static_cast<float *>(workspace);
+      g.tail_ws_bytes = workspace_bytes;
+    }
+  }
   return gemm_dispatch(policy, flags, g);
 }
 
@@ -712,7 +790,30 @@ int wmmae_tcec_gemm_packed_workspace_bytes(const int policy, const int m,
   const int splits = (m == 0 || n == 0 || k == 0 || batch == 0)
                          ? 1
                          : choose_splits(m, n, k, batch);
-  *bytes = splits > 1 ? static_cast<size_t>(splits) * batch * m * n * 4u : 0;
+  if (splits > 1) {
+    *bytes = static_cast<size_t>(splits) * batch * m * n * 4u;
+  } else if (batch == 1 && m > 0 && n > 0) {
+    // K slices of the tiles of a partly empty last round: the largest need
+    // over the tile shapes and residencies the launch may choose
+    const int KT = packed_k_tiles(k);
+    size_t need = 0;
+    const int shapes[3][2] = {{256, 128}, {128, 128}, {64, 64}};
+    for (const auto &sh : shapes) {
+      const int lds = ring_depth(sh[0], sh[1], p.terms) *
+                      (sh[0] / 16 + sh[1] / 16) * p.terms * 1024;
+      const int per_cu = std::min(4, (160 * 1024) / lds);
+      const TailPlan t =
+          plan_tail(ceil_div(m, sh[0]) * ceil_div(n, sh[1]),
+                    static_cast<long long>(device_cus()) * per_cu, KT);
+      if (t.slices >= 2)
+        need = std::max<size_t>(need, static_cast<size_t>(t.slices) *
+                                          static_cast<size_t>(t.tail) * sh[0] *
+                                          sh[1] * 4u);
+    }
+    *bytes = need;
+  } else {
+    *bytes = 0;
+  }
   return WMMAE_STATUS_SUCCESS;
 }
 

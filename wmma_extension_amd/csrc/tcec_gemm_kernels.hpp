@@ -173,6 +173,91 @@ __global__ void __launch_bounds__(256)
 }
 
 // --------------------------------------------------------------------------
+// Tile id -> tile coordinates.  Ids x, x+8, x+16, ... run on XCD x, 32 of
+// them at a time.  With `interleave`, these 32 get one GROUP x (32/GROUP)
+// patch of a column-by-column walk through GROUP tile rows (a patch that is
+// close to square in elements needs the fewest L2 fills), and the eight XCDs
+// get eight neighbouring patches, which share the patches' A row panels: what
+// misses in one XCD's L2 is then in flight to, or already in, the memory-side
+// cache for the others.  The ids beyond the last full round of 8 x 32 are cut
+// into eight runs, one per XCD.  Without `interleave` the ids walk the patches
+// in order (one XCD owns the whole tile grid).
+// --------------------------------------------------------------------------
+template <unsigned GROUP>
+__device__ __forceinline__ void tile_of(unsigned pid, const unsigned num_tiles,
+                                        const unsigned tiles_m,
+                                        const unsigned tiles_n,
+                                        const bool interleave, int &tm,
+                                        int &tn) {
+  constexpr unsigned XCDS = 8, PATCH = 32;
+  if (interleave) {
+    const unsigned full = num_tiles / (XCDS * PATCH) * (XCDS * PATCH);
+    if (pid < full) {
+      const unsigned xcd = pid % XCDS, local = pid / XCDS;
+      pid = ((local / PATCH) * XCDS + xcd) * PATCH + local % PATCH;
+    } else {
+      const unsigned rem = num_tiles - full, t = pid - full;
+      const unsigned per = (rem + XCDS - 1) / XCDS;
+      const unsigned tall = (rem % XCDS == 0) ? XCDS : (rem % XCDS);
+      const unsigned xcd = t % XCDS, local = t / XCDS;
+      pid = full + (xcd < tall ? xcd * per + local
+                               : tall * per + (xcd - tall) * (per - 1) + local);
+    }
+  }
+  const unsigned width = GROUP * tiles_n;
+  const unsigned group = pid / width;
+  const unsigned first_m = group * GROUP;
+  const unsigned gsz = (tiles_m - first_m) < GROUP ? (tiles_m - first_m) : GROUP;
+  const unsigned in_group = pid - group * width;
+  const unsigned col = in_group / gsz;
+  tm = static_cast<int>(first_m + in_group - col * gsz);
+  tn = static_cast<int>(col);
+}
+
+// --------------------------------------------------------------------------
+// reduce_tail_kernel: C tile = alpha * sum_z partial[z][t] + beta * C tile for
+// the tail tiles t (tile ids tail_begin + t) that tcec_gemm_kernel has cut
+// into K slices.  partial[z][t] are dense column-major BM x BN tiles; the sum
+// runs over z in ascending order in double precision.  grid: (tail tiles,
+// BM*BN/1024), a thread owns four consecutive rows of one column.
+// --------------------------------------------------------------------------
+template <int BM, int BN>
+__global__ void __launch_bounds__(256)
+    reduce_tail_kernel(const float *__restrict__ partial, const int slices,
+                       const unsigned tail_begin, const unsigned num_tiles,
+                       const int tiles_m, const int tiles_n,
+                       float *__restrict__ C, const int M, const int N,
+                       const long long ldc, const float alpha,
+                       const float beta) {
+  const unsigned t = blockIdx.x, tail_tiles = gridDim.x;
+  int tm, tn;
+  tile_of<(BM > BN ? 4u : 8u)>(tail_begin + t, num_tiles, tiles_m, tiles_n,
+                               true, tm, tn);
+  const int e4 = static_cast<int>(blockIdx.y) * 256 + threadIdx.x;
+  const int col_l = e4 / (BM / 4), row_l = 4 * (e4 % (BM / 4));
+  const int row = tm * BM + row_l, col = tn * BN + col_l;
+  if (col_l >= BN || col >= N || row >= M)
+    return;
+  double s[4] = {0., 0., 0., 0.};
+  for (int z = 0; z < slices; z++) {
+    const f32x4 v = *reinterpret_cast<const f32x4 *>(
+        partial + (static_cast<long long>(z) * tail_tiles + t) * (BM * BN) +
+        col_l * BM + row_l);
+#pragma unroll
+    for (int x = 0; x < 4; x++)
+      s[x] += static_cast<double>(v[x]);
+  }
+  float *const p = C + row + static_cast<long long>(col) * ldc;
+#pragma unroll
+  for (int x = 0; x < 4; x++) {
+    if (row + x < M) {
+      const float v = alpha * static_cast<float>(s[x]);
+      p[x] = beta == 0.f ? v : v + beta * p[x];
+    }
+  }
+}
+
+// --------------------------------------------------------------------------
 // tcec_gemm_kernel: C = alpha * (A*B) + beta * C from packed operands.
 //
 //   MT      : MFMA element type (_Float16 or __bf16)
@@ -243,7 +328,9 @@ __global__ void __launch_bounds__(WGM *WGN * 64)
                      const long long batch_stride_c, const int split_stages,
                      float *__restrict__ partial,
                      float *const *__restrict__ c_ptrs, const int batches,
-                     const int splits, const int entry_per_xcd) {
+                     const int splits, const int entry_per_xcd,
+                     const unsigned tail_begin, const int tail_stages,
+                     float *__restrict__ tail_partial) {
   using Cfg = GemmConfig<MT, TERMS, BM, BN, WGM, WGN, NSTAGE, RN_MAIN>;
   typedef MT ab_vec __attribute__((ext_vector_type(8)));
   constexpr int NCH = Cfg::NCH, CH_A = Cfg::CH_A, CPW = Cfg::CPW;
@@ -277,64 +364,48 @@ __global__ void __launch_bounds__(WGM *WGN * 64)
   const unsigned my_xcd = blockIdx.x % XCDS;
   const unsigned my_first = entry_per_xcd ? blockIdx.x / XCDS : blockIdx.x;
   const unsigned my_step = entry_per_xcd ? gridDim.x / XCDS : gridDim.x;
+  // K slices for the tiles of the last, partly empty round only (one entry,
+  // no other split; tail_begin >= num_tiles switches it off): the tiles
+  // tail_begin .. num_tiles-1 are cut into slices of tail_stages k stages,
+  // the items after the whole tiles are (slice, tail tile) pairs, and a slice
+  // writes its raw sums as a dense BM x BN tile to
+  // tail_partial[slice][tail tile]; reduce_tail_kernel folds them into C.
+  const unsigned tail_tiles = tail_begin < num_tiles ? num_tiles - tail_begin : 0;
+  const unsigned tail_slices =
+      tail_tiles ? (KT + tail_stages - 1) / tail_stages : 0;
   const unsigned list_items =
-      entry_per_xcd
-          ? num_tiles * ((batches - my_xcd + XCDS - 1) / XCDS)
-          : num_tiles * batches * splits;
+      entry_per_xcd ? num_tiles * ((batches - my_xcd + XCDS - 1) / XCDS)
+      : tail_tiles  ? tail_begin + tail_tiles * tail_slices
+                    : num_tiles * batches * splits;
   if (my_first >= list_items)
     return; // nothing for this workgroup (before any barrier)
   const int n_my =
       static_cast<int>((list_items - my_first + my_step - 1) / my_step);
   struct Item {
     int tm, tn, batch, z;
+    int tail; // index among the tail tiles, -1 for a whole tile
   };
   auto decode = [&](const int i) {
     const unsigned v = my_first + static_cast<unsigned>(i) * my_step;
     Item it;
-    const unsigned rest = v / num_tiles;
+    it.tail = -1;
+    unsigned rest = v / num_tiles;
     unsigned pid = v - rest * num_tiles;
-    if (entry_per_xcd) {
+    if (tail_tiles && v >= tail_begin) {
+      const unsigned w = v - tail_begin;
+      it.z = static_cast<int>(w / tail_tiles);
+      it.tail = static_cast<int>(w - it.z * tail_tiles);
+      it.batch = 0;
+      pid = tail_begin + it.tail;
+    } else if (entry_per_xcd) {
       it.z = 0;
       it.batch = static_cast<int>(my_xcd + XCDS * rest);
     } else {
       it.z = static_cast<int>(rest / batches);
       it.batch = static_cast<int>(rest - it.z * batches);
     }
-    if (!entry_per_xcd) {
-      // Ids x, x+8, x+16, ... run on XCD x, 32 of them at a time: these 32
-      // get one patch of the walk below, and the eight XCDs get eight
-      // neighbouring patches, which share the patches' A row panels: what
-      // misses in one XCD's L2 is then in flight to, or already in, the
-      // memory-side cache for the others.  The ids beyond the last full
-      // round of 8 x 32 are cut into eight runs, one per XCD.
-      constexpr unsigned PATCH = 32;
-      const unsigned full = num_tiles / (XCDS * PATCH) * (XCDS * PATCH);
-      if (pid < full) {
-        const unsigned xcd = pid % XCDS, local = pid / XCDS;
-        pid = ((local / PATCH) * XCDS + xcd) * PATCH + local % PATCH;
-      } else {
-        const unsigned rem = num_tiles - full, t = pid - full;
-        const unsigned per = (rem + XCDS - 1) / XCDS;
-        const unsigned tall = (rem % XCDS == 0) ? XCDS : (rem % XCDS);
-        const unsigned xcd = t % XCDS, local = t / XCDS;
-        pid = full + (xcd < tall ? xcd * per + local
-                                 : tall * per + (xcd - tall) * (per - 1) + local);
-      }
-    }
-    {
-      // 32 workgroups run on one XCD at a time: a GROUP x (32/GROUP) patch of
-      // tiles that is close to square in elements needs the fewest L2 fills
-      constexpr unsigned GROUP = BM > BN ? 4 : 8;
-      const unsigned width = GROUP * tiles_n;
-      const unsigned group = pid / width;
-      const unsigned first_m = group * GROUP;
-      const unsigned gsz =
-          (tiles_m - first_m) < GROUP ? (tiles_m - first_m) : GROUP;
-      const unsigned in_group = pid - group * width;
-      const unsigned col = in_group / gsz;
-      it.tm = static_cast<int>(first_m + in_group - col * gsz);
-      it.tn = static_cast<int>(col);
-    }
+    tile_of<(BM > BN ? 4u : 8u)>(pid, num_tiles, tiles_m, tiles_n,
+                                 !entry_per_xcd, it.tm, it.tn);
     if constexpr ((ABLATE & 32) != 0)
       it.tm = it.tn = 0;
     return it;
@@ -344,11 +415,15 @@ __global__ void __launch_bounds__(WGM *WGN * 64)
   // to partial[z][batch] as a dense column-major M x N matrix;
   // reduce_splits_kernel adds the slices.  Used when there are too few output
   // tiles to fill the chip.
+  auto slice_stages = [&](const Item &it) {
+    return it.tail >= 0 ? tail_stages : split_stages;
+  };
   auto stages_of = [&](const Item &it) {
-    if (partial == nullptr)
+    if (partial == nullptr && it.tail < 0)
       return KT;
-    const int begin = it.z * split_stages;
-    return KT - begin < split_stages ? KT - begin : split_stages;
+    const int per = slice_stages(it);
+    const int begin = it.z * per;
+    return KT - begin < per ? KT - begin : per;
   };
 
   // ---- request cursor: the item and stage requested next, and the global
@@ -377,7 +452,9 @@ __global__ void __launch_bounds__(WGM *WGN * 64)
     const Item it = decode(i);
     req_stages = stages_of(it);
     const long long first_stage =
-        partial != nullptr ? static_cast<long long>(it.z) * split_stages : 0;
+        partial != nullptr || it.tail >= 0
+            ? static_cast<long long>(it.z) * slice_stages(it)
+            : 0;
 #pragma unroll
     for (int g = 0; g < RPW; g++) {
       // row block inside the stage: A's, then B's
@@ -610,23 +687,33 @@ __global__ void __launch_bounds__(WGM *WGN * 64)
   };
 
   // ---- epilogue of one item: recombine, scale, store
+  const int M_ = M, N_ = N;
   auto store_item = [&](const Item &it) {
-    const bool to_partial = partial != nullptr;
+    const bool to_tail = it.tail >= 0;
+    const bool to_partial = partial != nullptr || to_tail;
     float *const Cb =
-        to_partial
+        to_tail ? tail_partial +
+                      (static_cast<long long>(it.z) * tail_tiles + it.tail) *
+                          (BM * BN)
+        : to_partial
             ? partial + (static_cast<long long>(it.z) * batches + it.batch) *
                             (static_cast<long long>(M) * N)
             : (c_ptrs != nullptr ? c_ptrs[it.batch]
                                  : C + it.batch * batch_stride_c);
-    const long long ld_out = to_partial ? M : ldc;
+    // a tail slice stores its whole tile, tile-local, into its own BM x BN area
+    const int M = to_tail ? BM : M_;
+    const int N = to_tail ? BN : N_;
+    const long long ld_out = to_tail ? BM : (to_partial ? M : ldc);
     const float a_out = to_partial ? 1.f : alpha;
     const float b_out = to_partial ? 0.f : beta;
     const int vec_out =
-        to_partial ? (M % 4 == 0)
-                   : (vec_store && (reinterpret_cast<uintptr_t>(Cb) & 15u) == 0);
-    const int row_base =
-        it.tm * BM + wm * Cfg::WM + 4 * static_cast<int>(lane >> 4);
-    const int col_base = it.tn * BN + wn * Cfg::WN + static_cast<int>(lane & 15u);
+        to_tail      ? 1
+        : to_partial ? (M % 4 == 0)
+                     : (vec_store && (reinterpret_cast<uintptr_t>(Cb) & 15u) == 0);
+    const int row_base = (to_tail ? 0 : it.tm * BM) + wm * Cfg::WM +
+                         4 * static_cast<int>(lane >> 4);
+    const int col_base = (to_tail ? 0 : it.tn * BN) + wn * Cfg::WN +
+                         static_cast<int>(lane & 15u);
 #pragma unroll
     for (int j = 0; j < NT_; j++) {
       const int col = col_base + 16 * j;
