@@ -86,7 +86,8 @@ int wmmae_query(int what, long long *out);
  * larger with a short k; no K slices) are split inside the GEMM
  * kernel (as the reference's bgemm_kernel splits at fragment load,
  * batch_gemm.cu:196-386): they use no workspace, allocate nothing and ignore
- * the workspace arguments.  Both paths give the same bits. */
+ * the workspace arguments.  Both paths give the same bits as long as no K
+ * slices are made (those add the partial sums' rounding). */
 int wmmae_tcec_sgemm_workspace_bytes(int m, int n, int k, int batch, int policy,
                                      size_t *bytes);
 
