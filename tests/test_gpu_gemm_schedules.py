@@ -144,11 +144,14 @@ def test_pointer_arrays_through_packed_operands_and_xcd_owned_entries(tc, orc, d
 
 def test_random_shapes_packed_path_and_driver_choice_agree(tc, orc, dev):
     """120 seeded problems (1..5000 rows and columns, 1..3000 of k, 1..40 entries, all five
-    policies): pack + gemm_packed and the driver's own choice of path give the same bits,
-    and both stay within the policy's error bound of an FP64 product computed on the GPU."""
+    policies): pack + gemm_packed and the driver's own choice of path give the same bits
+    wherever the driver does not cut the K loop into slices (the partial sums of slices are
+    rounded on their own), and both stay within the policy's error bound of an FP64 product
+    computed on the GPU."""
     import random
     rnd = random.Random(20240)
     bound = {0: 4e-6, 2: 4e-6, 1: 3e-3, 3: 3e-4, 4: 3e-2}
+    sliced = 0
     for case in range(120):
         policy = rnd.choice([0, 0, 2, 2, 1, 3, 4])
         batch = rnd.choice([1, 1, 1, 2, 3, 9, 17, 40])
@@ -173,7 +176,13 @@ def test_random_shapes_packed_path_and_driver_choice_agree(tc, orc, dev):
         err = ((C.transpose(1, 2).double() - ref).abs().amax(dim=(1, 2)) / scale).max().item()
         tag = (case, policy, batch, m, n, k)
         assert err < bound[policy], tag
-        assert torch.equal(C, C2), tag
+        if tc.sgemm_path(m, n, k, batch, policy, 0) == tc.PATH_PACKED_SPLIT_K:
+            sliced += 1
+            err2 = ((C2.transpose(1, 2).double() - ref).abs().amax(dim=(1, 2)) / scale).max().item()
+            assert err2 < bound[policy], tag
+        else:
+            assert torch.equal(C, C2), tag
+    assert 0 < sliced < 40, sliced
 
 
 @pytest.mark.parametrize("policy", [0, 2])

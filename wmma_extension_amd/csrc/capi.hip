@@ -164,21 +164,28 @@ inline hipError_t allow_dynamic_lds(const void *const kernel, const int bytes,
   return e;
 }
 
-// Number of K slices: only when the output tiles cannot fill the chip and
-// every slice still has a long K loop.
+// Number of K slices of every tile: only when the output tiles cannot fill the
+// chip, in slices of at least 16 stages (512 of k).  Long K loops (4096 of k
+// or more): as many slices as fill the chip, 32 at most.  Shorter ones (from
+// 1536 of k): only when even 128x128 tiles would leave 40 % of the compute
+// units idle, and not more items than compute units (1536^3: 121 -> 150
+// effective TFLOPS; 1792^3 and 2048^3 are faster uncut).
 inline int choose_splits(const int m, const int n, const int k,
                          const int batch) {
   const long long tiles = ceil_div(m, 256) * ceil_div(n, 128) * batch;
+  const long long mid = ceil_div(m, 128) * ceil_div(n, 128) * batch;
   const int cus = device_cus();
   const int kt = static_cast<int>(ceil_div(k, 32));
-  if (tiles * 2 > cus || kt < 128)
+  if (tiles * 2 > cus)
     return 1;
-  long long s = ceil_div(cus, tiles);
-  const long long max_by_k = kt / 64; // at least 64 stages (2048 of k) a slice
-  if (s > max_by_k)
-    s = max_by_k;
-  if (s > 64)
-    s = 64;
+  long long s;
+  if (kt >= 128) {
+    s = std::min<long long>({ceil_div(cus, tiles), kt / 16, 32});
+  } else if (kt >= 48 && mid * 10 <= static_cast<long long>(cus) * 6) {
+    s = std::min<long long>(cus / tiles, kt / 16);
+  } else {
+    return 1;
+  }
   return s < 1 ? 1 : static_cast<int>(s);
 }
 
