@@ -216,3 +216,62 @@ def test_k_slices_for_the_last_round_of_tiles(tc, orc, dev, policy, shape):
     assert ((cut.double() - ref).abs().max() / scale).item() < 4e-6
     assert ((plain.double() - ref).abs().max() / scale).item() < 4e-6
     assert ((cut - plain).abs().max().double() / scale).item() < 1e-6
+
+
+def test_random_blas_arguments_against_fp64(tc, dev):
+    """100 seeded calls of the strided-batched entry point the way a BLAS user makes them:
+    both transposes of both operands, padded leading dimensions, alpha and beta other than
+    1 and 0, the round-to-nearest flag, with and without a caller's workspace, shapes drawn
+    so that all three paths (fused, packed, packed with K slices) are taken.  Each result is
+    compared with alpha * op(A) op(B) + beta * C in FP64, and the padding rows of C
+    (ldc > m) must keep their bytes."""
+    import random
+    rnd = random.Random(77)
+    bound = {0: 4e-6, 2: 4e-6, 1: 3e-3, 3: 3e-4, 4: 3e-2}
+    paths = [0, 0, 0]
+    for case in range(100):
+        policy = rnd.choice([0, 0, 2, 2, 1, 3, 4])
+        batch = rnd.choice([1, 1, 1, 1, 2, 3, 9])
+        kind = rnd.random()
+        if kind < 0.4:      # small outputs, long k
+            m, n, k = rnd.randint(1, 1200), rnd.randint(1, 1200), rnd.randint(1000, 30000)
+        elif kind < 0.7:
+            m, n, k = rnd.randint(1, 3000), rnd.randint(1, 3000), rnd.randint(1, 4000)
+        else:
+            m, n, k = rnd.randint(1, 600), rnd.randint(1, 600), rnd.randint(1, 600)
+        while batch * (m * k + n * k + m * n) * 4 > 6.0e8:
+            if batch > 1:
+                batch //= 2
+            else:
+                k = max(1, k // 2)
+        ta, tb = rnd.choice("NT"), rnd.choice("NT")
+        # column-major storage: A holds ra x ca elements, ra contiguous, in columns of lda
+        ra, ca = (m, k) if ta == "N" else (k, m)
+        rb, cb = (k, n) if tb == "N" else (n, k)
+        lda, ldb, ldc = (x + rnd.choice([0, 0, 1, 3, 4, 16]) for x in (ra, rb, m))
+        A = _uniform((batch, ca, lda), 5000 + case, dev)      # [entry, column, row]
+        B = _uniform((batch, cb, ldb), 6000 + case, dev)
+        C0 = _uniform((batch, n, ldc), 7000 + case, dev)
+        alpha = rnd.choice([1.0, 1.0, -0.5, 2.25])
+        beta = rnd.choice([0.0, 0.0, 1.0, -1.5])
+        flags = rnd.choice([0, 0, 0, tc.FLAG_RN_MAIN]) if policy in (0, 2) else 0
+        a_cm = A[:, :, :ra].double()                          # [entry, column, row]
+        b_cm = B[:, :, :rb].double()
+        op_a = a_cm.transpose(1, 2) if ta == "N" else a_cm    # (entry, m, k)
+        op_b = b_cm.transpose(1, 2) if tb == "N" else b_cm    # (entry, k, n)
+        prod = torch.matmul(op_a, op_b)
+        ref = alpha * prod + beta * C0[:, :, :m].transpose(1, 2).double()
+        scale = (abs(alpha) * prod.abs().amax(dim=(1, 2)) + abs(beta)).clamp_min(1e-30)
+        ws = None
+        if rnd.random() < 0.7:
+            ws = torch.empty(max(16, tc.workspace_bytes(m, n, k, batch, policy)), dtype=torch.uint8,
+                             device=dev)
+        C = C0.clone()
+        tc.sgemm_strided_batched(ta, tb, m, n, k, alpha, A, lda, ca * lda, B, ldb, cb * ldb, beta,
+                                 C, ldc, n * ldc, batch, policy, flags, ws)
+        err = ((C[:, :, :m].transpose(1, 2).double() - ref).abs().amax(dim=(1, 2)) / scale).max().item()
+        tag = (case, policy, flags, batch, ta + tb, m, n, k, lda, ldb, ldc, alpha, beta, ws is not None)
+        assert err < bound[policy], (tag, err)
+        assert torch.equal(C[:, :, m:], C0[:, :, m:]), tag
+        paths[tc.sgemm_path(m, n, k, batch, policy, flags)] += 1
+    assert min(paths) >= 10, paths
