@@ -72,45 +72,75 @@ inline long long packed_elems(const int rows, const int k, const int terms) {
 }
 
 // ------------------------------------------------------------------ pack
+// One operand of a split launch as the caller describes it.
+struct PackSource {
+  int rows;
+  const float *X;
+  const float *const *ptrs;
+  long long row_stride, k_stride, batch_stride;
+  void *packed;
+};
+
+inline wmmae_gemm::PackOperand pack_operand(const PackSource &src,
+                                            const int KT) {
+  wmmae_gemm::PackOperand o;
+  o.X = src.X;
+  o.ptrs = src.ptrs;
+  o.row_stride = src.row_stride;
+  o.k_stride = src.k_stride;
+  o.batch_stride = src.batch_stride;
+  o.rows = src.rows;
+  o.chunks = packed_row_blocks(src.rows) * KT;
+  o.out = static_cast<u32x4 *>(src.packed);
+  return o;
+}
+
+// Splits one operand (b == nullptr) or both operands of a product in a single
+// launch.
 template <class T, int TERMS>
-int launch_pack(const int rows, const int k, const float *X,
-                const float *const *ptrs, const long long row_stride,
-                const long long k_stride, const long long batch_stride,
-                const int batch, void *packed, hipStream_t stream) {
+int launch_pack(const int k, const int batch, const PackSource &a,
+                const PackSource *const b, hipStream_t stream) {
   const int KT = packed_k_tiles(k);
-  const long long chunks = packed_row_blocks(rows) * KT;
-  const long long blocks = ceil_div(chunks * 64, 256);
-  if (blocks > 0x7fffffffLL || batch > 65535)
+  const wmmae_gemm::PackOperand oa = pack_operand(a, KT);
+  const long long blocks_a = ceil_div(oa.chunks * 64, 256);
+  if (batch > 65535)
     return WMMAE_STATUS_NOT_SUPPORTED;
-  hipLaunchKernelGGL((wmmae_gemm::split_pack_kernel<T, TERMS>),
-                     dim3(static_cast<unsigned>(blocks), batch), dim3(256), 0,
-                     stream, X, row_stride, k_stride, rows, k, KT, chunks,
-                     batch_stride, ptrs, static_cast<u32x4 *>(packed),
-                     chunks * TERMS * 64);
+  if (b == nullptr) {
+    if (blocks_a > 0x7fffffffLL)
+      return WMMAE_STATUS_NOT_SUPPORTED;
+    hipLaunchKernelGGL((wmmae_gemm::split_pack_kernel<T, TERMS>),
+                       dim3(static_cast<unsigned>(blocks_a), batch), dim3(256),
+                       0, stream, oa, k, KT);
+    return launch_status();
+  }
+  const wmmae_gemm::PackOperand ob = pack_operand(*b, KT);
+  const long long blocks_b = ceil_div(ob.chunks * 64, 256);
+  if (blocks_a + blocks_b > 0x7fffffffLL)
+    return WMMAE_STATUS_NOT_SUPPORTED;
+  hipLaunchKernelGGL((wmmae_gemm::split_pack_pair_kernel<T, TERMS>),
+                     dim3(static_cast<unsigned>(blocks_a + blocks_b), batch),
+                     dim3(256), 0, stream, oa, ob,
+                     static_cast<unsigned>(blocks_a), k, KT);
   return launch_status();
 }
 
-int pack_dispatch(const int policy, const int rows, const int k, const float *X,
-                  const float *const *ptrs, const long long row_stride,
-                  const long long k_stride, const long long batch_stride,
-                  const int batch, void *packed, hipStream_t stream) {
-#define WMMAE_PACK_ARGS                                                        \
-  rows, k, X, ptrs, row_stride, k_stride, batch_stride, batch, packed, stream
+int pack_dispatch(const int policy, const int k, const int batch,
+                  const PackSource &a, const PackSource *const b,
+                  hipStream_t stream) {
   switch (policy) {
   case WMMAE_POLICY_F16_EC:
-    return launch_pack<w::half, 2>(WMMAE_PACK_ARGS);
+    return launch_pack<w::half, 2>(k, batch, a, b, stream);
   case WMMAE_POLICY_F16_NOEC:
-    return launch_pack<w::half, 1>(WMMAE_PACK_ARGS);
+    return launch_pack<w::half, 1>(k, batch, a, b, stream);
   case WMMAE_POLICY_BF16X3_EC:
-    return launch_pack<w::precision::tf32, 3>(WMMAE_PACK_ARGS);
+    return launch_pack<w::precision::tf32, 3>(k, batch, a, b, stream);
   case WMMAE_POLICY_BF16X2_EC:
-    return launch_pack<w::bfloat16, 2>(WMMAE_PACK_ARGS);
+    return launch_pack<w::bfloat16, 2>(k, batch, a, b, stream);
   case WMMAE_POLICY_BF16_NOEC:
-    return launch_pack<w::bfloat16, 1>(WMMAE_PACK_ARGS);
+    return launch_pack<w::bfloat16, 1>(k, batch, a, b, stream);
   default:
     return WMMAE_STATUS_INVALID_VALUE;
   }
-#undef WMMAE_PACK_ARGS
 }
 
 // ------------------------------------------------------------------ gemm
@@ -560,16 +590,21 @@ int wmmae_tcec_pack_bytes(const int rows, const int k, const int batch,
 namespace {
 // Shared implementations; X / C may be given as a base pointer with a batch
 // stride or as a device array of per-matrix pointers.
-int pack_impl(const int policy, const int rows, const int k,
-              const float *const X, const float *const *const ptrs,
-              const long long row_stride, const long long k_stride,
-              const long long batch_stride, const int batch, void *const packed,
-              const size_t packed_bytes, void *const stream) {
+// Argument checks of one operand of a split; WMMAE_STATUS_SUCCESS with
+// `nothing` set when there is nothing to write.
+int pack_check(const int policy, const int rows, const int k,
+               const float *const X, const float *const *const ptrs,
+               const long long row_stride, const long long k_stride,
+               const int batch, void *const packed, const size_t packed_bytes,
+               bool &nothing) {
   PolicyInfo p;
+  nothing = false;
   if (!policy_info(policy, p) || rows < 0 || k < 0 || batch < 0)
     return WMMAE_STATUS_INVALID_VALUE;
-  if (rows == 0 || k == 0 || batch == 0)
+  if (rows == 0 || k == 0 || batch == 0) {
+    nothing = true;
     return WMMAE_STATUS_SUCCESS;
+  }
   if ((X == nullptr && ptrs == nullptr) || packed == nullptr)
     return WMMAE_STATUS_NULL_POINTER;
   if (row_stride < 1 || k_stride < 1 || (row_stride != 1 && k_stride != 1))
@@ -580,8 +615,21 @@ int pack_impl(const int policy, const int rows, const int k,
   wmmae_tcec_pack_bytes(rows, k, batch, policy, &need);
   if (packed_bytes < need)
     return WMMAE_STATUS_WORKSPACE_TOO_SMALL;
-  return pack_dispatch(policy, rows, k, X, ptrs, row_stride, k_stride,
-                       batch_stride, batch, packed,
+  return WMMAE_STATUS_SUCCESS;
+}
+
+int pack_impl(const int policy, const int rows, const int k,
+              const float *const X, const float *const *const ptrs,
+              const long long row_stride, const long long k_stride,
+              const long long batch_stride, const int batch, void *const packed,
+              const size_t packed_bytes, void *const stream) {
+  bool nothing = false;
+  const int st = pack_check(policy, rows, k, X, ptrs, row_stride, k_stride,
+                            batch, packed, packed_bytes, nothing);
+  if (st != WMMAE_STATUS_SUCCESS || nothing)
+    return st;
+  const PackSource src{rows, X, ptrs, row_stride, k_stride, batch_stride, packed};
+  return pack_dispatch(policy, k, batch, src, nullptr,
                        static_cast<hipStream_t>(stream));
 }
 
@@ -753,13 +801,20 @@ int sgemm_impl(const char transa, const char transb, const int m, const int n,
   int st = WMMAE_STATUS_SUCCESS;
   if (k > 0) {
     // op(A)(i,l): 'N' -> A[i + l*lda], 'T' -> A[l + i*lda]
-    st = pack_impl(policy, m, k, A, a_ptrs, is_n(transa) ? 1 : lda,
-                   is_n(transa) ? lda : 1, stride_a, batch, pa, bytes_a, stream);
+    const PackSource sa{m, A, a_ptrs, is_n(transa) ? 1 : lda,
+                        is_n(transa) ? lda : 1, stride_a, pa};
     // op(B)(l,j): 'N' -> B[l + j*ldb], 'T' -> B[j + l*ldb]; packed rows = j
+    const PackSource sb{n, B, b_ptrs, is_n(transb) ? ldb : 1,
+                        is_n(transb) ? 1 : ldb, stride_b, pb};
+    bool none_a = false, none_b = false;
+    st = pack_check(policy, sa.rows, k, sa.X, sa.ptrs, sa.row_stride,
+                    sa.k_stride, batch, pa, bytes_a, none_a);
     if (st == WMMAE_STATUS_SUCCESS)
-      st = pack_impl(policy, n, k, B, b_ptrs, is_n(transb) ? ldb : 1,
-                     is_n(transb) ? 1 : ldb, stride_b, batch, pb, bytes_b,
-                     stream);
+      st = pack_check(policy, sb.rows, k, sb.X, sb.ptrs, sb.row_stride,
+                      sb.k_stride, batch, pb, bytes_b, none_b);
+    // (m, n, k and batch are all positive here: both operands have work)
+    if (st == WMMAE_STATUS_SUCCESS && !none_a && !none_b)
+      st = pack_dispatch(policy, k, batch, sa, &sb, s); // one launch for both
   }
   if (st == WMMAE_STATUS_SUCCESS)
     st = gemm_packed_impl(policy, m, n, k, alpha, pa, pb, beta, C, c_ptrs, ldc,

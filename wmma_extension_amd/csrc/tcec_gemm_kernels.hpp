@@ -56,29 +56,35 @@ __host__ __device__ constexpr int reads_due(const int count, const int span,
 // split_pack_kernel: X (fp32, element (r,k) at X[r*row_stride + k*k_stride])
 // -> packed terms.  One thread per (chunk, lane).  Rows >= rows and k >= K are
 // zero filled, so the GEMM kernel needs no edge handling on its loads.
-// Batch entry y reads X + y*in_batch_stride, or in_ptrs[y] when in_ptrs is set
-// (the reference's harness passes arrays of matrix pointers,
+// Batch entry y (blockIdx.y) reads X + y*batch_stride, or ptrs[y] when ptrs is
+// set (the reference's harness passes arrays of matrix pointers,
 // test/tcec/batch_gemm.cu:433-443).
 //   T      : split tag (half, bfloat16, precision::tf32)
 //   TERMS  : number of terms stored (1 = leading term only, i.e. no correction)
 //   KT     : number of 32-wide k chunks per row block; chunks = row blocks * KT
 // --------------------------------------------------------------------------
+struct PackOperand {
+  const float *X;             // entry y at X + y*batch_stride ...
+  const float *const *ptrs;   // ... or at ptrs[y] when set
+  long long row_stride, k_stride, batch_stride;
+  int rows;
+  long long chunks;           // row blocks * KT
+  u32x4 *out;                 // entry y at out + y*chunks*TERMS*64
+};
+
+// the work of one 256-thread block: four chunks of batch entry `entry`
 template <class T, int TERMS>
-__global__ void __launch_bounds__(256)
-    split_pack_kernel(const float *__restrict__ X, const long long row_stride,
-                      const long long k_stride, const int rows, const int K,
-                      const int KT, const long long chunks,
-                      const long long in_batch_stride,
-                      const float *const *__restrict__ in_ptrs,
-                      u32x4 *__restrict__ out,
-                      const long long out_batch_stride) {
+__device__ __forceinline__ void split_pack_block(const PackOperand &o,
+                                                 const int K, const int KT,
+                                                 const unsigned block,
+                                                 const unsigned entry) {
   using traits = mtk::wmma::tcec::detail::split_traits<T>;
   using S = typename traits::storage;
   static_assert(TERMS >= 1 && TERMS <= traits::num_terms, "bad TERMS");
   const unsigned lane = threadIdx.x & 63u;
   const long long chunk =
-      (static_cast<long long>(blockIdx.x) * 256 + threadIdx.x) >> 6;
-  if (chunk >= chunks)
+      (static_cast<long long>(block) * 256 + threadIdx.x) >> 6;
+  if (chunk >= o.chunks)
     return;
   const long long rb = chunk / KT;
   const int kc = static_cast<int>(chunk - rb * KT);
@@ -89,14 +95,13 @@ __global__ void __launch_bounds__(256)
 #pragma unroll
   for (int x = 0; x < 8; x++)
     v[x] = 0.f;
-  if (r < rows && k0 < K) {
+  if (r < o.rows && k0 < K) {
     // batch entry: base + stride, or a device array of matrix pointers
-    const float *const base = in_ptrs != nullptr
-                                  ? in_ptrs[blockIdx.y]
-                                  : X + blockIdx.y * in_batch_stride;
+    const float *const base =
+        o.ptrs != nullptr ? o.ptrs[entry] : o.X + entry * o.batch_stride;
     const float *p =
-        base + r * row_stride + static_cast<long long>(k0) * k_stride;
-    if (k_stride == 1 && k0 + 8 <= K &&
+        base + r * o.row_stride + static_cast<long long>(k0) * o.k_stride;
+    if (o.k_stride == 1 && k0 + 8 <= K &&
         (reinterpret_cast<uintptr_t>(p) & 15u) == 0) {
       const f32x4 lo = *reinterpret_cast<const f32x4 *>(p);
       const f32x4 hi = *reinterpret_cast<const f32x4 *>(p + 4);
@@ -109,7 +114,7 @@ __global__ void __launch_bounds__(256)
 #pragma unroll
       for (int x = 0; x < 8; x++)
         if (k0 + x < K)
-          v[x] = p[x * k_stride];
+          v[x] = p[x * o.k_stride];
     }
   }
 
@@ -123,10 +128,30 @@ __global__ void __launch_bounds__(256)
     t[1][x] = t1;
     t[2][x] = t2;
   }
-  u32x4 *o = out + blockIdx.y * out_batch_stride + chunk * (TERMS * 64) + lane;
+  u32x4 *dst =
+      o.out + entry * (o.chunks * (TERMS * 64)) + chunk * (TERMS * 64) + lane;
 #pragma unroll
   for (int p = 0; p < TERMS; p++)
-    o[p * 64] = __builtin_bit_cast(u32x4, t[p]);
+    dst[p * 64] = __builtin_bit_cast(u32x4, t[p]);
+}
+
+template <class T, int TERMS>
+__global__ void __launch_bounds__(256)
+    split_pack_kernel(const PackOperand o, const int K, const int KT) {
+  split_pack_block<T, TERMS>(o, K, KT, blockIdx.x, blockIdx.y);
+}
+
+// Both operands of a product in one launch (the GEMM entry points pack A and B
+// back to back; for small products a launch costs as much as the packing):
+// blocks [0, blocks_a) take A, the rest B.
+template <class T, int TERMS>
+__global__ void __launch_bounds__(256)
+    split_pack_pair_kernel(const PackOperand a, const PackOperand b,
+                           const unsigned blocks_a, const int K, const int KT) {
+  if (blockIdx.x < blocks_a)
+    split_pack_block<T, TERMS>(a, K, KT, blockIdx.x, blockIdx.y);
+  else
+    split_pack_block<T, TERMS>(b, K, KT, blockIdx.x - blocks_a, blockIdx.y);
 }
 
 // --------------------------------------------------------------------------
