@@ -112,11 +112,16 @@ def test_reference_harness_command_prints_the_reference_csv(tc, orc, dev):
     import io
     from wmma_extension_amd import batch_gemm
     out = io.StringIO()
-    batch_gemm.main(["--m", "512", "--k", "128", "1024", "--batch", "6", "--count", "3"], out)
+    batch_gemm.main(["--m", "512", "--k", "128", "1024", "--batch", "6", "--count", "3", "--vendor"],
+                    out)
     lines = out.getvalue().strip().split("\n")
     assert lines[0] == "mode,m,n,k,batch_size,residual,throughput"
-    assert len(lines) == 3
-    for line, k in zip(lines[1:], (128, 1024)):
+    assert len(lines) == 5
+    # the vendor library's fp32 GEMM beside each line (the reference's TEST_CUBLAS lines, :609-637)
+    for line, k in zip(lines[2::2], (128, 1024)):
+        f = line.split(",")
+        assert f[:6] == ["vendor", "512", "512", str(k), "6", "-"] and float(f[6]) > 0.0
+    for line, k in zip(lines[1::2], (128, 1024)):
         f = line.split(",")
         assert f[:5] == ["wmmae", "512", "512", str(k), "6"]
         # all-positive ramps: the fp32 accumulators' error grows with k (1e-7 at k=128,
