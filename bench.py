@@ -50,7 +50,7 @@ MEASURED_TRAFFIC_BYTES = {
     "c4": (75_497_800 + 1_048_580) * 1024,
     "c3": (524_670 + 65_536) * 1024,
     "c5a": (524_500 + 262_283) * 1024,
-    "c2": (1_048_724 + 3_277_470) * 1024,
+    "c2": (1_048_622 + 3_276_830) * 1024,
 }
 
 

@@ -161,6 +161,36 @@ WMMAE_D void fill_fragment(fragment<Use, M, N, K, T, Layout> &frag,
 }
 
 // ------------------------------------------------- matrix load / store
+namespace detail {
+// An fp32 accumulator holds rows r .. r+3 of one column in registers 4q .. 4q+3
+// of a lane (the MFMA result layout), so a column-major tile whose base and
+// leading dimension keep those four floats 16-byte aligned moves with one
+// 16-byte access per four registers instead of four 4-byte ones.
+typedef float f32_quad __attribute__((ext_vector_type(4)));
+template <class L> constexpr bool rows_in_quads() {
+  if (L::num_elements % 4 != 0)
+    return false;
+  for (unsigned lane = 0; lane < wave_size; lane++)
+    for (unsigned x = 0; x < L::num_elements; x += 4)
+      for (unsigned e = 0; e < 4; e++)
+        if (L::row(lane, x) % 4 != 0 ||
+            L::row(lane, x + e) != L::row(lane, x) + e ||
+            L::col(lane, x + e) != L::col(lane, x))
+          return false;
+  return true;
+}
+template <int M, int N, int K, class T, class MEM_T> struct acc_quads {
+  static constexpr bool value =
+      std::is_same<T, float>::value &&
+      std::is_same<typename std::remove_cv<MEM_T>::type, float>::value &&
+      rows_in_quads<gfx950::frag_layout<accumulator, M, N, K>>();
+};
+template <class P>
+WMMAE_D bool quad_aligned(const P *const ptr, const unsigned ldm) {
+  return ldm % 4 == 0 && (reinterpret_cast<uintptr_t>(ptr) & 15u) == 0;
+}
+} // namespace detail
+
 // (reference: nvcuda::wmma::load_matrix_sync and wmma_mma.hpp:64-145; there
 // the dense mem_index is re-strided to ldm, here (i,j) is used directly.)
 template <class Use, int M, int N, int K, class T, class Layout, class MEM_T>
@@ -181,6 +211,21 @@ WMMAE_D void load_matrix_sync(fragment<accumulator, M, N, K, T> &frag,
                               const MEM_T *const ptr, const unsigned ldm,
                               const layout_t layout, const bool = true) {
   const bool col = layout == mem_col_major;
+  if constexpr (detail::acc_quads<M, N, K, T, MEM_T>::value) {
+    if (col && detail::quad_aligned(ptr, ldm)) {
+      using L = typename fragment<accumulator, M, N, K, T>::layout_model;
+      const unsigned lane = detail::common::get_lane_id();
+#pragma unroll
+      for (unsigned x = 0; x < frag.num_elements; x += 4) {
+        const detail::f32_quad v = *reinterpret_cast<const detail::f32_quad *>(
+            ptr + L::row(lane, x) + L::col(lane, x) * ldm);
+#pragma unroll
+        for (unsigned e = 0; e < 4; e++)
+          frag.x[x + e] = v[e];
+      }
+      return;
+    }
+  }
   foreach_ij<decltype(frag)>([&](const unsigned *list, const unsigned,
                                  const unsigned i, const unsigned j) {
     frag.x[list[0]] =
@@ -193,6 +238,20 @@ WMMAE_D void store_matrix_sync(MEM_T *const ptr,
                                const unsigned ldm, const layout_t layout,
                                const bool = true) {
   const bool col = layout == mem_col_major;
+  if constexpr (detail::acc_quads<M, N, K, T, MEM_T>::value) {
+    if (col && detail::quad_aligned(ptr, ldm)) {
+      using L = typename fragment<accumulator, M, N, K, T>::layout_model;
+      const unsigned lane = detail::common::get_lane_id();
+#pragma unroll
+      for (unsigned x = 0; x < frag.num_elements; x += 4) {
+        const detail::f32_quad v = {frag.x[x], frag.x[x + 1], frag.x[x + 2],
+                                    frag.x[x + 3]};
+        *reinterpret_cast<detail::f32_quad *>(ptr + L::row(lane, x) +
+                                              L::col(lane, x) * ldm) = v;
+      }
+      return;
+    }
+  }
   foreach_ij<decltype(frag)>([&](const unsigned *list, const unsigned,
                                  const unsigned i, const unsigned j) {
     ptr[col ? (i + j * ldm) : (i * ldm + j)] =

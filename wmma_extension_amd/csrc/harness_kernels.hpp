@@ -52,8 +52,8 @@ namespace w = mtk::wmma;
 namespace tcec = mtk::wmma::tcec;
 
 // --------------------------------------------------------------------------
-// Fragment primitives over a stream of tiles.  One wave per tile, grid-stride.
-// Per tile (256 fp32 in):
+// Fragment primitives over a stream of tiles.  One wave per tile, grid-stride,
+// four waves per block.  Per tile (256 fp32 in):
 //   a_row/a_col/b_row/b_col : (lane,reg) dump of a 16x16x16 half fragment filled
 //                             through foreach_ij from the tile read in that layout
 //   acc_out                 : tile read as a row-major accumulator through
@@ -83,8 +83,17 @@ __global__ void __launch_bounds__(256)
   using FB_C = w::fragment<w::matrix_b, 16, 16, 16, w::half, w::col_major>;
   using FC = w::fragment<w::accumulator, 16, 16, 16, float>;
 
+  // The tile is read from HBM once, 16 bytes per lane, into the wave's own
+  // 1 KiB of LDS; the primitives below then gather from LDS (where a user of
+  // the API keeps the tile it builds fragments from).  A wave's LDS accesses
+  // execute in program order, so no barrier is needed between the copy and
+  // the gathers, nor before the next tile overwrites the buffer.
+  __shared__ __attribute__((aligned(16))) float staged[4][256];
+  float *const tile = staged[threadIdx.x / w::wave_size];
+  typedef float f32x4 __attribute__((ext_vector_type(4)));
   for (long long t = wave; t < num_tiles; t += num_waves) {
-    const float *const tile = tiles + t * 256;
+    *reinterpret_cast<f32x4 *>(tile + 4 * lane) =
+        *reinterpret_cast<const f32x4 *>(tiles + t * 256 + 4 * lane);
     {
       FA_R f;
       w::foreach_ij<FA_R>([&](const unsigned *list, const unsigned count,
