@@ -150,6 +150,31 @@ def test_primitive_mma_all_shapes(tc, orc, dev, elem, shape):
         assert orc.max_rel_err(D, ref) < 16 * eps, (a_col, b_col, c_col, d_col, with_c)
 
 
+@pytest.mark.parametrize("shape", [0, 2])
+def test_accumulator_load_store_aligned_and_not(tc, dev, shape):
+    """Column-major accumulator tiles at a 16-byte aligned base move with 16-byte accesses,
+    any other base element by element: C read from, and D written to, views that start one,
+    two and three floats into an allocation give the bytes of the aligned call, and the
+    floats around D keep theirs."""
+    from wmma_extension_amd import tcec as T
+    m, n, k = T.PRIMITIVE_SHAPES[shape]
+    rng = np.random.default_rng(300 + shape)
+    a = torch.from_numpy(rng.integers(-4, 5, m * k).astype(np.float32)).to(dev)
+    b = torch.from_numpy(rng.integers(-4, 5, k * n).astype(np.float32)).to(dev)
+    c = torch.from_numpy(rng.integers(-9, 10, m * n).astype(np.float32)).to(dev)
+    for c_col, d_col in ((1, 1), (1, 0), (0, 1)):
+        want = tc.primitive_mma(2, shape, a, b, c, 0, 0, c_col, d_col)
+        for off in (1, 2, 3):
+            c_buf = torch.zeros(m * n + 8, device=dev)
+            c_buf[off:off + m * n] = c
+            d_buf = torch.full((m * n + 8,), -77.0, device=dev)
+            got = tc.primitive_mma(2, shape, a, b, c_buf[off:off + m * n], 0, 0, c_col, d_col,
+                                   d=d_buf[off:off + m * n])
+            assert got.data_ptr() % 16 == 4 * off
+            assert torch.equal(got, want), (c_col, d_col, off)
+            assert torch.all(d_buf[:off] == -77.0) and torch.all(d_buf[off + m * n:] == -77.0)
+
+
 def test_foreach_error_corrected_product(tc, orc, dev):
     """A, dA, B, dB filled through foreach's mem_index, three MMAs: error below 1e-6
     against FP64 on uniform[-1,1] inputs (test/primitive/foreach.cu:24-80, :120)."""

@@ -319,11 +319,14 @@ def clock_samples(nsamples, period_ticks, stream=None, device="cuda:0"):
 PRIMITIVE_SHAPES = {0: (16, 16, 16), 1: (16, 16, 32), 2: (32, 32, 8), 3: (32, 32, 16)}
 
 
-def primitive_mma(elem, shape, a, b, c, a_col, b_col, c_col, d_col):
-    """a, b, c: flat fp32 CUDA images of the operands in the given layouts; returns flat d."""
-    _need_cuda(a, b, c)
+def primitive_mma(elem, shape, a, b, c, a_col, b_col, c_col, d_col, d=None):
+    """a, b, c: flat fp32 CUDA images of the operands in the given layouts; returns flat d
+    (written into `d` when the caller passes one, e.g. a view at an odd offset)."""
+    _need_cuda(a, b, c, d)
     m, n, _ = PRIMITIVE_SHAPES[shape]
-    d = torch.full((m * n,), float("nan"), dtype=torch.float32, device=a.device)
+    if d is None:
+        d = torch.full((m * n,), float("nan"), dtype=torch.float32, device=a.device)
+    assert d.numel() == m * n and d.is_contiguous()
     st = _lib.lib().wmmae_primitive_mma(elem, shape, _ptr(d), _ptr(a), _ptr(b), _ptr(c), a_col, b_col,
                                         c_col, d_col, _stream())
     _lib.check(st, "wmmae_primitive_mma")
