@@ -304,9 +304,15 @@ int launch_gemm(const GemmArgs &g) {
   const long long resident = static_cast<long long>(device_cus()) * per_cu;
   int grid = static_cast<int>(std::min(items, resident));
   int entry_per_xcd = 0;
+  if (zdim > 1 && resident % 8 == 0) {
+    // split-K: eight runs of the item list, one per XCD, so that an XCD holds
+    // as few K slices as possible; the grid is padded to whole runs
+    entry_per_xcd = 2;
+    grid = static_cast<int>(std::min(8 * ceil_div(items, 8), resident));
+  }
   unsigned tail_begin = 0xffffffffu; // no tail slices
   TailPlan tail;
-  if (items > resident) {
+  if (items > resident && entry_per_xcd == 0) {
     if (g.batch >= 8 && zdim == 1 && resident % 8 == 0) {
       entry_per_xcd = 1;
     } else if (split_stages >= 64) {

@@ -380,15 +380,24 @@ __global__ void __launch_bounds__(WGM *WGN * 64)
   //     ids are spread over the 8 XCDs and then walk the grid in groups of
   //     GROUP tile rows, so that the workgroups resident on one XCD share A
   //     row panels and B column panels in its L2.
-  //   entry_per_xcd != 0 (no split-K, gridDim.x a multiple of 8): XCD x, i.e.
+  //   entry_per_xcd == 1 (no split-K, gridDim.x a multiple of 8): XCD x, i.e.
   //     the workgroups with blockIdx.x % 8 == x, owns batch entries x, x+8,
   //     ...: the operands of an entry are then read into one L2 only.
+  //   entry_per_xcd == 2 (split-K, gridDim.x a multiple of 8): the same list
+  //     as for 0, cut into eight runs of ceil(items / 8), one per XCD.  A K
+  //     slice of the operands is shared only by the tiles of that slice, so
+  //     an XCD should hold as few slices as possible: 32 tiles x 8 slices
+  //     become one whole slice per XCD, and each operand byte is read into
+  //     one L2 instead of up to eight.
   // (the host keeps the item count below 2^31: 32-bit divisions only)
   constexpr unsigned XCDS = 8;
   const unsigned num_tiles = static_cast<unsigned>(tiles_m * tiles_n);
   const unsigned my_xcd = blockIdx.x % XCDS;
   const unsigned my_first = entry_per_xcd ? blockIdx.x / XCDS : blockIdx.x;
   const unsigned my_step = entry_per_xcd ? gridDim.x / XCDS : gridDim.x;
+  const unsigned all_items = num_tiles * batches * splits;
+  const unsigned run_len = (all_items + XCDS - 1) / XCDS; // entry_per_xcd == 2
+  const unsigned run_begin = my_xcd * run_len;
   // K slices for the tiles of the last, partly empty round only (one entry,
   // no other split; tail_begin >= num_tiles switches it off): the tiles
   // tail_begin .. num_tiles-1 are cut into slices of tail_stages k stages,
@@ -399,9 +408,13 @@ __global__ void __launch_bounds__(WGM *WGN * 64)
   const unsigned tail_slices =
       tail_tiles ? (KT + tail_stages - 1) / tail_stages : 0;
   const unsigned list_items =
-      entry_per_xcd ? num_tiles * ((batches - my_xcd + XCDS - 1) / XCDS)
-      : tail_tiles  ? tail_begin + tail_tiles * tail_slices
-                    : num_tiles * batches * splits;
+      entry_per_xcd == 1 ? num_tiles * ((batches - my_xcd + XCDS - 1) / XCDS)
+      : entry_per_xcd == 2
+          ? (run_begin >= all_items           ? 0u
+             : all_items - run_begin < run_len ? all_items - run_begin
+                                               : run_len)
+      : tail_tiles ? tail_begin + tail_tiles * tail_slices
+                   : all_items;
   if (my_first >= list_items)
     return; // nothing for this workgroup (before any barrier)
   const int n_my =
@@ -411,7 +424,8 @@ __global__ void __launch_bounds__(WGM *WGN * 64)
     int tail; // index among the tail tiles, -1 for a whole tile
   };
   auto decode = [&](const int i) {
-    const unsigned v = my_first + static_cast<unsigned>(i) * my_step;
+    const unsigned v = (entry_per_xcd == 2 ? run_begin : 0u) + my_first +
+                       static_cast<unsigned>(i) * my_step;
     Item it;
     it.tail = -1;
     unsigned rest = v / num_tiles;
@@ -422,7 +436,7 @@ __global__ void __launch_bounds__(WGM *WGN * 64)
       it.tail = static_cast<int>(w - it.z * tail_tiles);
       it.batch = 0;
       pid = tail_begin + it.tail;
-    } else if (entry_per_xcd) {
+    } else if (entry_per_xcd == 1) {
       it.z = 0;
       it.batch = static_cast<int>(my_xcd + XCDS * rest);
     } else {
