@@ -51,6 +51,7 @@ MEASURED_TRAFFIC_BYTES = {
     "c3": (524_670 + 65_536) * 1024,
     "c5a": (524_500 + 262_283) * 1024,
     "c2": (1_048_622 + 3_276_830) * 1024,
+    "c5b": (2_100_460 + 32_768) * 1024,
 }
 
 
