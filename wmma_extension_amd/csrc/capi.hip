@@ -288,11 +288,13 @@ int launch_gemm(const GemmArgs &g) {
       static_cast<long long>(tiles_m) * tiles_n * g.batch * zdim;
   if (items >= (1ll << 31)) // the kernel counts items in 32 bits
     return WMMAE_STATUS_INVALID_VALUE;
-  // More items than resident workgroups (the large tiles take most of a
-  // compute unit's LDS, so one per unit):
-  //  * 8 or more batch entries: persistent workgroups, an XCD owns whole
-  //    entries, so that an entry's operands are read into one L2 only
-  //    (batch 256 of 1024x1024x256: 196 -> 256 effective TFLOPS);
+  // Who takes which item (the large tiles take most of a compute unit's LDS,
+  // so one workgroup per unit is resident):
+  //  * 8 or more batch entries: an XCD owns whole entries, so that an entry's
+  //    operands are read into one L2 only (batch 256 of 1024x1024x256:
+  //    196 -> 256 effective TFLOPS), persistent workgroups when there are
+  //    more items than resident workgroups;
+  // and with more items than resident workgroups otherwise
   //  * short K loops: persistent workgroups walking one shared list, their
   //    requests running ahead into the next item;
   //  * long K loops (64 stages = 2048 of k or more per item) of few entries:
@@ -312,10 +314,14 @@ int launch_gemm(const GemmArgs &g) {
   }
   unsigned tail_begin = 0xffffffffu; // no tail slices
   TailPlan tail;
-  if (items > resident && entry_per_xcd == 0) {
-    if (g.batch >= 8 && zdim == 1 && resident % 8 == 0) {
-      entry_per_xcd = 1;
-    } else if (split_stages >= 64) {
+  if (zdim == 1 && g.batch >= 8 && resident % 8 == 0) {
+    // also when every item gets a workgroup of its own: a workgroup for every
+    // item of the XCD that owns the most entries
+    entry_per_xcd = 1;
+    grid = static_cast<int>(std::min(
+        8ll * tiles_m * tiles_n * ceil_div(g.batch, 8), resident));
+  } else if (items > resident && entry_per_xcd == 0) {
+    if (split_stages >= 64) {
       grid = static_cast<int>(items);
       // one entry, no split-K, room for the slices: the tiles of a partly
       // empty last round are cut along K
@@ -453,17 +459,16 @@ template <class T, int TERMS, int BM, int BN> int launch_fused(FusedArgs f) {
 // 128x128 tiles, unless they leave compute units without work and 64x64 tiles
 // (four times as many workgroups; one takes 0.65 of a 128x128 tile's time at
 // these latency-bound sizes) finish sooner: 1024^3 went from 41 to 27 us.
-template <class T, int TERMS> int fused_by_size(const FusedArgs &f) {
+inline bool fused_small_tiles(const int m, const int n, const int batch) {
   const long long cus = device_cus();
-  const long long tiles128 =
-      ceil_div(f.p.M, 128) * ceil_div(f.p.N, 128) * f.p.batch;
-  const long long tiles64 =
-      ceil_div(f.p.M, 64) * ceil_div(f.p.N, 64) * f.p.batch;
-  const bool small_tiles =
-      (f.p.M <= 64 && f.p.N <= 64) ||
-      (tiles128 < cus && 0.65 * static_cast<double>(ceil_div(tiles64, cus)) <
-                             static_cast<double>(ceil_div(tiles128, cus)));
-  if (small_tiles)
+  const long long tiles128 = ceil_div(m, 128) * ceil_div(n, 128) * batch;
+  const long long tiles64 = ceil_div(m, 64) * ceil_div(n, 64) * batch;
+  return (m <= 64 && n <= 64) ||
+         (tiles128 < cus && 0.65 * static_cast<double>(ceil_div(tiles64, cus)) <
+                                static_cast<double>(ceil_div(tiles128, cus)));
+}
+template <class T, int TERMS> int fused_by_size(const FusedArgs &f) {
+  if (fused_small_tiles(f.p.M, f.p.N, f.p.batch))
     return launch_fused<T, TERMS, 64, 64>(f);
   return launch_fused<T, TERMS, 128, 128>(f);
 }
@@ -486,13 +491,20 @@ int fused_dispatch(const int policy, const FusedArgs &f) {
 }
 
 // Fused (split inside the GEMM kernel) or packed (split pass + MFMA kernel)?
-// The fused kernel does the same conversion and matrix work per 128x128x32
-// tile step whatever the shape, about 220 effective TFLOP/s with two terms, and
-// moves only the fp32 operands and C.  The packed path multiplies twice as
-// fast but first writes and re-reads the split operands, which pays off only
-// when every operand element is used by many tiles.  Both times are estimated
-// from rates measured on MI355X; K-heavy single products that want K slices
-// stay on the packed path.
+// The fused kernel moves only the fp32 operands and C but needs about twice as
+// long per 128x128x32 tile step; the packed path first writes and re-reads the
+// split operands, which pays off when every operand element is used by many
+// tiles.  Both times are estimated with the same shape, a launch cost plus
+// rounds of tiles over the compute units times (k stages * time per stage +
+// time per tile), bounded below by the bytes moved, with parameters fitted to
+// 573 measured products on MI355X (m = n = 384 .. 4096, k = 64 .. 8192, 1 to
+// 256 entries, one to three terms; median error of either estimate 5 %, the
+// choice costs 0.8 % over always taking the faster path).  K-heavy products
+// that want K slices stay on the packed path.
+struct PathRates {
+  double launch, stage, tile, bytes_per_s; // seconds, seconds, seconds, B/s
+  double split_bytes_per_s;                // packed path only
+};
 inline bool use_fused(const int m, const int n, const int k, const int batch,
                       const int flags, const int terms, const int policy) {
   // (the round-to-nearest flag with a policy that has no such variant is
@@ -502,24 +514,48 @@ inline bool use_fused(const int m, const int n, const int k, const int batch,
       policy != WMMAE_POLICY_BF16X3_EC;
   if (k <= 0 || rn_unsupported || choose_splits(m, n, k, batch) != 1)
     return false;
-  if (m <= 512 && n <= 512)
-    return true;
-  // Times of both paths, linear fits to measurements on MI355X (batched
-  // products, m = n = 512 .. 2048, k = 64 .. 2048).  Fused kernel: C stored
-  // at 7.5 TB/s (two waves per SIMD, one stores while the other multiplies),
-  // then 250 / 242 / 166 effective TFLOPS for 1 / 2 / 3 terms.  Packed path:
-  // two split launches moving 4 + 2*terms bytes per operand element at
-  // 6.6 TB/s, C stored at 5.3 (4.0 with the 128x128 tile of three terms) TB/s
-  // while the single wave per SIMD does nothing else, then 700 / 460 / 252.
-  const double ab = (static_cast<double>(m) + n) * k * batch; // operand elements
+  static const PathRates fused_rates[3] = {
+      {5.0e-6, 0.76e-6, 3.0e-6, 5.0e12, 0.},
+      {5.0e-6, 1.11e-6, 3.0e-6, 5.0e12, 0.},
+      {5.0e-6, 1.41e-6, 3.1e-6, 5.0e12, 0.}};
+  static const PathRates packed_rates[3] = {
+      {6.0e-6, 0.24e-6, 3.4e-6, 4.5e12, 7.0e12},
+      {6.5e-6, 0.50e-6, 3.8e-6, 3.6e12, 5.6e12},
+      {8.8e-6, 0.99e-6, 3.4e-6, 3.4e12, 5.9e12}};
+  const PathRates &f = fused_rates[terms - 1], &p = packed_rates[terms - 1];
+  const long long cus = device_cus();
+  const double kt = static_cast<double>(ceil_div(k, 32));
   const double c_bytes = 4.0 * m * n * batch;
-  const double flops = 2.0 * m * n * k * batch;
-  const double fused_rate = terms == 1 ? 250e12 : terms == 2 ? 242e12 : 166e12;
-  const double packed_rate = terms == 1 ? 700e12 : terms == 2 ? 460e12 : 252e12;
-  const double t_fused = c_bytes / 7.5e12 + flops / fused_rate;
-  const double t_packed = 12e-6 + (4.0 + 2.0 * terms) * ab / 6.6e12 +
-                          c_bytes / (terms == 3 ? 4.0e12 : 5.3e12) +
-                          flops / packed_rate;
+  const double ab = (static_cast<double>(m) + n) * k * batch; // operand elements
+  const long long tiles64 = ceil_div(m, 64) * ceil_div(n, 64) * batch;
+  const long long tiles128 = ceil_div(m, 128) * ceil_div(n, 128) * batch;
+  const long long tiles256 = ceil_div(m, 256) * ceil_div(n, 128) * batch;
+
+  // fused kernel: 128x128 tiles, or 64x64 ones (a third of the stage time,
+  // half of the per-tile time) under fused_by_size's rule
+  const bool small = fused_small_tiles(m, n, batch);
+  const double f_rounds =
+      static_cast<double>(ceil_div(small ? tiles64 : tiles128, cus));
+  const double t_fused =
+      f.launch + std::max(f_rounds * (kt * f.stage * (small ? 0.33 : 1.0) +
+                                      f.tile * (small ? 0.5 : 1.0)),
+                          (c_bytes + 4.0 * ab) / f.bytes_per_s);
+
+  // packed path: rounds in units of one 128x128 tile as gemm_by_size counts
+  // them (a 256x128 tile 2.0, a 128x128 tile 1.2 for one and two terms, a
+  // 64x64 tile 0.4)
+  double units;
+  const double r128 = static_cast<double>(ceil_div(tiles128, cus));
+  if (terms <= 2 && tiles256 >= cus &&
+      2.0 * static_cast<double>(ceil_div(tiles256, cus)) <= 1.2 * r128)
+    units = 2.0 * static_cast<double>(ceil_div(tiles256, cus));
+  else if (tiles128 >= cus || (m > 64 && n > 64))
+    units = r128 * (terms <= 2 ? 1.2 : 1.0);
+  else
+    units = 0.4 * static_cast<double>(ceil_div(tiles64, cus));
+  const double t_packed =
+      p.launch + (4.0 + 2.0 * terms) * ab / p.split_bytes_per_s +
+      std::max(units * (kt * p.stage + p.tile), c_bytes / p.bytes_per_s);
   return t_fused < t_packed;
 }
 
