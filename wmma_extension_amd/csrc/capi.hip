@@ -194,29 +194,62 @@ inline hipError_t allow_dynamic_lds(const void *const kernel, const int bytes,
   return e;
 }
 
-// Number of K slices of every tile: only when the output tiles cannot fill the
-// chip, in slices of at least 16 stages (512 of k).  Long K loops (4096 of k
-// or more): as many slices as fill the chip, 32 at most.  Shorter ones (from
-// 1536 of k): only when even 128x128 tiles would leave 40 % of the compute
-// units idle, and not more items than compute units (1536^3: 121 -> 150
-// effective TFLOPS; 1792^3 and 2048^3 are faster uncut).
-inline int choose_splits(const int m, const int n, const int k,
+// Number of K slices of every tile, when the 256x128 output tiles cannot fill
+// half the chip.  For every candidate (at most 32 slices of at least 6 stages)
+// the GEMM's time is estimated the way gemm_by_size will run it: the tile that
+// the slice count leads to, rounds of those tiles over the compute units,
+// stages per slice at that tile's time per stage, a fixed time per tile, and
+// for more than one slice the fold (a launch plus the planes written and
+// read).  The cheapest count is taken, any split having to beat the uncut run
+// by 5 %.  Times per stage and tile: fits to measurements on MI355X (144
+// products, m = n = 512 .. 2048, k = 512 .. 4096, each run with 1, 2, 3, 4, 6
+// and 8 slices: the choice is within 0.7 % of the best measured count on
+// average; "as many slices as fill the chip with 256x128 tiles" was 7 % off,
+// over-cutting outputs from 1280^2 up and not cutting short loops at all).
+inline double split_time(const int terms, const int m, const int n,
+                         const int batch, const int kt, const int slices) {
+  const long long cus = device_cus();
+  const int stages = static_cast<int>(ceil_div(kt, slices));
+  const long long z = ceil_div(kt, stages);
+  const long long big = ceil_div(m, 256) * ceil_div(n, 128) * batch * z;
+  const long long mid = ceil_div(m, 128) * ceil_div(n, 128) * batch * z;
+  double stage_time, rounds;
+  const double r_big = static_cast<double>(ceil_div(big, cus));
+  const double r_mid = static_cast<double>(ceil_div(mid, cus));
+  if (terms <= 2 && big >= cus && r_big * 2.0 <= r_mid * 1.2) {
+    stage_time = 1.0e-6; // 256x128
+    rounds = r_big;
+  } else if (mid >= cus || (m > 64 && n > 64)) {
+    stage_time = terms <= 2 ? 0.6e-6 : 0.99e-6; // 128x128
+    rounds = r_mid;
+  } else {
+    stage_time = 0.25e-6; // 64x64
+    rounds = static_cast<double>(
+        ceil_div(ceil_div(m, 64) * ceil_div(n, 64) * batch * z, cus));
+  }
+  double t = rounds * (stages * stage_time + 7e-6);
+  if (z > 1)
+    t += 6e-6 + static_cast<double>(z + 1) * m * n * batch * 4.0 / 3e12;
+  return t;
+}
+inline int choose_splits(const int terms, const int m, const int n, const int k,
                          const int batch) {
   const long long tiles = ceil_div(m, 256) * ceil_div(n, 128) * batch;
-  const long long mid = ceil_div(m, 128) * ceil_div(n, 128) * batch;
-  const int cus = device_cus();
   const int kt = static_cast<int>(ceil_div(k, 32));
-  if (tiles * 2 > cus)
+  if (tiles * 2 > device_cus())
     return 1;
-  long long s;
-  if (kt >= 128) {
-    s = std::min<long long>({ceil_div(cus, tiles), kt / 16, 32});
-  } else if (kt >= 48 && mid * 10 <= static_cast<long long>(cus) * 6) {
-    s = std::min<long long>(cus / tiles, kt / 16);
-  } else {
-    return 1;
+  int best = 1;
+  double t_best = 0.95 * split_time(terms, m, n, batch, kt, 1);
+  for (int s = 2; s <= 32 && s * 6 <= kt; s++) {
+    if (ceil_div(kt, ceil_div(kt, s)) != s)
+      continue; // the same slices as a smaller count
+    const double t = split_time(terms, m, n, batch, kt, s);
+    if (t < t_best) {
+      t_best = t;
+      best = s;
+    }
   }
-  return s < 1 ? 1 : static_cast<int>(s);
+  return best;
 }
 
 // K slices for the tiles of the last round only.  `tiles` output tiles run in
@@ -512,7 +545,7 @@ inline bool use_fused(const int m, const int n, const int k, const int batch,
   const bool rn_unsupported =
       (flags & WMMAE_FLAG_RN_MAIN) != 0 && policy != WMMAE_POLICY_F16_EC &&
       policy != WMMAE_POLICY_BF16X3_EC;
-  if (k <= 0 || rn_unsupported || choose_splits(m, n, k, batch) != 1)
+  if (k <= 0 || rn_unsupported || choose_splits(terms, m, n, k, batch) != 1)
     return false;
   static const PathRates fused_rates[3] = {
       {5.0e-6, 0.76e-6, 3.0e-6, 5.0e12, 0.},
@@ -727,7 +760,7 @@ int gemm_packed_impl(const int policy, const int m, const int n, const int k,
   g.terms = p.terms;
   g.stream = static_cast<hipStream_t>(stream);
   // split-K only when the caller supplied room for the slices
-  g.splits = choose_splits(m, n, k, batch);
+  g.splits = choose_splits(p.terms, m, n, k, batch);
   g.partial = nullptr;
   g.tail_ws = nullptr;
   g.tail_ws_bytes = 0;
@@ -905,7 +938,7 @@ int wmmae_tcec_gemm_packed_workspace_bytes(const int policy, const int m,
     return WMMAE_STATUS_INVALID_VALUE;
   const int splits = (m == 0 || n == 0 || k == 0 || batch == 0)
                          ? 1
-                         : choose_splits(m, n, k, batch);
+                         : choose_splits(p.terms, m, n, k, batch);
   if (splits > 1) {
     *bytes = static_cast<size_t>(splits) * batch * m * n * 4u;
   } else if (batch == 1 && m > 0 && n > 0) {
@@ -946,7 +979,7 @@ int wmmae_tcec_sgemm_path(const int m, const int n, const int k,
     *path = 0;
   else
     *path = (m > 0 && n > 0 && k > 0 && batch > 0 &&
-             choose_splits(m, n, k, batch) > 1)
+             choose_splits(p.terms, m, n, k, batch) > 1)
                 ? 2
                 : 1;
   return WMMAE_STATUS_SUCCESS;
