@@ -201,9 +201,9 @@ inline hipError_t allow_dynamic_lds(const void *const kernel, const int bytes,
 // stages per slice at that tile's time per stage, a fixed time per tile, and
 // for more than one slice the fold (a launch plus the planes written and
 // read).  The cheapest count is taken, any split having to beat the uncut run
-// by 5 %.  Times per stage and tile: fits to measurements on MI355X (144
-// products, m = n = 512 .. 2048, k = 512 .. 4096, each run with 1, 2, 3, 4, 6
-// and 8 slices: the choice is within 0.7 % of the best measured count on
+// by 5 %.  Times per stage and tile: fits to measurements on MI355X (216
+// products, m = n = 512 .. 2048, k = 512 .. 4096, one to three terms, each run
+// with 1, 2, 3, 4, 6 and 8 slices: the choice is within 0.7 % of the best measured count on
 // average; "as many slices as fill the chip with 256x128 tiles" was 7 % off,
 // over-cutting outputs from 1280^2 up and not cutting short loops at all).
 inline double split_time(const int terms, const int m, const int n,
@@ -217,10 +217,10 @@ inline double split_time(const int terms, const int m, const int n,
   const double r_big = static_cast<double>(ceil_div(big, cus));
   const double r_mid = static_cast<double>(ceil_div(mid, cus));
   if (terms <= 2 && big >= cus && r_big * 2.0 <= r_mid * 1.2) {
-    stage_time = 1.0e-6; // 256x128
+    stage_time = terms == 1 ? 0.8e-6 : 1.0e-6; // 256x128
     rounds = r_big;
   } else if (mid >= cus || (m > 64 && n > 64)) {
-    stage_time = terms <= 2 ? 0.6e-6 : 0.99e-6; // 128x128
+    stage_time = terms == 1 ? 0.45e-6 : terms == 2 ? 0.6e-6 : 0.99e-6; // 128x128
     rounds = r_mid;
   } else {
     stage_time = 0.25e-6; // 64x64
