@@ -70,7 +70,8 @@ const char *wmmae_status_string(int status);
 /* what: 0 = library version (major*10000 + minor*100 + patch),
  *       1 = compute units of the current device,
  *       2 = max engine clock in kHz,
- *       3 = number of policies */
+ *       3 = number of policies
+ * (No counterpart in the reference, which is header-only.) */
 int wmmae_query(int what, long long *out);
 
 /* ------------------------------------------------------------------ GEMM
@@ -144,7 +145,10 @@ int wmmae_tcec_pack(int policy, int rows, int k, const float *X,
  * when its tiles leave the last round over the compute units mostly empty
  * (single large products: only that round's tiles are cut); size from
  * wmmae_tcec_gemm_packed_workspace_bytes (0 when no cut would be made).
- * Without it the product runs uncut. */
+ * Without it the product runs uncut.
+ * Replaces: launch_bgemm on operands that are already split,
+ * test/tcec/batch_gemm.cu:433-443 (the reference's kernel has no K slices: its
+ * grid is one block per output tile and batch entry, :396-399, :418). */
 int wmmae_tcec_gemm_packed_workspace_bytes(int policy, int m, int n, int k,
                                            int batch, size_t *bytes);
 int wmmae_tcec_gemm_packed(int policy, int m, int n, int k, const float *alpha,
@@ -195,7 +199,8 @@ int wmmae_tcec_mma_tile(int shape, int type, int ec, int inst, float *d,
                         int rounding, void *stream);
 
 /* Same with m=n=k=32, 16x16x32, operands loaded through the load_matrix_sync
- * overload that takes the memory layout from the fragment's Layout argument. */
+ * overload that takes the memory layout from the fragment's Layout argument
+ * (tcec/tcec.hpp:281-291). */
 int wmmae_tcec_mma_tile_native(int type, int ec, int a_frag_col,
                                int b_frag_col, float *d, const float *a,
                                const float *b, int d_col, void *stream);
@@ -310,7 +315,7 @@ int wmmae_utils_cp_async(int size, int mode, void *dst, const void *src,
 
 /* out[i] = utils::cast<DST>(in[i]); dst_type 0 half, 1 bfloat16 (out: 16-bit
  * patterns), 2 tf32, 3 float (out: fp32).
- * Replaces: test/utils/cast.cu. */
+ * Replaces: test/utils/cast.cu:1-6 (utils::cast, utils.hpp:21-26). */
 int wmmae_utils_cast(int dst_type, const float *in, void *out, long long n,
                      void *stream);
 
