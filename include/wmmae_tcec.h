@@ -65,6 +65,8 @@ typedef enum {
                                 outside the matrix core (the reference's
                                 mma_rn_sync, tcec/tcec.hpp:640-706) */
 
+/* Text for a wmmae_status value.  (No counterpart in the reference: its
+ * harness aborts through WMMAE_CUDA_CHECK_ERROR, test/tcec/utils.hpp:11-20.) */
 const char *wmmae_status_string(int status);
 
 /* what: 0 = library version (major*10000 + minor*100 + patch),
