@@ -206,6 +206,17 @@ inline hipError_t allow_dynamic_lds(const void *const kernel, const int bytes,
 // with 1, 2, 3, 4, 6 and 8 slices: the choice is within 0.7 % of the best measured count on
 // average; "as many slices as fill the chip with 256x128 tiles" was 7 % off,
 // over-cutting outputs from 1280^2 up and not cutting short loops at all).
+// Whether the 256x128 tile is a candidate at all: only where the 128x128 tiles
+// need more than one round over the compute units (in a single round the
+// smaller tile always finishes first), and not for the one-term kernels on
+// loops of 32 stages or fewer, where the stores of C dominate and the smaller
+// tile measured 8 to 12 % faster.  (Forced-tile runs of 124 products: the
+// choice below is within 0.4 % of the faster tile on average; requiring a full
+// round of 256x128 tiles instead had cost 2 %, up to 13 % at 2560^2 .. 2816^2.)
+inline bool big_tile_candidate(const int terms, const long long mid,
+                               const int kt) {
+  return terms <= 2 && mid > device_cus() && !(terms == 1 && kt <= 32);
+}
 inline double split_time(const int terms, const int m, const int n,
                          const int batch, const int kt, const int slices) {
   const long long cus = device_cus();
@@ -216,7 +227,7 @@ inline double split_time(const int terms, const int m, const int n,
   double stage_time, rounds;
   const double r_big = static_cast<double>(ceil_div(big, cus));
   const double r_mid = static_cast<double>(ceil_div(mid, cus));
-  if (terms <= 2 && big >= cus && r_big * 2.0 <= r_mid * 1.2) {
+  if (big_tile_candidate(terms, mid, stages) && r_big * 2.0 <= r_mid * 1.2) {
     stage_time = terms == 1 ? 0.8e-6 : 1.0e-6; // 256x128
     rounds = r_big;
   } else if (mid >= cus || (m > 64 && n > 64)) {
@@ -403,7 +414,7 @@ int launch_gemm(const GemmArgs &g) {
 }
 
 // Tile choice: the 256x128 tile moves the fewest operand bytes per flop and is
-// the choice whenever its tiles fill the chip evenly; the tiles run in rounds
+// the choice whenever its rounds cost less; the tiles run in rounds
 // of one per compute unit, so when the last round would be mostly empty the
 // 128x128 tile (5 to 25 % slower per flop) can still finish sooner; 64x64
 // tiles for problems too small to give the larger ones work.
@@ -417,9 +428,9 @@ template <class MT, int TERMS, bool RN> int gemm_by_size(const GemmArgs &g) {
   // (not with the separate fp32 adds of RN: their temporaries do not fit the
   // register file next to the large tile's accumulators)
   if constexpr (TERMS <= 2 && !RN) {
-    if (big >= cus) {
+    const int KT = packed_k_tiles(g.k);
+    if (big_tile_candidate(TERMS, mid, static_cast<int>(ceil_div(KT, z)))) {
       // time in units of one 128x128 tile: rounds * tile cost
-      const int KT = packed_k_tiles(g.k);
       const bool tail_ok = g.batch == 1 && z == 1 && g.c_ptrs == nullptr &&
                            g.tail_ws != nullptr;
       const double t_big = rounds_cost(big, cus, KT, tail_ok) * 2.0;
@@ -579,7 +590,7 @@ inline bool use_fused(const int m, const int n, const int k, const int batch,
   // 64x64 tile 0.4)
   double units;
   const double r128 = static_cast<double>(ceil_div(tiles128, cus));
-  if (terms <= 2 && tiles256 >= cus &&
+  if (big_tile_candidate(terms, tiles128, static_cast<int>(kt)) &&
       2.0 * static_cast<double>(ceil_div(tiles256, cus)) <= 1.2 * r128)
     units = 2.0 * static_cast<double>(ceil_div(tiles256, cus));
   else if (tiles128 >= cus || (m > 64 && n > 64))
