@@ -358,7 +358,14 @@ int launch_gemm(const GemmArgs &g) {
   }
   unsigned tail_begin = 0xffffffffu; // no tail slices
   TailPlan tail;
-  if (zdim == 1 && g.batch >= 8 && resident % 8 == 0) {
+  // (an XCD that owns one entry more than the others must not cost more
+  // rounds than the shared list would take: 9 entries of 128 tiles are 8
+  // rounds on the XCD with two entries, 5 on the shared list)
+  const long long owned_rounds = ceil_div(
+      static_cast<long long>(tiles_m) * tiles_n * ceil_div(g.batch, 8),
+      resident / 8);
+  if (zdim == 1 && g.batch >= 8 && resident % 8 == 0 &&
+      owned_rounds * 100 <= ceil_div(items, resident) * 115) {
     // also when every item gets a workgroup of its own: a workgroup for every
     // item of the XCD that owns the most entries
     entry_per_xcd = 1;
