@@ -493,7 +493,15 @@ template <class T, int TERMS, int BM, int BN> int launch_fused(FusedArgs f) {
   // one persistent workgroup per compute unit at most; with 8 or more batch
   // entries an XCD (block index mod 8) owns whole entries
   const int per_xcd_max = device_cus() / 8 > 0 ? device_cus() / 8 : 1;
-  long long per_xcd = p.batch >= 8
+  // (not when the XCD that owns one entry more than the others would need
+  // over 15 % more rounds of tiles than an even spread)
+  const long long all_tiles =
+      static_cast<long long>(p.batch) * p.tiles_per_batch;
+  p.grouped =
+      p.batch >= 8 &&
+      ceil_div(ceil_div(p.batch, 8) * p.tiles_per_batch, per_xcd_max) * 100 <=
+          ceil_div(all_tiles, 8ll * per_xcd_max) * 115;
+  long long per_xcd = p.grouped
                           ? ceil_div(p.batch, 8) * p.tiles_per_batch
                           : ceil_div(static_cast<long long>(p.batch) *
                                          p.tiles_per_batch,

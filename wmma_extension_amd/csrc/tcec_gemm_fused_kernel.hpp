@@ -62,6 +62,9 @@ struct FusedParams {
   long long ldc, c_bs;
   int M, N, K, batch;
   int tiles_m, tiles_per_batch;
+  // XCD x (block index mod 8) owns the batch entries x, x+8, ... (set by the
+  // launcher for 8 or more entries that spread evenly enough)
+  int grouped;
   // 16-byte requests are possible as far as the host can tell: k contiguous,
   // K and the strides multiples of 4, base pointers aligned (pointer-array
   // entries are checked by the kernel)
@@ -124,7 +127,7 @@ __global__ void __launch_bounds__(64 * NW)
 
   // ---- this workgroup's tiles: v = first + i*stride while v < count
   const int tpb = p.tiles_per_batch;
-  const bool grouped = p.batch >= 8;
+  const bool grouped = p.grouped != 0;
   const int xcd = grouped ? static_cast<int>(blockIdx.x & 7u) : 0;
   const int first = grouped ? static_cast<int>(blockIdx.x >> 3)
                             : static_cast<int>(blockIdx.x);
