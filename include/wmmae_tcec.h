@@ -99,7 +99,11 @@ int wmmae_tcec_sgemm_workspace_bytes(int m, int n, int k, int batch, int policy,
  * reference, whose harness fixes one kernel configuration at compile time,
  * batch_gemm.cu:408-431, 659): *path = 0 the single kernel that splits the
  * operands on the fly (no workspace), 1 packed operands in the workspace,
- * 2 packed operands and K slices (when the workspace has room for them). */
+ * 2 packed operands and K slices (when the workspace has room for them).
+ * The answer assumes operands the single kernel can read 16 bytes at a time
+ * (k the contiguous direction, k and the leading dimensions multiples of 4,
+ * 16-byte aligned bases); other operands with k > 96 take path 1 where this
+ * says 0. */
 int wmmae_tcec_sgemm_path(int m, int n, int k, int batch, int policy, int flags,
                           int *path);
 

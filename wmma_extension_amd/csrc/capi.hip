@@ -564,14 +564,23 @@ struct PathRates {
   double launch, stage, tile, bytes_per_s; // seconds, seconds, seconds, B/s
   double split_bytes_per_s;                // packed path only
 };
+// fused_vec: the fused kernel can request 16 bytes per lane from both
+// operands (k contiguous, k and the strides multiples of 4, aligned bases).
+// Without that it issues four times as many requests and ran at 0.55 of the
+// packed path's speed in the median over 114 random products with k % 4 != 0
+// (faster than the packed path in one of them, by 10 %, at k = 77), so such
+// products take the packed path unless k is very short.
 inline bool use_fused(const int m, const int n, const int k, const int batch,
-                      const int flags, const int terms, const int policy) {
+                      const int flags, const int terms, const int policy,
+                      const bool fused_vec = true) {
   // (the round-to-nearest flag with a policy that has no such variant is
   // turned down by the packed path's dispatch)
   const bool rn_unsupported =
       (flags & WMMAE_FLAG_RN_MAIN) != 0 && policy != WMMAE_POLICY_F16_EC &&
       policy != WMMAE_POLICY_BF16X3_EC;
   if (k <= 0 || rn_unsupported || choose_splits(terms, m, n, k, batch) != 1)
+    return false;
+  if (!fused_vec && k > 96)
     return false;
   static const PathRates fused_rates[3] = {
       {5.0e-6, 0.76e-6, 3.0e-6, 5.0e12, 0.},
@@ -596,7 +605,8 @@ inline bool use_fused(const int m, const int n, const int k, const int batch,
   const double f_rounds =
       static_cast<double>(ceil_div(small ? tiles64 : tiles128, cus));
   const double t_fused =
-      f.launch + std::max(f_rounds * (kt * f.stage * (small ? 0.33 : 1.0) +
+      f.launch + std::max(f_rounds * (kt * f.stage * (fused_vec ? 1.0 : 2.5) *
+                                          (small ? 0.33 : 1.0) +
                                       f.tile * (small ? 0.5 : 1.0)),
                           (c_bytes + 4.0 * ab) / f.bytes_per_s);
 
@@ -834,20 +844,31 @@ int sgemm_impl(const char transa, const char transb, const int m, const int n,
       ldc < m)
     return WMMAE_STATUS_BAD_LEADING_DIM;
 
-  if (use_fused(m, n, k, batch, flags, p.terms, policy)) {
+  const auto aligned16 = [](const void *ptr) {
+    return reinterpret_cast<uintptr_t>(ptr) % 16 == 0;
+  };
+  // 16-byte requests of the fused kernel (entries of pointer arrays are
+  // checked by the kernel itself)
+  const long long a_rs = is_n(transa) ? 1 : lda, a_ks = is_n(transa) ? lda : 1;
+  const long long b_rs = is_n(transb) ? ldb : 1, b_ks = is_n(transb) ? 1 : ldb;
+  const bool vec_a = a_ks == 1 && k % 4 == 0 && a_rs % 4 == 0 &&
+                     (a_ptrs != nullptr || (aligned16(A) && stride_a % 4 == 0));
+  const bool vec_b = b_ks == 1 && k % 4 == 0 && b_rs % 4 == 0 &&
+                     (b_ptrs != nullptr || (aligned16(B) && stride_b % 4 == 0));
+  if (use_fused(m, n, k, batch, flags, p.terms, policy, vec_a && vec_b)) {
     if (batch > (1 << 26)) // tile indices are 32-bit
       return WMMAE_STATUS_NOT_SUPPORTED;
     FusedArgs f;
     wmmae_gemm::FusedParams &q = f.p;
     q.A = A;
     q.a_ptrs = a_ptrs;
-    q.a_rs = is_n(transa) ? 1 : lda;
-    q.a_ks = is_n(transa) ? lda : 1;
+    q.a_rs = a_rs;
+    q.a_ks = a_ks;
     q.a_bs = stride_a;
     q.B = B;
     q.b_ptrs = b_ptrs;
-    q.b_rs = is_n(transb) ? ldb : 1;
-    q.b_ks = is_n(transb) ? 1 : ldb;
+    q.b_rs = b_rs;
+    q.b_ks = b_ks;
     q.b_bs = stride_b;
     q.C = C;
     q.c_ptrs = c_ptrs;
@@ -857,13 +878,8 @@ int sgemm_impl(const char transa, const char transb, const int m, const int n,
     q.N = n;
     q.K = k;
     q.batch = batch;
-    const auto aligned16 = [](const void *ptr) {
-      return reinterpret_cast<uintptr_t>(ptr) % 16 == 0;
-    };
-    q.vec_a = q.a_ks == 1 && k % 4 == 0 && q.a_rs % 4 == 0 &&
-              (a_ptrs != nullptr || (aligned16(A) && stride_a % 4 == 0));
-    q.vec_b = q.b_ks == 1 && k % 4 == 0 && q.b_rs % 4 == 0 &&
-              (b_ptrs != nullptr || (aligned16(B) && stride_b % 4 == 0));
+    q.vec_a = vec_a;
+    q.vec_b = vec_b;
     q.vec_store = (ldc % 4 == 0) &&
                   (c_ptrs != nullptr || (aligned16(C) && stride_c % 4 == 0));
     q.rn_main = (flags & WMMAE_FLAG_RN_MAIN) != 0;
