@@ -187,3 +187,29 @@ def test_sgemm_path_query_on_the_baseline_workloads():
     assert h.wmmae_tcec_sgemm_path(-1, 16, 16, 1, 0, 0, ctypes.byref(out)) == -1
     assert h.wmmae_tcec_sgemm_path(16, 16, 16, 1, 9, 0, ctypes.byref(out)) == -1
     assert h.wmmae_tcec_sgemm_path(16, 16, 16, 1, 0, 2, ctypes.byref(out)) == -1
+
+
+def test_slice_counts_the_estimates_choose():
+    """The number of K slices is what the workspace query sizes its planes for (planes of
+    m*n*batch floats).  Pinned on the shapes the estimate was checked against on MI355X
+    (with no GPU the library plans for 256 compute units): the K-heavy baseline product is
+    cut into one slice per XCD, outputs from 1792^2 up are not cut at k = 4096 with two
+    terms, small outputs with a short loop are."""
+    import ctypes
+    from wmma_extension_amd import _lib
+    h = _lib.lib()
+    h.wmmae_tcec_gemm_packed_workspace_bytes.argtypes = [ctypes.c_int] * 5 + [ctypes.POINTER(ctypes.c_size_t)]
+    def planes(policy, m, n, k, batch=1):
+        out = ctypes.c_size_t(0)
+        assert h.wmmae_tcec_gemm_packed_workspace_bytes(policy, m, n, k, batch, ctypes.byref(out)) == 0
+        assert out.value % (m * n * batch * 4) == 0
+        return out.value // (m * n * batch * 4)
+    assert planes(0, 1024, 1024, 262144) == 8
+    assert planes(2, 1024, 1024, 262144) == 4
+    assert planes(0, 1024, 1024, 4096) == 4
+    assert planes(0, 1280, 1280, 4096) == 5      # 250 tiles of 256x128: one round
+    assert planes(0, 512, 512, 1024) == 5
+    assert planes(0, 1000, 900, 50000, 2) == 4
+    out = ctypes.c_int(-1)
+    for shape in ((1792, 1792, 4096), (2048, 2048, 2048)):
+        assert h.wmmae_tcec_sgemm_path(*shape, 1, 0, 0, ctypes.byref(out)) == 0 and out.value == 1, shape
