@@ -86,8 +86,10 @@ int wmmae_query(int what, long long *out);
  * from wmmae_tcec_sgemm_workspace_bytes.  workspace == NULL lets the library
  * take it from the stream-ordered allocator (hipMallocAsync / hipFreeAsync on
  * `stream`; measured at 3 to 9 us a call on MI355X, which a product of 20 us
- * feels - keep a workspace across calls where calls are small).  Products whose operands are reused by few tiles (m, n <= 512, or
- * larger with a short k; no K slices) are split inside the GEMM
+ * feels - keep a workspace across calls where calls are small).  Products
+ * whose operand elements are used by few tiles (small m and n, or a short k;
+ * an estimate of both paths' times decides; no K slices; operands readable
+ * 16 bytes at a time) are split inside the GEMM
  * kernel (as the reference's bgemm_kernel splits at fragment load,
  * batch_gemm.cu:196-386): they use no workspace, allocate nothing and ignore
  * the workspace arguments.  Both paths give the same bits as long as no K
