@@ -587,7 +587,7 @@ inline bool use_fused(const int m, const int n, const int k, const int batch,
       {5.0e-6, 1.11e-6, 3.0e-6, 5.0e12, 0.},
       {5.0e-6, 1.41e-6, 3.1e-6, 5.0e12, 0.}};
   static const PathRates packed_rates[3] = {
-      {6.0e-6, 0.24e-6, 3.4e-6, 4.5e12, 7.0e12},
+      {8.9e-6, 0.31e-6, 2.0e-6, 5.0e12, 6.6e12},
       {6.5e-6, 0.50e-6, 3.8e-6, 3.6e12, 5.6e12},
       {8.8e-6, 0.99e-6, 3.4e-6, 3.4e12, 5.9e12}};
   const PathRates &f = fused_rates[terms - 1], &p = packed_rates[terms - 1];
