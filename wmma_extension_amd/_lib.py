@@ -59,17 +59,36 @@ EXPORTS = [
 ]
 
 
-def build(verbose=False):
-    """Compile the HIP sources into LIB_PATH (always recompiles)."""
-    os.makedirs(LIB_DIR, exist_ok=True)
-    hipcc = os.environ.get("HIPCC", "/opt/rocm/bin/hipcc")
-    cmd = [hipcc, *HIPCC_FLAGS, "-I" + INCLUDE_DIR,
-           os.path.join(CSRC_DIR, "capi.hip"), "-o", LIB_PATH]
+# one object per translation unit; compiled side by side, then linked
+SOURCES = ["capi_gemm.hip", "capi_harness.hip", "capi_api_gemm.hip"]
+
+
+def _run(cmd, verbose):
     res = subprocess.run(cmd, stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True)
     if verbose or res.returncode != 0:
         print(res.stdout)
     if res.returncode != 0:
         raise RuntimeError("hipcc failed building libwmmae_tcec.so:\n" + res.stdout[-4000:])
+
+
+def build(verbose=False, only=None):
+    """Compile the HIP sources into LIB_PATH.  Always recompiles every source
+    (`only` = list of source names restricts that to a few, the other objects
+    being reused if present: for work on one kernel)."""
+    from concurrent.futures import ThreadPoolExecutor
+    os.makedirs(LIB_DIR, exist_ok=True)
+    hipcc = os.environ.get("HIPCC", "/opt/rocm/bin/hipcc")
+    flags = [f for f in HIPCC_FLAGS if f != "-shared"]
+    objs, jobs = [], []
+    for name in SOURCES:
+        obj = os.path.join(LIB_DIR, name.replace(".hip", ".o"))
+        objs.append(obj)
+        if only is None or name in only or not os.path.exists(obj):
+            jobs.append([hipcc, *flags, "-I" + INCLUDE_DIR, "-c",
+                         os.path.join(CSRC_DIR, name), "-o", obj])
+    with ThreadPoolExecutor(max_workers=len(SOURCES)) as pool:
+        list(pool.map(lambda c: _run(c, verbose), jobs))
+    _run([hipcc, "--offload-arch=gfx950", "-shared", "-fPIC", *objs, "-o", LIB_PATH], verbose)
     return LIB_PATH
 
 
