@@ -1,7 +1,7 @@
 // Elementwise arithmetic on fragments (reference:
 // include/wmma_extension/operators.hpp:6-58, detail/operators.hpp,
 // docs/ops.md): a + b, a - b, a * s, a / s, fma(s, a, b) = s*a + b and
-// fma(a, s, b) = a*s + b, where s has the fragment's storage element type.
+// fma(a, s, b) = a + s*b, where s has the fragment's storage element type.
 //
 // Every result element is the correctly rounded result in the fragment's
 // element type: half uses native fp16 arithmetic (fp16 fused multiply-add for
@@ -91,12 +91,13 @@ WMMAE_D WMMAE_FRAG fma(const typename WMMAE_FRAG::storage_element_type alpha,
     res.x[i] = ops::fma_elem(alpha, a.x[i], b.x[i]);
   return res;
 }
-// a * alpha + b
+// a + alpha * b (reference: operators.hpp:50-58 forwards (alpha, b, a); its
+// test labels the overload "fma(A+a*B)", test/primitive/operators.cu:211-225)
 template <WMMAE_FRAG_TPARAMS>
 WMMAE_D WMMAE_FRAG fma(const WMMAE_FRAG &a,
                        const typename WMMAE_FRAG::storage_element_type alpha,
                        const WMMAE_FRAG &b) {
-  return fma(alpha, a, b);
+  return fma(alpha, b, a);
 }
 
 #undef WMMAE_FRAG

@@ -83,6 +83,11 @@ struct fragment {
   // main + error; operands keep as many terms as the split produces.
   static constexpr int num_terms =
       !has_ec ? 1 : (is_acc ? 2 : split::num_terms);
+  // (the reference has no default_policy<float, with_ec, ...> either,
+  // tcec/detail/policy.hpp:63-99)
+  static_assert(!has_ec || split::num_terms >= 2,
+                "error correction needs a split of at least two terms: fp32 "
+                "operands (op_simt) go with without_ec");
 
   sub_frag_t sub_frag[num_sub_frags];
   sub_frag_t sub_d_frag[num_terms >= 2 ? num_sub_frags : 0];

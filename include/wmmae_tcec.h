@@ -15,7 +15,9 @@
  *   - `stream` is a hipStream_t passed as void* (NULL = the default stream);
  *     all work is asynchronous on that stream, nothing synchronises
  *   - return value: WMMAE_STATUS_SUCCESS (0) or a negative wmmae_status
- *   - no global state; calls may come from any thread
+ *   - no state a caller could observe (the library remembers, per device, the
+ *     compute-unit count and which kernels it has raised the LDS limit for);
+ *     calls may come from any thread
  *   - matrices follow the column-major BLAS convention; the reference's layout
  *     (A row-major m x k, B column-major k x n, C column-major m x n,
  *     test/tcec/batch_gemm.cu:259-260, 542-543) is transa='T', transb='N',
@@ -284,8 +286,8 @@ int wmmae_gevm(float *y, const float *x, const float *e, void *stream);
 
 /* Elementwise operators on 16x16x16 fragments: a, b are 16x16 row-major fp32
  * tiles cast to the element type on the way in, out is the result fragment
- * cast back.  op: 0 a+b, 1 a-b, 2 a*alpha, 3 a/alpha, 4 fma(alpha,a,b),
- * 5 fma(a,alpha,b); use: 0 matrix_a, 1 matrix_b, 2 accumulator (elem 2 only);
+ * cast back.  op: 0 a+b, 1 a-b, 2 a*alpha, 3 a/alpha, 4 fma(alpha,a,b) =
+ * alpha*a + b, 5 fma(a,alpha,b) = a + alpha*b; use: 0 matrix_a, 1 matrix_b, 2 accumulator (elem 2 only);
  * elem: 0 half, 1 bfloat16, 2 float.
  * Replaces: test/primitive/operators.cu:14-57. */
 int wmmae_fragment_ops(int op, int use, int elem, float alpha, const float *a,

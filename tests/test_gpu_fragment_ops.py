@@ -37,13 +37,14 @@ def test_fragment_operators(tc, dev, elem, use):
     B = rng.uniform(-1, 1, (16, 16)).astype(np.float32)
     a, b = _round(A, elem).astype(np.float64), _round(B, elem).astype(np.float64)
     alpha = 1.5
-    expect = {0: a + b, 1: a - b, 2: a * alpha, 3: a / alpha, 4: alpha * a + b, 5: a * alpha + b}
+    expect = {0: a + b, 1: a - b, 2: a * alpha, 3: a / alpha, 4: alpha * a + b, 5: a + alpha * b}
     dA, dB = torch.from_numpy(A).to(dev), torch.from_numpy(B).to(dev)
     for op in range(6):
         got = tc.fragment_ops(op, use, elem, alpha, dA, dB).cpu().numpy()
         if elem == 1 and op >= 4:
             # bf16 fma: fp32 fused multiply-add, then one rounding to bf16
-            want = _round(np.float32(alpha) * a.astype(np.float32) + b.astype(np.float32), 1)
+            x, y = (a, b) if op == 4 else (b, a)  # op 5 is a + alpha*b (operators.cu:211-225)
+            want = _round(np.float32(alpha) * x.astype(np.float32) + y.astype(np.float32), 1)
             assert np.abs(got - want).max() <= 2.0**-8 * np.abs(want).max()
             continue
         if elem == 2 and op == 3:

@@ -72,6 +72,11 @@ inline wmmae_gemm::PackOperand pack_operand(const PackSource &src,
   return o;
 }
 
+// The batch index of the split, scale and fold kernels is the grid's y
+// coordinate, which ends at 65535: longer batches take one launch per 65535
+// entries.
+constexpr int kMaxGridY = 65535;
+
 // Splits one operand (b == nullptr) or both operands of a product in a single
 // launch.
 template <class T, int TERMS>
@@ -80,24 +85,28 @@ int launch_pack(const int k, const int batch, const PackSource &a,
   const int KT = packed_k_tiles(k);
   const wmmae_gemm::PackOperand oa = pack_operand(a, KT);
   const long long blocks_a = ceil_div(oa.chunks * 64, 256);
-  if (batch > 65535)
-    return WMMAE_STATUS_NOT_SUPPORTED;
   if (b == nullptr) {
     if (blocks_a > 0x7fffffffLL)
       return WMMAE_STATUS_NOT_SUPPORTED;
-    hipLaunchKernelGGL((wmmae_gemm::split_pack_kernel<T, TERMS>),
-                       dim3(static_cast<unsigned>(blocks_a), batch), dim3(256),
-                       0, stream, oa, k, KT);
+    for (int e0 = 0; e0 < batch; e0 += kMaxGridY)
+      hipLaunchKernelGGL((wmmae_gemm::split_pack_kernel<T, TERMS>),
+                         dim3(static_cast<unsigned>(blocks_a),
+                              std::min(batch - e0, kMaxGridY)),
+                         dim3(256), 0, stream, oa, k, KT,
+                         static_cast<unsigned>(e0));
     return launch_status();
   }
   const wmmae_gemm::PackOperand ob = pack_operand(*b, KT);
   const long long blocks_b = ceil_div(ob.chunks * 64, 256);
   if (blocks_a + blocks_b > 0x7fffffffLL)
     return WMMAE_STATUS_NOT_SUPPORTED;
-  hipLaunchKernelGGL((wmmae_gemm::split_pack_pair_kernel<T, TERMS>),
-                     dim3(static_cast<unsigned>(blocks_a + blocks_b), batch),
-                     dim3(256), 0, stream, oa, ob,
-                     static_cast<unsigned>(blocks_a), k, KT);
+  for (int e0 = 0; e0 < batch; e0 += kMaxGridY)
+    hipLaunchKernelGGL((wmmae_gemm::split_pack_pair_kernel<T, TERMS>),
+                       dim3(static_cast<unsigned>(blocks_a + blocks_b),
+                            std::min(batch - e0, kMaxGridY)),
+                       dim3(256), 0, stream, oa, ob,
+                       static_cast<unsigned>(blocks_a), k, KT,
+                       static_cast<unsigned>(e0));
   return launch_status();
 }
 
@@ -138,17 +147,25 @@ struct GemmArgs {
   hipStream_t stream;
 };
 
+// Compute units of the current device, looked up once per device.
 inline int device_cus() {
-  static const int cached = [] {
-    int dev = 0;
-    hipDeviceProp_t prop;
-    if (hipGetDevice(&dev) == hipSuccess &&
-        hipGetDeviceProperties(&prop, dev) == hipSuccess &&
-        prop.multiProcessorCount > 0)
-      return prop.multiProcessorCount;
+  static std::atomic<int> cached[64];
+  int dev = 0;
+  if (hipGetDevice(&dev) != hipSuccess)
     return 256; // MI355X; also the answer when no device is visible
-  }();
-  return cached;
+  const bool tracked = dev >= 0 && dev < 64;
+  if (tracked) {
+    const int c = cached[dev].load(std::memory_order_relaxed);
+    if (c > 0)
+      return c;
+  }
+  hipDeviceProp_t prop;
+  if (hipGetDeviceProperties(&prop, dev) != hipSuccess ||
+      prop.multiProcessorCount <= 0)
+    return 256;
+  if (tracked)
+    cached[dev].store(prop.multiProcessorCount, std::memory_order_relaxed);
+  return prop.multiProcessorCount;
 }
 
 // Number of K slices of every tile, when the 256x128 output tiles cannot fill
@@ -307,7 +324,7 @@ int launch_gemm(const GemmArgs &g) {
   const long long resident = static_cast<long long>(device_cus()) * per_cu;
   int grid = static_cast<int>(std::min(items, resident));
   int entry_per_xcd = 0;
-  if (zdim > 1 && resident % 8 == 0) {
+  if (zdim > 1 && resident >= 8 && resident % 8 == 0) {
     // split-K: eight runs of the item list, one per XCD, so that an XCD holds
     // as few K slices as possible; the grid is padded to whole runs
     entry_per_xcd = 2;
@@ -318,10 +335,13 @@ int launch_gemm(const GemmArgs &g) {
   // (an XCD that owns one entry more than the others must not cost more
   // rounds than the shared list would take: 9 entries of 128 tiles are 8
   // rounds on the XCD with two entries, 5 on the shared list)
-  const long long owned_rounds = ceil_div(
-      static_cast<long long>(tiles_m) * tiles_n * ceil_div(g.batch, 8),
-      resident / 8);
-  if (zdim == 1 && g.batch >= 8 && resident % 8 == 0 &&
+  const bool by_xcd = resident >= 8 && resident % 8 == 0;
+  const long long owned_rounds =
+      by_xcd ? ceil_div(static_cast<long long>(tiles_m) * tiles_n *
+                            ceil_div(g.batch, 8),
+                        resident / 8)
+             : 0;
+  if (zdim == 1 && g.batch >= 8 && by_xcd &&
       owned_rounds * 100 <= ceil_div(items, resident) * 115) {
     // also when every item gets a workgroup of its own: a workgroup for every
     // item of the XCD that owns the most entries
@@ -368,10 +388,14 @@ int launch_gemm(const GemmArgs &g) {
   }
   if (st == WMMAE_STATUS_SUCCESS && zdim > 1) {
     const long long blocks = ceil_div(static_cast<long long>(g.m) * g.n, 256);
-    hipLaunchKernelGGL(wmmae_gemm::reduce_splits_kernel,
-                       dim3(static_cast<unsigned>(blocks), g.batch), dim3(256),
-                       0, g.stream, g.partial, zdim, g.c, g.m, g.n, g.ldc,
-                       g.stride_c, g.c_ptrs, g.alpha, g.beta);
+    for (int e0 = 0; e0 < g.batch; e0 += kMaxGridY)
+      hipLaunchKernelGGL(wmmae_gemm::reduce_splits_kernel,
+                         dim3(static_cast<unsigned>(blocks),
+                              std::min(g.batch - e0, kMaxGridY)),
+                         dim3(256), 0, g.stream, g.partial, zdim, g.c, g.m, g.n,
+                         g.ldc, g.stride_c, g.c_ptrs, g.alpha, g.beta,
+                         static_cast<long long>(g.batch),
+                         static_cast<unsigned>(e0));
     st = launch_status();
   }
   return st;
@@ -721,8 +745,6 @@ int gemm_packed_impl(const int policy, const int m, const int n, const int k,
     return WMMAE_STATUS_NULL_POINTER;
   if (ldc < m)
     return WMMAE_STATUS_BAD_LEADING_DIM;
-  if (batch > 65535)
-    return WMMAE_STATUS_NOT_SUPPORTED;
   if (k > 0 && (reinterpret_cast<uintptr_t>(packed_a) % 16 != 0 ||
                 reinterpret_cast<uintptr_t>(packed_b) % 16 != 0))
     return WMMAE_STATUS_MISALIGNED;
@@ -730,10 +752,13 @@ int gemm_packed_impl(const int policy, const int m, const int n, const int k,
     const long long blocks = ceil_div(static_cast<long long>(m) * n, 256);
     if (blocks > 0x7fffffffLL)
       return WMMAE_STATUS_NOT_SUPPORTED;
-    hipLaunchKernelGGL(wmmae_gemm::scale_c_kernel,
-                       dim3(static_cast<unsigned>(blocks), batch), dim3(256), 0,
-                       static_cast<hipStream_t>(stream), C, m, n,
-                       static_cast<long long>(ldc), stride_c, c_ptrs, *beta);
+    for (int e0 = 0; e0 < batch; e0 += kMaxGridY)
+      hipLaunchKernelGGL(wmmae_gemm::scale_c_kernel,
+                         dim3(static_cast<unsigned>(blocks),
+                              std::min(batch - e0, kMaxGridY)),
+                         dim3(256), 0, static_cast<hipStream_t>(stream), C, m, n,
+                         static_cast<long long>(ldc), stride_c, c_ptrs, *beta,
+                         static_cast<unsigned>(e0));
     return launch_status();
   }
   GemmArgs g;

@@ -56,8 +56,9 @@ __host__ __device__ constexpr int reads_due(const int count, const int span,
 // split_pack_kernel: X (fp32, element (r,k) at X[r*row_stride + k*k_stride])
 // -> packed terms.  One thread per (chunk, lane).  Rows >= rows and k >= K are
 // zero filled, so the GEMM kernel needs no edge handling on its loads.
-// Batch entry y (blockIdx.y) reads X + y*batch_stride, or ptrs[y] when ptrs is
-// set (the reference's harness passes arrays of matrix pointers,
+// Batch entry y (entry0 + blockIdx.y: a launch covers at most 65535 entries,
+// the host loops over longer batches) reads X + y*batch_stride, or ptrs[y]
+// when ptrs is set (the reference's harness passes arrays of matrix pointers,
 // test/tcec/batch_gemm.cu:433-443).
 //   T      : split tag (half, bfloat16, precision::tf32)
 //   TERMS  : number of terms stored (1 = leading term only, i.e. no correction)
@@ -137,8 +138,9 @@ __device__ __forceinline__ void split_pack_block(const PackOperand &o,
 
 template <class T, int TERMS>
 __global__ void __launch_bounds__(256)
-    split_pack_kernel(const PackOperand o, const int K, const int KT) {
-  split_pack_block<T, TERMS>(o, K, KT, blockIdx.x, blockIdx.y);
+    split_pack_kernel(const PackOperand o, const int K, const int KT,
+                      const unsigned entry0) {
+  split_pack_block<T, TERMS>(o, K, KT, blockIdx.x, entry0 + blockIdx.y);
 }
 
 // Both operands of a product in one launch (the GEMM entry points pack A and B
@@ -147,11 +149,13 @@ __global__ void __launch_bounds__(256)
 template <class T, int TERMS>
 __global__ void __launch_bounds__(256)
     split_pack_pair_kernel(const PackOperand a, const PackOperand b,
-                           const unsigned blocks_a, const int K, const int KT) {
+                           const unsigned blocks_a, const int K, const int KT,
+                           const unsigned entry0) {
   if (blockIdx.x < blocks_a)
-    split_pack_block<T, TERMS>(a, K, KT, blockIdx.x, blockIdx.y);
+    split_pack_block<T, TERMS>(a, K, KT, blockIdx.x, entry0 + blockIdx.y);
   else
-    split_pack_block<T, TERMS>(b, K, KT, blockIdx.x - blocks_a, blockIdx.y);
+    split_pack_block<T, TERMS>(b, K, KT, blockIdx.x - blocks_a,
+                               entry0 + blockIdx.y);
 }
 
 // --------------------------------------------------------------------------
@@ -160,12 +164,14 @@ __global__ void __launch_bounds__(256)
 __global__ void __launch_bounds__(256)
     scale_c_kernel(float *__restrict__ C, const int M, const int N,
                    const long long ldc, const long long batch_stride_c,
-                   float *const *__restrict__ c_ptrs, const float beta) {
+                   float *const *__restrict__ c_ptrs, const float beta,
+                   const unsigned entry0) {
   const long long e = static_cast<long long>(blockIdx.x) * 256 + threadIdx.x;
   if (e >= static_cast<long long>(M) * N)
     return;
+  const long long entry = entry0 + blockIdx.y;
   float *const cb =
-      c_ptrs != nullptr ? c_ptrs[blockIdx.y] : C + blockIdx.y * batch_stride_c;
+      c_ptrs != nullptr ? c_ptrs[entry] : C + entry * batch_stride_c;
   float *const p = cb + (e % M) + (e / M) * ldc;
   *p = beta == 0.f ? 0.f : beta * *p;
 }
@@ -181,17 +187,18 @@ __global__ void __launch_bounds__(256)
                          float *__restrict__ C, const int M, const int N,
                          const long long ldc, const long long batch_stride_c,
                          float *const *__restrict__ c_ptrs, const float alpha,
-                         const float beta) {
+                         const float beta, const long long batches,
+                         const unsigned entry0) {
   const long long e = static_cast<long long>(blockIdx.x) * 256 + threadIdx.x;
   const long long mn = static_cast<long long>(M) * N;
   if (e >= mn)
     return;
-  const long long batches = gridDim.y;
+  const long long entry = entry0 + blockIdx.y;
   double s = 0.;
   for (int z = 0; z < splits; z++)
-    s += static_cast<double>(partial[(z * batches + blockIdx.y) * mn + e]);
+    s += static_cast<double>(partial[(z * batches + entry) * mn + e]);
   float *const cb =
-      c_ptrs != nullptr ? c_ptrs[blockIdx.y] : C + blockIdx.y * batch_stride_c;
+      c_ptrs != nullptr ? c_ptrs[entry] : C + entry * batch_stride_c;
   float *const p = cb + (e % M) + (e / M) * ldc;
   const float v = alpha * static_cast<float>(s);
   *p = beta == 0.f ? v : v + beta * *p;

@@ -47,6 +47,48 @@ def _need_cuda(*tensors):
             raise ValueError("device tensors required")
 
 
+def _room(t):
+    """Bytes from t's first element to the end of its storage."""
+    return t.untyped_storage().nbytes() - t.storage_offset() * t.element_size()
+
+
+def _check_matrix(name, t, rows, cols, ld, batch=1, stride=0, device=None):
+    """A column-major rows x cols fp32 matrix (leading dimension ld, `batch` of them `stride`
+    apart) must lie inside the tensor's storage: the kernels take raw pointers, so a wrong dtype
+    or a short tensor would read or write out of bounds on the GPU."""
+    if t is None:
+        return
+    if t.dtype != torch.float32:
+        raise ValueError(f"{name}: float32 tensor required, got {t.dtype}")
+    if device is not None and t.device != device:
+        raise ValueError(f"{name}: on {t.device}, expected {device}")
+    if rows <= 0 or cols <= 0 or batch <= 0:
+        return
+    if stride < 0:
+        raise ValueError(f"{name}: negative batch stride")
+    need = ((batch - 1) * stride + (cols - 1) * ld + rows) * 4
+    if ld >= rows and _room(t) < need:
+        raise ValueError(f"{name}: needs {need} bytes from its first element, tensor has {_room(t)}")
+
+
+def _check_gemm_operands(transa, transb, m, n, k, A, lda, B, ldb, C, ldc, batch=1,
+                         stride_a=0, stride_b=0, stride_c=0):
+    dev = C.device if C is not None else None
+    ta, tb = transa in "Nn", transb in "Nn"
+    _check_matrix("A", A, m if ta else k, k if ta else m, lda, batch, stride_a, dev)
+    _check_matrix("B", B, k if tb else n, n if tb else k, ldb, batch, stride_b, dev)
+    _check_matrix("C", C, m, n, ldc, batch, stride_c, dev)
+
+
+def _check_bytes(name, t, need, device=None):
+    if t is None:
+        return
+    if device is not None and t.device != device:
+        raise ValueError(f"{name}: on {t.device}, expected {device}")
+    if _room(t) < need:
+        raise ValueError(f"{name}: needs {need} bytes, tensor has {_room(t)}")
+
+
 def query(what):
     out = ctypes.c_longlong(0)
     _lib.check(_lib.lib().wmmae_query(int(what), ctypes.byref(out)), "wmmae_query")
@@ -83,6 +125,7 @@ def sgemm(transa, transb, m, n, k, alpha, A, lda, B, ldb, beta, C, ldc,
           policy=Policy.F16_EC, flags=0, workspace=None):
     """C = alpha*op(A)*op(B) + beta*C, column-major BLAS convention."""
     _need_cuda(A, B, C, workspace)
+    _check_gemm_operands(transa, transb, m, n, k, A, lda, B, ldb, C, ldc)
     ws_bytes = workspace.numel() * workspace.element_size() if workspace is not None else 0
     st = _lib.lib().wmmae_tcec_sgemm(transa.encode(), transb.encode(), m, n, k, _f(alpha),
                                      _ptr(A), lda, _ptr(B), ldb, _f(beta), _ptr(C), ldc,
@@ -94,6 +137,8 @@ def sgemm_strided_batched(transa, transb, m, n, k, alpha, A, lda, stride_a, B, l
                           beta, C, ldc, stride_c, batch, policy=Policy.F16_EC, flags=0,
                           workspace=None):
     _need_cuda(A, B, C, workspace)
+    _check_gemm_operands(transa, transb, m, n, k, A, lda, B, ldb, C, ldc, batch,
+                         stride_a, stride_b, stride_c)
     ws_bytes = workspace.numel() * workspace.element_size() if workspace is not None else 0
     st = _lib.lib().wmmae_tcec_sgemm_strided_batched(
         transa.encode(), transb.encode(), m, n, k, _f(alpha), _ptr(A), lda, stride_a,
@@ -107,6 +152,9 @@ def sgemm_batched(transa, transb, m, n, k, alpha, A_array, lda, B_array, ldb, be
     """A_array / B_array / C_array: int64 device tensors holding `batch` device pointers
     (the launch_bgemm / cublasSgemmBatched convention)."""
     _need_cuda(A_array, B_array, C_array, workspace)
+    for name, arr in (("A_array", A_array), ("B_array", B_array), ("C_array", C_array)):
+        if arr is not None and (arr.dtype != torch.int64 or arr.numel() < batch):
+            raise ValueError(f"{name}: int64 tensor of at least {batch} device pointers required")
     ws_bytes = workspace.numel() * workspace.element_size() if workspace is not None else 0
     st = _lib.lib().wmmae_tcec_sgemm_batched(
         transa.encode(), transb.encode(), m, n, k, _f(alpha), _ptr(A_array), lda, _ptr(B_array), ldb,
@@ -116,6 +164,11 @@ def sgemm_batched(transa, transb, m, n, k, alpha, A_array, lda, B_array, ldb, be
 
 def pack(policy, rows, k, X, row_stride, k_stride, packed, batch=1, batch_stride=0):
     _need_cuda(X, packed)
+    if X is not None and X.dtype != torch.float32:
+        raise ValueError(f"X: float32 tensor required, got {X.dtype}")
+    if X is not None and rows > 0 and k > 0 and batch > 0 and min(row_stride, k_stride, batch_stride) >= 0:
+        _check_bytes("X", X, 4 * ((batch - 1) * batch_stride + (rows - 1) * row_stride
+                                  + (k - 1) * k_stride + 1), packed.device)
     st = _lib.lib().wmmae_tcec_pack(int(policy), rows, k, _ptr(X), row_stride, k_stride,
                                     batch_stride, batch, _ptr(packed),
                                     packed.numel() * packed.element_size(), _stream())
@@ -133,6 +186,10 @@ def gemm_packed_workspace_bytes(policy, m, n, k, batch=1):
 def gemm_packed(policy, m, n, k, alpha, packed_a, packed_b, beta, C, ldc, batch=1,
                 stride_c=0, flags=0, workspace=None):
     _need_cuda(packed_a, packed_b, C, workspace)
+    _check_matrix("C", C, m, n, ldc, batch, stride_c)
+    if k > 0 and m > 0 and n > 0 and batch > 0:
+        _check_bytes("packed_a", packed_a, pack_bytes(m, k, batch, policy), C.device)
+        _check_bytes("packed_b", packed_b, pack_bytes(n, k, batch, policy), C.device)
     ws_bytes = workspace.numel() * workspace.element_size() if workspace is not None else 0
     st = _lib.lib().wmmae_tcec_gemm_packed(int(policy), m, n, k, _f(alpha), _ptr(packed_a),
                                            _ptr(packed_b), _f(beta), _ptr(C), ldc, stride_c,
@@ -149,6 +206,8 @@ def matmul_tn(A, B, policy=Policy.F16_EC, flags=0, workspace=None, out=None):
     assert k == k2 and A.is_contiguous() and B.is_contiguous()
     if out is None:
         out = torch.empty((n, m), dtype=torch.float32, device=A.device)
+    elif tuple(out.shape) != (n, m) or not out.is_contiguous():
+        raise ValueError(f"out: contiguous ({n}, {m}) tensor required, got {tuple(out.shape)}")
     sgemm("T", "N", m, n, k, 1.0, A, k, B, k, 0.0, out, m, policy, flags, workspace)
     return out
 
@@ -235,8 +294,9 @@ def elementwise(type_, ec, inst, base, do_neg, do_integrate, device="cuda"):
 
 
 def api_gemm(type_, ec, m, n, k, alpha, A, lda, B, ldb, beta, C, ldc):
-    """Tiled GEMM written against the public device API only (comparator)."""
+    """Tiled GEMM written against the public device API only."""
     _need_cuda(A, B, C)
+    _check_gemm_operands("T", "N", m, n, k, A, lda, B, ldb, C, ldc)
     st = _lib.lib().wmmae_tcec_api_gemm(type_, int(ec), m, n, k, _f(alpha), _ptr(A), lda, _ptr(B), ldb,
                                         _f(beta), _ptr(C), ldc, _stream())
     _lib.check(st, "wmmae_tcec_api_gemm")
