@@ -127,6 +127,26 @@ int wmmae_tcec_sgemm_strided_batched(char transa, char transb, int m, int n,
                                      void *workspace, size_t workspace_bytes,
                                      void *stream);
 
+/* wmmae_tcec_sgemm for callers that cannot allocate device memory (code under
+ * HIP graph capture, tight serving loops, harnesses that forbid hipMalloc).
+ * No counterpart in the reference.  Same arguments and results as
+ * wmmae_tcec_sgemm; the workspace is a fixed device array of
+ * WMMAE_STATIC_SCRATCH_BYTES inside the library image (every GPU the library
+ * runs on holds it until the process ends), so the call makes no hipMalloc /
+ * hipFree of any kind.  Products whose split operands need more
+ * (wmmae_tcec_sgemm_workspace_bytes; fp16 hi+lo: 4*(m+n)*k bytes rounded up to
+ * 16 rows and 32 of k) return WMMAE_STATUS_WORKSPACE_TOO_SMALL; K slices are
+ * made only when they fit next to the operands.  All calls on one GPU share
+ * the one array: calls that overlap in time on the same GPU (two streams, two
+ * threads) race and must be serialised by the caller.  Nothing in the array
+ * has to survive between calls and nothing is assumed zero. */
+#define WMMAE_STATIC_SCRATCH_BYTES (64u << 20)
+int wmmae_tcec_sgemm_static(char transa, char transb, int m, int n, int k,
+                            const float *alpha, const float *A, int lda,
+                            const float *B, int ldb, const float *beta,
+                            float *C, int ldc, int policy, int flags,
+                            void *stream);
+
 /* Batched product on device arrays of matrix pointers, the calling convention
  * of the reference's launch_bgemm(conf, m, n, k, alpha, a_ptr_array, lda,
  * b_ptr_array, ldb, beta, c_ptr_array, ldc, batch) (batch_gemm.cu:433-443) and

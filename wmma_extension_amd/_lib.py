@@ -31,6 +31,7 @@ EXPORTS = [
     "wmmae_tcec_sgemm_workspace_bytes",
     "wmmae_tcec_sgemm_path",
     "wmmae_tcec_sgemm",
+    "wmmae_tcec_sgemm_static",
     "wmmae_tcec_sgemm_strided_batched",
     "wmmae_tcec_sgemm_batched",
     "wmmae_tcec_pack_bytes",
@@ -105,6 +106,8 @@ _SIGNATURES = {
     "wmmae_tcec_sgemm_path": (_i, [_i, _i, _i, _i, _i, _i, _c.POINTER(_i)]),
     "wmmae_tcec_sgemm": (_i, [_c.c_char, _c.c_char, _i, _i, _i, _fp, _vp, _i, _vp, _i, _fp,
                               _vp, _i, _i, _i, _vp, _sz, _vp]),
+    "wmmae_tcec_sgemm_static": (_i, [_c.c_char, _c.c_char, _i, _i, _i, _fp, _vp, _i, _vp, _i, _fp,
+                                     _vp, _i, _i, _i, _vp]),
     "wmmae_tcec_sgemm_strided_batched": (_i, [_c.c_char, _c.c_char, _i, _i, _i, _fp, _vp, _i, _ll,
                                               _vp, _i, _ll, _fp, _vp, _i, _ll, _i, _i, _i,
                                               _vp, _sz, _vp]),

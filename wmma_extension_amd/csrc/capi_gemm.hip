@@ -1058,6 +1058,58 @@ int wmmae_tcec_sgemm_batched(const char transa, const char transb, const int m,
                     batch, policy, flags, workspace, workspace_bytes, stream);
 }
 
+// ---------------------------------------------- entry point that allocates
+// nothing: the workspace is a device array that is part of the library image.
+// Each GPU holds its own copy at its own address; in host code the array's
+// name is only a handle for hipGetSymbolAddress, never a device address.
+} // extern "C"
+
+namespace {
+constexpr size_t kStaticScratchBytes = WMMAE_STATIC_SCRATCH_BYTES;
+static __device__ __align__(256) unsigned char scratch[kStaticScratchBytes];
+
+// Device address of `scratch` on the current device, looked up once per
+// device (with that device current) and kept.
+int static_scratch(void **const out) {
+  static std::atomic<void *> ptrs[64];
+  int dev = 0;
+  WMMAE_HIP_TRY(hipGetDevice(&dev));
+  if (dev < 0 || dev >= 64)
+    return WMMAE_STATUS_NOT_SUPPORTED;
+  void *p = ptrs[dev].load(std::memory_order_acquire);
+  if (p == nullptr) {
+    WMMAE_HIP_TRY(
+        hipGetSymbolAddress(reinterpret_cast<void **>(&p), HIP_SYMBOL(scratch)));
+    if (p == nullptr)
+      return WMMAE_STATUS_RUNTIME_ERROR;
+    ptrs[dev].store(p, std::memory_order_release);
+  }
+  *out = p;
+  return WMMAE_STATUS_SUCCESS;
+}
+} // namespace
+
+extern "C" {
+
+int wmmae_tcec_sgemm_static(const char transa, const char transb, const int m,
+                            const int n, const int k, const float *const alpha,
+                            const float *const A, const int lda,
+                            const float *const B, const int ldb,
+                            const float *const beta, float *const C,
+                            const int ldc, const int policy, const int flags,
+                            void *const stream) {
+  void *ws = nullptr;
+  const int st = static_scratch(&ws);
+  if (st != WMMAE_STATUS_SUCCESS)
+    return st;
+  // sgemm_impl allocates only when it is handed no workspace; with one it
+  // returns WMMAE_STATUS_WORKSPACE_TOO_SMALL when the split operands do not
+  // fit, and makes K slices only if they fit as well
+  return sgemm_impl(transa, transb, m, n, k, alpha, A, nullptr, lda, 0, B,
+                    nullptr, ldb, 0, beta, C, nullptr, ldc, 0, 1, policy, flags,
+                    ws, kStaticScratchBytes, stream);
+}
+
 int wmmae_tcec_sgemm(const char transa, const char transb, const int m,
                      const int n, const int k, const float *const alpha,
                      const float *const A, const int lda, const float *const B,

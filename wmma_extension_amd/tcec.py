@@ -133,6 +133,20 @@ def sgemm(transa, transb, m, n, k, alpha, A, lda, B, ldb, beta, C, ldc,
     _lib.check(st, "wmmae_tcec_sgemm")
 
 
+STATIC_SCRATCH_BYTES = 64 << 20
+
+
+def sgemm_static(transa, transb, m, n, k, alpha, A, lda, B, ldb, beta, C, ldc,
+                 policy=Policy.F16_EC, flags=0):
+    """sgemm on the library's own fixed workspace: allocates nothing."""
+    _need_cuda(A, B, C)
+    _check_gemm_operands(transa, transb, m, n, k, A, lda, B, ldb, C, ldc)
+    st = _lib.lib().wmmae_tcec_sgemm_static(transa.encode(), transb.encode(), m, n, k, _f(alpha),
+                                            _ptr(A), lda, _ptr(B), ldb, _f(beta), _ptr(C), ldc,
+                                            int(policy), flags, _stream())
+    _lib.check(st, "wmmae_tcec_sgemm_static")
+
+
 def sgemm_strided_batched(transa, transb, m, n, k, alpha, A, lda, stride_a, B, ldb, stride_b,
                           beta, C, ldc, stride_c, batch, policy=Policy.F16_EC, flags=0,
                           workspace=None):
