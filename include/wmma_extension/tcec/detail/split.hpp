@@ -74,6 +74,44 @@ template <> struct split_traits<float> {
   }
 };
 
+// split4: split() applied to four values at once.  The arithmetic per element
+// is that of split_traits<T>::split; it is written on two-element vectors so
+// that the packed conversions (v_cvt_pk_f16_f32 / v_cvt_pk_bf16_f32) are used.
+typedef float f32x2_t __attribute__((ext_vector_type(2)));
+typedef float f32x4_t __attribute__((ext_vector_type(4)));
+template <class T, class S = typename split_traits<T>::storage>
+WMMAE_HD void split4(const f32x4_t v, S *const t0, S *const t1, S *const t2) {
+  using traits = split_traits<T>;
+  if constexpr (std::is_same<S, float>::value) {
+#pragma unroll
+    for (int e = 0; e < 4; e++)
+      t0[e] = v[e];
+  } else {
+    typedef S s2_t __attribute__((ext_vector_type(2)));
+#pragma unroll
+    for (int e = 0; e < 4; e += 2) {
+      const f32x2_t vv = {v[e], v[e + 1]};
+      const s2_t h0 = __builtin_convertvector(vv, s2_t);
+      t0[e] = h0[0];
+      t0[e + 1] = h0[1];
+      if constexpr (traits::num_terms >= 2) {
+        f32x2_t r = vv - __builtin_convertvector(h0, f32x2_t);
+        if constexpr (traits::scale != 1.f)
+          r *= traits::scale;
+        const s2_t h1 = __builtin_convertvector(r, s2_t);
+        t1[e] = h1[0];
+        t1[e + 1] = h1[1];
+        if constexpr (traits::num_terms >= 3) {
+          const s2_t h2 = __builtin_convertvector(
+              r - __builtin_convertvector(h1, f32x2_t), s2_t);
+          t2[e] = h2[0];
+          t2[e + 1] = h2[1];
+        }
+      }
+    }
+  }
+}
+
 // Scale applied to the residual before rounding it (0) and removed when the
 // error accumulator is folded back (1) (reference: tcec/detail/scale.hpp:8-20).
 template <class T> WMMAE_HD float correction_scale_0(const float v) {

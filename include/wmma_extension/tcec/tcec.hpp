@@ -149,6 +149,39 @@ WMMAE_D void put_split(Frag &frag, const unsigned block,
     frag.sub_d2_frag[block].x[frag_index] = t2;
 }
 
+// Operand sub-fragments keep runs of four consecutive k of one row (matrix_a)
+// or one column (matrix_b) in registers 4q .. 4q+3 of a lane (a lane of the
+// 16x16x32 instruction owns eight consecutive k).  When k is the contiguous
+// direction of the memory being read - row-major memory for matrix_a,
+// column-major for matrix_b: the layout of the reference's GEMM
+// (test/tcec/batch_gemm.cu:259-260) - such a run is 16 contiguous bytes.
+template <class L, bool is_a> constexpr bool k_runs_of_four() {
+  if (L::num_elements % 4 != 0)
+    return false;
+  for (unsigned lane = 0; lane < wave_size; lane++)
+    for (unsigned x = 0; x < L::num_elements; x += 4)
+      for (unsigned e = 0; e < 4; e++) {
+        const unsigned fixed0 = is_a ? L::row(lane, x) : L::col(lane, x);
+        const unsigned fixed = is_a ? L::row(lane, x + e) : L::col(lane, x + e);
+        const unsigned k0 = is_a ? L::col(lane, x) : L::row(lane, x);
+        const unsigned kk = is_a ? L::col(lane, x + e) : L::row(lane, x + e);
+        if (fixed != fixed0 || k0 % 4 != 0 || kk != k0 + e)
+          return false;
+      }
+  return true;
+}
+template <class F, class MatrixLayout, class MEM_T> struct operand_quads {
+  static constexpr bool is_a = std::is_same<typename F::sub_frag_t::use,
+                                            matrix_a>::value;
+  static constexpr bool value =
+      !F::is_acc &&
+      std::is_same<typename std::remove_cv<MEM_T>::type, float>::value &&
+      std::is_same<MatrixLayout,
+                   typename std::conditional<is_a, row_major,
+                                             col_major>::type>::value &&
+      k_runs_of_four<typename F::sub_frag_t::layout_model, is_a>();
+};
+
 // Value an accumulator element stands for.
 template <class Frag>
 WMMAE_D float combined(const Frag &frag, const unsigned block,
@@ -221,6 +254,75 @@ WMMAE_D void load_matrix_sync_with_mul(WMMAE_TCEC_FRAG(Use, Layout) & frag,
   constexpr unsigned bm_size =
       detail::select_value<Use, fm, fk, fm>::value; // rows of one sub-block
   constexpr unsigned bn_size = detail::select_value<Use, fk, fn, fn>::value;
+  if constexpr (F::is_acc && std::is_same<MatrixLayout, col_major>::value &&
+                mtk::wmma::detail::acc_quads<fm, fn, fk, float,
+                                             MEM_T>::value) {
+    // column-major fp32 memory, four consecutive rows per register quad
+    if (mtk::wmma::detail::quad_aligned(ptr, ldm)) {
+      using L = typename F::sub_frag_t::layout_model;
+      const unsigned lane = mtk::wmma::detail::common::get_lane_id();
+#pragma unroll
+      for (unsigned bn = 0; bn < unsigned(F::num_sub_frag_n); bn++) {
+#pragma unroll
+        for (unsigned bm = 0; bm < unsigned(F::num_sub_frag_m); bm++) {
+          const unsigned block = bm + F::num_sub_frag_m * bn;
+#pragma unroll
+          for (unsigned x = 0; x < L::num_elements; x += 4) {
+            const detail::f32x4_t v =
+                *reinterpret_cast<const detail::f32x4_t *>(
+                    ptr + detail::mem_offset<col_major>(
+                              L::row(lane, x), L::col(lane, x), ldm,
+                              bm * bm_size, bn * bn_size)) *
+                static_cast<float>(mul);
+#pragma unroll
+            for (unsigned e = 0; e < 4; e++) {
+              frag.sub_frag[block].x[x + e] = v[e];
+              if constexpr (F::num_terms >= 2)
+                frag.sub_d_frag[block].x[x + e] = 0.f;
+            }
+          }
+        }
+      }
+      return;
+    }
+  }
+  if constexpr (detail::operand_quads<F, MatrixLayout, MEM_T>::value) {
+    // k contiguous in memory, base and leading dimension keeping every run
+    // of four k 16-byte aligned: one 16-byte read per four registers, split
+    // two elements at a time (same arithmetic, same bits as the path below)
+    if (mtk::wmma::detail::quad_aligned(ptr, ldm)) {
+      using L = typename F::sub_frag_t::layout_model;
+      const unsigned lane = mtk::wmma::detail::common::get_lane_id();
+#pragma unroll
+      for (unsigned bn = 0; bn < unsigned(F::num_sub_frag_n); bn++) {
+#pragma unroll
+        for (unsigned bm = 0; bm < unsigned(F::num_sub_frag_m); bm++) {
+          const unsigned block = bm + F::num_sub_frag_m * bn;
+#pragma unroll
+          for (unsigned x = 0; x < L::num_elements; x += 4) {
+            const unsigned off = detail::mem_offset<MatrixLayout>(
+                L::row(lane, x), L::col(lane, x), ldm, bm * bm_size,
+                bn * bn_size);
+            const detail::f32x4_t v =
+                *reinterpret_cast<const detail::f32x4_t *>(ptr + off) *
+                static_cast<float>(mul);
+            typename F::storage_t *d1 = nullptr, *d2 = nullptr;
+            if constexpr (F::num_terms >= 2)
+              d1 = &frag.sub_d_frag[block].x[x];
+            if constexpr (F::num_terms >= 3)
+              d2 = &frag.sub_d2_frag[block].x[x];
+            if constexpr (F::num_terms == F::split::num_terms) {
+              detail::split4<T>(v, &frag.sub_frag[block].x[x], d1, d2);
+            } else { // without_ec: the leading term only
+              typename F::storage_t t1[4], t2[4];
+              detail::split4<T>(v, &frag.sub_frag[block].x[x], t1, t2);
+            }
+          }
+        }
+      }
+      return;
+    }
+  }
   mtk::wmma::foreach_ij<typename F::sub_frag_t>(
       [&](const unsigned *list, const unsigned, const unsigned i,
           const unsigned j) {
@@ -304,6 +406,34 @@ store_matrix_sync_with_mul(MEM_T *const ptr,
                            const unsigned ldm, const MEM_T mul,
                            const bool = true) {
   using F = WMMAE_TCEC_FRAG(accumulator, void);
+  if constexpr (std::is_same<Layout, col_major>::value &&
+                mtk::wmma::detail::acc_quads<fm, fn, fk, float,
+                                             MEM_T>::value) {
+    if (mtk::wmma::detail::quad_aligned(ptr, ldm)) {
+      using L = typename F::sub_frag_t::layout_model;
+      const unsigned lane = mtk::wmma::detail::common::get_lane_id();
+#pragma unroll
+      for (unsigned bn = 0; bn < unsigned(F::num_sub_frag_n); bn++) {
+#pragma unroll
+        for (unsigned bm = 0; bm < unsigned(F::num_sub_frag_m); bm++) {
+          const unsigned block = bm + F::num_sub_frag_m * bn;
+#pragma unroll
+          for (unsigned x = 0; x < L::num_elements; x += 4) {
+            detail::f32x4_t v;
+#pragma unroll
+            for (unsigned e = 0; e < 4; e++)
+              v[e] = detail::combined(frag, block, x + e) *
+                     static_cast<float>(mul);
+            *reinterpret_cast<detail::f32x4_t *>(
+                ptr + detail::mem_offset<col_major>(L::row(lane, x),
+                                                    L::col(lane, x), ldm,
+                                                    bm * fm, bn * fn)) = v;
+          }
+        }
+      }
+      return;
+    }
+  }
   mtk::wmma::foreach_ij<typename F::sub_frag_t>(
       [&](const unsigned *list, const unsigned, const unsigned i,
           const unsigned j) {

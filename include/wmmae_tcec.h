@@ -261,16 +261,26 @@ int wmmae_tcec_elementwise(int type, int ec, int inst, float *out, float base,
                            int do_neg, int do_integrate, void *stream);
 
 /* C = alpha*A*B + beta*C by a tiled kernel written only against the public
- * tcec:: device API (fp32 tiles in LDS, split at fragment load in every wave).
+ * tcec:: device API: fp32 tiles staged in LDS by utils::cp_async (two stages),
+ * split at fragment load in every wave (tcec::load_matrix_sync), tcec::mma_sync.
  * A row-major m x k (lda), B column-major k x n (ldb), C column-major (ldc);
  * m, n multiples of 128, k of 32, lda/ldb multiples of 4, 16-byte aligned.
  * type/ec as in wmmae_tcec_mma_tile.
- * Replaces: bgemm_kernel + mma_core, test/tcec/batch_gemm.cu:196-386, kept as
- * the API-level comparator of wmmae_tcec_sgemm. */
+ * Replaces: bgemm_kernel + mma_core + dmem2smem, test/tcec/batch_gemm.cu:74-116,
+ * 196-386: what a user of the headers gets, beside wmmae_tcec_sgemm. */
 int wmmae_tcec_api_gemm(int type, int ec, int m, int n, int k,
                         const float *alpha, const float *A, int lda,
                         const float *B, int ldb, const float *beta, float *C,
                         int ldc, void *stream);
+/* The same kernel on device arrays of `batch` matrix pointers (each 16-byte
+ * aligned), the calling convention of the reference's launch_bgemm
+ * (test/tcec/batch_gemm.cu:433-443). */
+int wmmae_tcec_api_gemm_batched(int type, int ec, int m, int n, int k,
+                                const float *alpha,
+                                const float *const *A_array, int lda,
+                                const float *const *B_array, int ldb,
+                                const float *beta, float *const *C_array,
+                                int ldc, int batch, void *stream);
 
 /* One-wave complex TCEC product D = A*B (+C), m = n = k = 32, operands in
  * tcec::fragment_complex (16x16x32 policy; 16x16x16 for type 3).  a, b, c, d:

@@ -46,6 +46,7 @@ EXPORTS = [
     "wmmae_tcec_frag_dump",
     "wmmae_tcec_elementwise",
     "wmmae_tcec_api_gemm",
+    "wmmae_tcec_api_gemm_batched",
     "wmmae_tcec_mma_complex",
     "wmmae_primitive_mma",
     "wmmae_foreach_ec",
@@ -126,6 +127,7 @@ _SIGNATURES = {
     "wmmae_tcec_frag_dump": (_i, [_i, _i, _i, _i, _vp, _vp, _i, _i, _vp]),
     "wmmae_tcec_elementwise": (_i, [_i, _i, _i, _vp, _c.c_float, _i, _i, _vp]),
     "wmmae_tcec_api_gemm": (_i, [_i, _i, _i, _i, _i, _fp, _vp, _i, _vp, _i, _fp, _vp, _i, _vp]),
+    "wmmae_tcec_api_gemm_batched": (_i, [_i, _i, _i, _i, _i, _fp, _vp, _i, _vp, _i, _fp, _vp, _i, _i, _vp]),
     "wmmae_tcec_mma_complex": (_i, [_i, _i, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _c.c_float, _vp]),
     "wmmae_primitive_mma": (_i, [_i, _i, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _vp]),
     "wmmae_foreach_ec": (_i, [_vp, _vp, _vp, _vp]),

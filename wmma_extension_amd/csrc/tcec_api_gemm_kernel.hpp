@@ -1,6 +1,26 @@
-// A tiled SGEMM written only against the public device API of this library
-// (tcec::fragment, load_matrix_sync, mma_sync, store_matrix_sync,
-// utils::cp_async), the way a user of the reference writes one.
+// A tiled, batched SGEMM written only against the public device API of this
+// library (tcec::fragment, load_matrix_sync, mma_sync, store_matrix_sync,
+// utils::cp_async), the way a user of the reference writes one: the shape of
+// the reference's bgemm_kernel / mma_core / dmem2smem
+// (test/tcec/batch_gemm.cu:74-116, 196-257, 261-386).
+//
+//   * fp32 tiles of A (row-major) and B (column-major) are staged in LDS by
+//     utils::cp_async, two stages: the copies of stage s+1 are in flight while
+//     stage s is multiplied;
+//   * every wave splits the elements it needs while loading its fragments
+//     (tcec::load_matrix_sync; k is contiguous in both tiles, so the loads
+//     are 16 bytes wide) and multiplies with tcec::mma_sync;
+//   * the operand fragments are double buffered over the k steps of a stage.
+//
+// Rows of a staged tile are SK + 4 floats apart: sixteen lanes reading 16
+// bytes of sixteen consecutive rows then cover all 64 LDS banks once.  The
+// direct global->LDS copy of gfx950 writes lane-linear destinations only, so
+// the copy walks the padded tile image linearly, 16 bytes per lane, and lets
+// the lanes that land on a row's padding fetch that row's last piece again.
+//
+// Two workgroups of four waves share a compute unit (72 KiB of LDS and at
+// most 256 registers each), so that one wave's conversion arithmetic runs
+// beside another's MFMAs.
 #pragma once
 #include <wmma_extension/tcec/tcec.hpp>
 #include <wmma_extension/utils.hpp>
@@ -8,68 +28,144 @@
 namespace wmmae_harness {
 namespace w = mtk::wmma;
 namespace tcec = mtk::wmma::tcec;
+namespace cpa = mtk::wmma::utils::cp_async;
 
-// --------------------------------------------------------------------------
-// A tiled SGEMM written only against the public tcec:: API, the way a user of
-// the reference writes one (reference: bgemm_kernel / mma_core,
-// test/tcec/batch_gemm.cu:196-386): fp32 tiles are staged in LDS, every wave
-// splits the elements it needs while loading its fragments
-// (tcec::load_matrix_sync), multiplies with tcec::mma_sync and writes the
-// result with the element accessors.  A is row-major m x k (lda), B is
-// column-major k x n (ldb), C column-major (ldc); m, n multiples of 128, k of 32.
-// It exists to show the drop-in at GEMM scale and as the comparator for the
-// packed-operand driver, which does the split once per element instead.
-// --------------------------------------------------------------------------
+struct ApiGemmShape {
+  static constexpr int BM = 128, BN = 128; // block tile
+  static constexpr int SK = 32;            // k per stage
+  static constexpr int WM = 64, WN = 64;   // wave tile (2 x 2 waves)
+  static constexpr int WK = 32;            // k per fragment
+  static constexpr int SKEW = 4;
+  static constexpr int LD = SK + SKEW;
+  static constexpr int STAGES = 2;
+  static constexpr int THREADS = 256;
+  static constexpr int STAGE_FLOATS = (BM + BN) * LD;
+  static constexpr int LDS_BYTES = STAGES * STAGE_FLOATS * 4;
+};
+
+// Copy ROWS x SK floats (row r at src + r*ld) into a tile with rows LD apart.
+template <int ROWS, int SK, int LD, int THREADS>
+__device__ __forceinline__ void stage_tile(float *const dst,
+                                           const float *const src,
+                                           const long long ld) {
+  constexpr int PIECES = ROWS * LD / 4; // 16-byte pieces of the padded image
+#pragma unroll
+  for (int p0 = 0; p0 < PIECES; p0 += THREADS) {
+    const int p = p0 + static_cast<int>(threadIdx.x);
+    if (p0 + THREADS <= PIECES || p < PIECES) {
+      const int r = p / (LD / 4);
+      int c = p - r * (LD / 4);
+      c = c < SK / 4 ? c : SK / 4 - 1; // padding: the last piece once more
+      cpa::cp_async<16>(dst + 4 * p, src + r * ld + 4 * c);
+    }
+  }
+}
+
+// C tile = alpha * A tile * B tile + beta * C tile for one 128 x 128 tile of
+// one batch entry.  A: m x k row-major (lda), B: k x n column-major (ldb), C:
+// m x n column-major (ldc); m, n multiples of 128, k of 32; batch entry y at
+// base + y*stride or, when the pointer arrays are set, at ptrs[y].
 template <class T, class Policy>
-__global__ void __launch_bounds__(256)
+__global__ void __launch_bounds__(ApiGemmShape::THREADS, 2)
     tcec_api_gemm_kernel(const int m, const int n, const int k,
-                         const float alpha, const float *__restrict__ A,
-                         const int lda, const float *__restrict__ B,
-                         const int ldb, const float beta,
-                         float *__restrict__ C, const int ldc) {
-  constexpr int BM = 128, BN = 128, BK = 32, LD = BK + 4; // +4 floats: skewed rows
-  constexpr int WM = 64, WN = 64;
-  __shared__ float sa[BM * LD];
-  __shared__ float sb[BN * LD];
+                         const float alpha, const float *const A,
+                         const float *const *const a_ptrs, const int lda,
+                         const long long stride_a, const float *const B,
+                         const float *const *const b_ptrs, const int ldb,
+                         const long long stride_b, const float beta,
+                         float *const C, float *const *const c_ptrs,
+                         const int ldc, const long long stride_c) {
+  using S = ApiGemmShape;
+  extern __shared__ __attribute__((aligned(16))) float smem[];
+
+  // tile of this workgroup: consecutive block ids run on different XCDs, so
+  // ids are regrouped to give each XCD (id % 8) one contiguous run of tiles,
+  // walked column by column through bands of eight tile rows
+  const unsigned tiles_m = m / S::BM, tiles_n = n / S::BN;
+  const unsigned tiles = tiles_m * tiles_n;
+  const unsigned entry = blockIdx.x / tiles;
+  unsigned t = blockIdx.x - entry * tiles;
+  if (tiles % 8 == 0)
+    t = (t % 8) * (tiles / 8) + t / 8;
+  const unsigned band = t / (8 * tiles_n);
+  const unsigned band_rows = tiles_m - 8 * band < 8 ? tiles_m - 8 * band : 8;
+  const unsigned in_band = t - band * 8 * tiles_n;
+  const unsigned tn = in_band / band_rows;
+  const unsigned tm = 8 * band + in_band - tn * band_rows;
+
+  const float *const a_base =
+      (a_ptrs != nullptr ? a_ptrs[entry] : A + entry * stride_a) +
+      static_cast<long long>(tm * S::BM) * lda;
+  const float *const b_base =
+      (b_ptrs != nullptr ? b_ptrs[entry] : B + entry * stride_b) +
+      static_cast<long long>(tn * S::BN) * ldb;
+
   const int wave = threadIdx.x / 64;
   const int wm = wave % 2, wn = wave / 2;
-  const int m0 = blockIdx.x * BM, n0 = blockIdx.y * BN;
 
-  tcec::fragment<w::matrix_a, WM, WN, BK, T, w::row_major, Policy> fa;
-  tcec::fragment<w::matrix_b, WM, WN, BK, T, w::col_major, Policy> fb;
-  tcec::fragment<w::accumulator, WM, WN, BK, T, void, Policy> fc;
+  using FragA =
+      tcec::fragment<w::matrix_a, S::WM, S::WN, S::WK, T, w::row_major, Policy>;
+  using FragB =
+      tcec::fragment<w::matrix_b, S::WM, S::WN, S::WK, T, w::col_major, Policy>;
+  using FragC =
+      tcec::fragment<w::accumulator, S::WM, S::WN, S::WK, T, void, Policy>;
+  FragC fc;
   tcec::fill_zero(fc);
 
-  for (int k0 = 0; k0 < k; k0 += BK) {
-    // 128 rows x 32 floats per operand = 1024 float4, 4 per thread
-    for (int f = threadIdx.x; f < BM * BK / 4; f += 256) {
-      const int r = f / (BK / 4), c4 = f % (BK / 4);
-      const float4 va = *reinterpret_cast<const float4 *>(
-          A + static_cast<long long>(m0 + r) * lda + k0 + 4 * c4);
-      const float4 vb = *reinterpret_cast<const float4 *>(
-          B + static_cast<long long>(n0 + r) * ldb + k0 + 4 * c4);
-      *reinterpret_cast<float4 *>(&sa[r * LD + 4 * c4]) = va;
-      *reinterpret_cast<float4 *>(&sb[r * LD + 4 * c4]) = vb;
+  auto stage_in = [&](const int stage, const int k0) {
+    float *const sa = smem + stage * S::STAGE_FLOATS;
+    float *const sb = sa + S::BM * S::LD;
+    stage_tile<S::BM, S::SK, S::LD, S::THREADS>(sa, a_base + k0, lda);
+    stage_tile<S::BN, S::SK, S::LD, S::THREADS>(sb, b_base + k0, ldb);
+    cpa::commit();
+  };
+
+  stage_in(0, 0);
+  cpa::wait_all();
+  __syncthreads();
+
+  int stage = 0;
+  for (int k0 = 0; k0 < k; k0 += S::SK) {
+    if (k0 + S::SK < k)
+      stage_in(1 - stage, k0 + S::SK);
+
+    const float *const sa = smem + stage * S::STAGE_FLOATS + wm * S::WM * S::LD;
+    const float *const sb =
+        smem + stage * S::STAGE_FLOATS + (S::BM + wn * S::WN) * S::LD;
+    // fragments double buffered over the k steps of the stage
+    FragA fa[2];
+    FragB fb[2];
+    tcec::load_matrix_sync(fa[0], sa, S::LD, false);
+    tcec::load_matrix_sync(fb[0], sb, S::LD, false);
+#pragma unroll
+    for (int kk = S::WK; kk < S::SK; kk += S::WK) {
+      const int cur = (kk / S::WK) & 1;
+      tcec::load_matrix_sync(fa[cur], sa + kk, S::LD, false);
+      tcec::load_matrix_sync(fb[cur], sb + kk, S::LD, false);
+      tcec::mma_sync(fc, fa[1 - cur], fb[1 - cur], fc);
     }
+    constexpr int last = ((S::SK / S::WK) - 1) & 1;
+    tcec::mma_sync(fc, fa[last], fb[last], fc);
+
+    cpa::wait_all();
     __syncthreads();
-    tcec::load_matrix_sync(fa, sa + wm * WM * LD, LD);  // memory layout = row_major
-    tcec::load_matrix_sync(fb, sb + wn * WN * LD, LD);  // memory layout = col_major
-    tcec::mma_sync(fc, fa, fb, fc);
-    __syncthreads();
+    stage = 1 - stage;
   }
 
-  float *const cw = C + (m0 + wm * WM) + static_cast<long long>(n0 + wn * WN) * ldc;
+  float *const cw = (c_ptrs != nullptr ? c_ptrs[entry] : C + entry * stride_c) +
+                    (tm * S::BM + wm * S::WM) +
+                    static_cast<long long>(tn * S::BN + wn * S::WN) * ldc;
   if (beta == 0.f) {
     tcec::store_matrix_sync_with_mul<w::col_major>(cw, fc, ldc, alpha);
   } else {
-    tcec::fragment<w::accumulator, WM, WN, BK, T, void, Policy> fin;
+    FragC fin;
     tcec::load_matrix_sync(fin, cw, ldc, w::mem_col_major);
     fc.integrate();
+#pragma unroll
     for (unsigned i = 0; i < fc.num_elements; i++)
       fc.x(i) = alpha * fc.x(i) + beta * fin.x(i);
     tcec::store_matrix_sync(cw, fc, ldc, w::mem_col_major);
   }
 }
-
 
 } // namespace wmmae_harness

@@ -316,6 +316,18 @@ def api_gemm(type_, ec, m, n, k, alpha, A, lda, B, ldb, beta, C, ldc):
     _lib.check(st, "wmmae_tcec_api_gemm")
 
 
+def api_gemm_batched(type_, ec, m, n, k, alpha, A_array, lda, B_array, ldb, beta, C_array, ldc, batch):
+    """api_gemm on int64 device tensors of `batch` matrix pointers (launch_bgemm's convention)."""
+    _need_cuda(A_array, B_array, C_array)
+    for name, arr in (("A_array", A_array), ("B_array", B_array), ("C_array", C_array)):
+        if arr.dtype != torch.int64 or arr.numel() < batch:
+            raise ValueError(f"{name}: int64 tensor of at least {batch} device pointers required")
+    st = _lib.lib().wmmae_tcec_api_gemm_batched(type_, int(ec), m, n, k, _f(alpha), _ptr(A_array), lda,
+                                                _ptr(B_array), ldb, _f(beta), _ptr(C_array), ldc, batch,
+                                                _stream())
+    _lib.check(st, "wmmae_tcec_api_gemm_batched")
+
+
 def mfma_probe(type_, m, n, k, a_bits, b_bits, c):
     """a_bits (m,k) / b_bits (k,n): int16 tensors of raw 16-bit patterns; c (m,n) fp32."""
     _need_cuda(a_bits, b_bits, c)
