@@ -74,13 +74,20 @@ template <> struct split_traits<float> {
   }
 };
 
-// split4: split() applied to four values at once.  The arithmetic per element
-// is that of split_traits<T>::split; it is written on two-element vectors so
-// that the packed conversions (v_cvt_pk_f16_f32 / v_cvt_pk_bf16_f32) are used.
+// split4: split() applied to four values at once (device code).  The
+// arithmetic per element is that of split_traits<T>::split, arranged for the
+// packed conversions of gfx950:
+//   half : hi pair = v_cvt_pk_f16_f32; (v - hi) * 2048 is evaluated as
+//          fma(hi, -2048, v * 2048) - v - hi and both scalings by a power of
+//          two are exact, so this is the same number - by the mixed-precision
+//          fma that reads hi as fp16 and writes its fp32 result rounded to one
+//          half of a register (v_fma_mixlo_f16 / v_fma_mixhi_f16): five
+//          instructions per two elements
+//   bf16 : v_cvt_pk_bf16_f32 pairs, residuals by fp32 subtraction
 typedef float f32x2_t __attribute__((ext_vector_type(2)));
 typedef float f32x4_t __attribute__((ext_vector_type(4)));
 template <class T, class S = typename split_traits<T>::storage>
-WMMAE_HD void split4(const f32x4_t v, S *const t0, S *const t1, S *const t2) {
+WMMAE_D void split4(const f32x4_t v, S *const t0, S *const t1, S *const t2) {
   using traits = split_traits<T>;
   if constexpr (std::is_same<S, float>::value) {
 #pragma unroll
@@ -95,10 +102,24 @@ WMMAE_HD void split4(const f32x4_t v, S *const t0, S *const t1, S *const t2) {
       t0[e] = h0[0];
       t0[e + 1] = h0[1];
       if constexpr (traits::num_terms >= 2) {
-        f32x2_t r = vv - __builtin_convertvector(h0, f32x2_t);
-        if constexpr (traits::scale != 1.f)
-          r *= traits::scale;
-        const s2_t h1 = __builtin_convertvector(r, s2_t);
+        f32x2_t r = {0.f, 0.f};
+        s2_t h1;
+        if constexpr (std::is_same<S, _Float16>::value) {
+          static_assert(traits::num_terms == 2, "two-term fp16 split");
+          const float m0 = vv[0] * traits::scale, m1 = vv[1] * traits::scale;
+          const float neg_scale = -traits::scale;
+          asm("v_fma_mixlo_f16 %0, %1, %2, %3 op_sel:[0,0,0] op_sel_hi:[1,0,0]"
+              : "=v"(h1)
+              : "v"(h0), "s"(neg_scale), "v"(m0));
+          asm("v_fma_mixhi_f16 %0, %1, %2, %3 op_sel:[1,0,0] op_sel_hi:[1,0,0]"
+              : "+v"(h1)
+              : "v"(h0), "s"(neg_scale), "v"(m1));
+        } else {
+          r = vv - __builtin_convertvector(h0, f32x2_t);
+          if constexpr (traits::scale != 1.f)
+            r *= traits::scale;
+          h1 = __builtin_convertvector(r, s2_t);
+        }
         t1[e] = h1[0];
         t1[e + 1] = h1[1];
         if constexpr (traits::num_terms >= 3) {

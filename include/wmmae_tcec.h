@@ -349,7 +349,9 @@ int wmmae_clock_samples(unsigned long long *out, int nsamples,
  * elements from src to dst through LDS.  mode 0: lane-linear destinations
  * (the reference's test), 1: scattered destinations, 2: every third thread
  * inactive (its element comes back as zero), 3: two copies in flight released
- * one after the other.  src must be `size`-aligned.
+ * one after the other, 4 and 5: modes 0 and 2 through
+ * utils::cp_async::cp_async_lane_linear (size 4 or 16; size 8 returns
+ * WMMAE_STATUS_NOT_SUPPORTED).  src must be `size`-aligned.
  * Replaces: cp_async_test_kernel, test/utils/cp_async.cu:15-25. */
 int wmmae_utils_cp_async(int size, int mode, void *dst, const void *src,
                          void *stream);

@@ -332,6 +332,38 @@ def test_api_level_gemm_matches_driver(tc, orc, dev, type_ec):
     assert e.value.status == -4
 
 
+def test_api_level_gemm_pointer_arrays(tc, orc, dev):
+    """The API-level kernel on device arrays of matrix pointers (launch_bgemm's calling
+    convention, batch_gemm.cu:433-443): every entry equals the single-matrix call bit for bit,
+    and the reference harness's ramp inputs A[j] = j/k, B[j] = j/n (batch_gemm.cu:507-513) keep
+    its residual gate."""
+    batch, m, n, k = 5, 256, 128, 96
+    rng = np.random.default_rng(4242)
+    A = rng.uniform(-1, 1, (batch, m, k)).astype(np.float32)
+    Bt = rng.uniform(-1, 1, (batch, n, k)).astype(np.float32)
+    A[0] = (np.arange(m * k, dtype=np.float32) / k).reshape(m, k)
+    Bt[0] = (np.arange(n * k, dtype=np.float32) / n).reshape(n, k)
+    dA = [torch.from_numpy(A[b]).to(dev) for b in range(batch)]
+    dB = [torch.from_numpy(Bt[b]).to(dev) for b in range(batch)]
+    dC = [torch.zeros((n, m), dtype=torch.float32, device=dev) for _ in range(batch)]
+    pa = torch.tensor([t.data_ptr() for t in dA], dtype=torch.int64, device=dev)
+    pb = torch.tensor([t.data_ptr() for t in dB], dtype=torch.int64, device=dev)
+    pc = torch.tensor([t.data_ptr() for t in dC], dtype=torch.int64, device=dev)
+    for type_, ec in ((0, 1), (2, 1), (0, 0)):
+        tc.api_gemm_batched(type_, ec, m, n, k, 1.0, pa, k, pb, k, 0.0, pc, m, batch)
+        torch.cuda.synchronize()
+        for b in range(batch):
+            single = torch.zeros((n, m), dtype=torch.float32, device=dev)
+            tc.api_gemm(type_, ec, m, n, k, 1.0, dA[b], k, dB[b], k, 0.0, single, m)
+            torch.cuda.synchronize()
+            assert torch.equal(single, dC[b]), (type_, ec, b)
+        if ec:
+            got = dC[0].cpu().numpy().T.astype(np.float64)
+            ref = orc.gemm_f64(A[0], Bt[0].T)
+            assert np.linalg.norm(got - ref) / np.linalg.norm(ref) < 1e-6
+    tc.api_gemm_batched(0, 1, m, n, k, 1.0, pa, k, pb, k, 0.0, pc, m, 0)     # empty batch: nothing to do
+
+
 def test_api_level_gemm_fp32_policy(tc, orc, dev):
     """The same API-level GEMM with default_policy<float, without_ec, op_simt>: a plain
     fp32 product on the matrix core's fp32 path, the on-GPU comparator of the 2x gate."""

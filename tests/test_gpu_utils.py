@@ -8,15 +8,22 @@ pytestmark = pytest.mark.gpu
 
 
 @pytest.mark.parametrize("size", [4, 8, 16])
-@pytest.mark.parametrize("mode", [0, 1, 2, 3])
+@pytest.mark.parametrize("mode", [0, 1, 2, 3, 4, 5])
 def test_cp_async_copies_every_byte(tc, dev, size, mode):
     """The reference's check: input word i holds float(i); the copy through LDS returns
-    it unchanged (error = 0), for lane-linear, scattered, partially masked and pipelined use."""
+    it unchanged (error = 0), for lane-linear, scattered, partially masked and pipelined use,
+    and for cp_async_lane_linear (modes 4, 5: full and partially masked waves)."""
     words = 256 * size // 4
     src = torch.arange(words, dtype=torch.float32, device=dev)
+    if mode >= 4 and size == 8:
+        from wmma_extension_amd._lib import WmmaeError
+        with pytest.raises(WmmaeError) as e:
+            tc.utils_cp_async(size, mode, src)
+        assert e.value.status == -4
+        return
     got = tc.utils_cp_async(size, mode, src).cpu().numpy()
     expect = np.arange(words, dtype=np.float32)
-    if mode == 2:
+    if mode in (2, 5):
         elem = (np.arange(words) // (size // 4)) % 128
         expect = np.where(elem % 3 != 0, expect, 0.0).astype(np.float32)
     assert np.array_equal(got, expect)

@@ -47,7 +47,7 @@ int api_gemm_impl(const int type, const int ec, const int m, const int n,
     return with_ec(ec, [&](auto te) -> int {
       using EC = typename decltype(te)::type;
       using P = typename harness_policy<T, EC, 16, 16, 32>::type;
-      auto kernel = wmmae_harness::tcec_api_gemm_kernel<T, P>;
+      auto kernel = wmmae_harness::tcec_api_gemm_kernel<T, P, 2>;
       static std::atomic<unsigned long long> lds_allowed{0};
       WMMAE_HIP_TRY(allow_dynamic_lds(reinterpret_cast<const void *>(kernel),
                                       S::LDS_BYTES, lds_allowed));

@@ -448,8 +448,10 @@ int wmmae_utils_cp_async(const int size, const int mode, void *const dst,
                          const void *const src, void *const stream) {
   if (!dst || !src)
     return WMMAE_STATUS_NULL_POINTER;
-  if (mode < 0 || mode > 3 || (size != 4 && size != 8 && size != 16))
+  if (mode < 0 || mode > 5 || (size != 4 && size != 8 && size != 16))
     return WMMAE_STATUS_INVALID_VALUE;
+  if (mode >= 4 && size == 8) // the direct load moves 4 or 16 bytes per lane
+    return WMMAE_STATUS_NOT_SUPPORTED;
   if (reinterpret_cast<uintptr_t>(src) % size != 0 ||
       reinterpret_cast<uintptr_t>(dst) % 4 != 0)
     return WMMAE_STATUS_MISALIGNED;

@@ -694,6 +694,8 @@ __global__ void __launch_bounds__(64)
 //   mode 2: only threads with t % 3 != 0 copy; the others' slots are zeroed
 //           first (direct load under a partial execution mask)
 //   mode 3: two groups in flight, wait_pending<1> releases the first
+//   mode 4: mode 0 through cp_async_lane_linear (Size 4 or 16)
+//   mode 5: mode 2 through cp_async_lane_linear (Size 4 or 16)
 // --------------------------------------------------------------------------
 template <unsigned Size>
 __global__ void __launch_bounds__(128)
@@ -734,6 +736,22 @@ __global__ void __launch_bounds__(128)
     cpa::wait_all();
     out(t, &smem[0][t * W]);
     out(128 + t, &smem[1][t * W]);
+  } else if (mode == 4 || mode == 5) {
+    if constexpr (Size != 8) {
+      if (mode == 5) {
+        for (unsigned i = 0; i < W; i++)
+          smem[0][t * W + i] = smem[1][t * W + i] = 0u;
+        __syncthreads();
+      }
+      if (mode == 4 || t % 3 != 0) {
+        cpa::cp_async_lane_linear<Size>(&smem[0][t * W], src + t * W);
+        cpa::cp_async_lane_linear<Size>(&smem[1][t * W], src + (128 + t) * W);
+      }
+      cpa::commit();
+      cpa::wait_all();
+      out(t, &smem[0][t * W]);
+      out(128 + t, &smem[1][t * W]);
+    }
   } else {
     cpa::cp_async<Size>(&smem[0][t * W], src + t * W);
     cpa::commit();

@@ -15,12 +15,22 @@
 // Rows of a staged tile are SK + 4 floats apart: sixteen lanes reading 16
 // bytes of sixteen consecutive rows then cover all 64 LDS banks once.  The
 // direct global->LDS copy of gfx950 writes lane-linear destinations only, so
-// the copy walks the padded tile image linearly, 16 bytes per lane, and lets
-// the lanes that land on a row's padding fetch that row's last piece again.
+// the copy walks the padded tile image linearly, 16 bytes per lane
+// (cp_async_lane_linear), and lets the lanes that land on a row's padding
+// fetch that row's last piece again.
 //
 // Two workgroups of four waves share a compute unit (72 KiB of LDS and at
-// most 256 registers each), so that one wave's conversion arithmetic runs
-// beside another's MFMAs.
+// most 256 registers each, WAVES_PER_SIMD = 2): while one waits at its
+// barrier or for its copies, the other computes.  (One workgroup per compute
+// unit with up to 512 registers measured slower for every policy, the
+// three-term split included: 144 against 183 TFLOPS at 4096^3.)
+//
+// Three things the compiler has to be told for the stage loop to become one
+// basic block whose MFMAs and conversions it can interleave: the wave index is
+// wave-uniform (readfirstlane), the tile pointers handed to load_matrix_sync
+// are 16-byte aligned (__builtin_assume_aligned: its 16-byte path is then
+// chosen at compile time), and the wait for the copies stays where it is
+// written (cp_async::wait_all is a scheduling barrier).
 #pragma once
 #include <wmma_extension/tcec/tcec.hpp>
 #include <wmma_extension/utils.hpp>
@@ -44,20 +54,26 @@ struct ApiGemmShape {
 };
 
 // Copy ROWS x SK floats (row r at src + r*ld) into a tile with rows LD apart.
+// A pass moves as many whole padded rows as the workgroup has lanes for (28
+// rows of nine 16-byte pieces with 256 threads; the last four threads idle),
+// so that a thread keeps its place inside a row and its source address moves
+// by the same amount from pass to pass.
 template <int ROWS, int SK, int LD, int THREADS>
 __device__ __forceinline__ void stage_tile(float *const dst,
                                            const float *const src,
                                            const long long ld) {
-  constexpr int PIECES = ROWS * LD / 4; // 16-byte pieces of the padded image
+  constexpr int PR = LD / 4;             // 16-byte pieces per padded row
+  constexpr int RP = THREADS / PR;       // rows per pass
+  const int tid = static_cast<int>(threadIdx.x);
+  const int r_in = tid / PR;
+  int c = tid - r_in * PR;
+  c = c < SK / 4 ? c : SK / 4 - 1;       // padding: the last piece once more
+  const float *const from = src + r_in * ld + 4 * c;
+  if (tid < RP * PR) {
 #pragma unroll
-  for (int p0 = 0; p0 < PIECES; p0 += THREADS) {
-    const int p = p0 + static_cast<int>(threadIdx.x);
-    if (p0 + THREADS <= PIECES || p < PIECES) {
-      const int r = p / (LD / 4);
-      int c = p - r * (LD / 4);
-      c = c < SK / 4 ? c : SK / 4 - 1; // padding: the last piece once more
-      cpa::cp_async<16>(dst + 4 * p, src + r * ld + 4 * c);
-    }
+    for (int r0 = 0; r0 < ROWS; r0 += RP)
+      if (r0 + RP <= ROWS || r0 + r_in < ROWS)
+        cpa::cp_async_lane_linear<16>(dst + 4 * (r0 * PR + tid), from + r0 * ld);
   }
 }
 
@@ -65,8 +81,8 @@ __device__ __forceinline__ void stage_tile(float *const dst,
 // one batch entry.  A: m x k row-major (lda), B: k x n column-major (ldb), C:
 // m x n column-major (ldc); m, n multiples of 128, k of 32; batch entry y at
 // base + y*stride or, when the pointer arrays are set, at ptrs[y].
-template <class T, class Policy>
-__global__ void __launch_bounds__(ApiGemmShape::THREADS, 2)
+template <class T, class Policy, int WAVES_PER_SIMD>
+__global__ void __launch_bounds__(ApiGemmShape::THREADS, WAVES_PER_SIMD)
     tcec_api_gemm_kernel(const int m, const int n, const int k,
                          const float alpha, const float *const A,
                          const float *const *const a_ptrs, const int lda,
@@ -100,7 +116,7 @@ __global__ void __launch_bounds__(ApiGemmShape::THREADS, 2)
       (b_ptrs != nullptr ? b_ptrs[entry] : B + entry * stride_b) +
       static_cast<long long>(tn * S::BN) * ldb;
 
-  const int wave = threadIdx.x / 64;
+  const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x / 64);
   const int wm = wave % 2, wn = wave / 2;
 
   using FragA =
@@ -129,9 +145,12 @@ __global__ void __launch_bounds__(ApiGemmShape::THREADS, 2)
     if (k0 + S::SK < k)
       stage_in(1 - stage, k0 + S::SK);
 
-    const float *const sa = smem + stage * S::STAGE_FLOATS + wm * S::WM * S::LD;
+    const float *const sa =
+        static_cast<const float *>(__builtin_assume_aligned(
+            smem + stage * S::STAGE_FLOATS + wm * S::WM * S::LD, 16));
     const float *const sb =
-        smem + stage * S::STAGE_FLOATS + (S::BM + wn * S::WN) * S::LD;
+        static_cast<const float *>(__builtin_assume_aligned(
+            smem + stage * S::STAGE_FLOATS + (S::BM + wn * S::WN) * S::LD, 16));
     // fragments double buffered over the k steps of the stage
     FragA fa[2];
     FragB fb[2];
