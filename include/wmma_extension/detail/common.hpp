@@ -59,20 +59,22 @@ template <> struct storage_t<__half> {
 };
 #endif
 
-// Round-to-nearest-even fp32 -> tf32 (10 explicit mantissa bits) done with
-// integer arithmetic.  The reference uses cvt.rna (ties away); ties-to-even is
-// used here so the result matches the IEEE conversions of the other types.
+// fp32 -> tf32 (10 explicit mantissa bits in an fp32 container), round to
+// nearest with ties away from zero: the reference converts with PTX
+// cvt.rna.tf32.f32 (detail/common.hpp:36-48).  On the sign-magnitude bit
+// pattern that is "add half a unit of the kept precision, drop the low 13
+// bits".  inf / nan pass through.
 WMMAE_HD float to_tf32(const float a) {
   uint32_t u = __builtin_bit_cast(uint32_t, a);
   if ((u & 0x7f800000u) == 0x7f800000u)
-    return a; // inf / nan pass through
-  u += 0x00000fffu + ((u >> 13) & 1u);
-  u &= 0xffffe000u;
+    return a;
+  u = (u + 0x00001000u) & 0xffffe000u;
   return __builtin_bit_cast(float, u);
 }
 
-// cast<T>(v): convert v to the storage type of tag T, round to nearest even
-// (reference: detail/common.hpp:25-61).
+// cast<T>(v): convert v to the storage type of tag T: round to nearest even
+// for half and bfloat16, ties away from zero for precision::tf32, as in the
+// reference (detail/common.hpp:25-61).
 template <class T, class S>
 WMMAE_HD typename storage_t<T>::type cast(const S v) {
   if constexpr (std::is_same<T, precision::tf32>::value) {

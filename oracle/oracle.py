@@ -66,6 +66,16 @@ def lib():
         h.orc_tcec_matmul.restype = None
         h.orc_tcec_matmul.argtypes = [_i, _i, _i, _i, _fp, _ll, _ll, _fp, _ll, _ll,
                                       _c.c_void_p, _fp, _ll, _ll, _i, _i, _i]
+        h.orc_tcec_matmul_model.restype = None
+        h.orc_tcec_matmul_model.argtypes = [_i, _i, _i, _i, _fp, _ll, _ll, _fp, _ll, _ll,
+                                            _c.c_void_p, _fp, _ll, _ll, _i, _i, _i, _i]
+        h.orc_mfma_dot.restype = _c.c_float
+        h.orc_mfma_dot.argtypes = [_fp, _fp, _i, _i, _c.c_float]
+        h.orc_mfma_tile.restype = None
+        h.orc_mfma_tile.argtypes = [_i, _i, _i, _i, np.ctypeslib.ndpointer(np.uint16, flags="C"),
+                                    np.ctypeslib.ndpointer(np.uint16, flags="C"), _c.c_void_p, _fp]
+        h.orc_to_tf32.restype = _c.c_float
+        h.orc_to_tf32.argtypes = [_c.c_float]
         h.orc_gemm_f64.restype = None
         h.orc_gemm_f64.argtypes = [_i, _i, _i, _fp, _ll, _ll, _fp, _ll, _ll, _dp, _ll, _ll]
         h.orc_gemm_f32.restype = None
@@ -228,8 +238,41 @@ def gemm_f32_tn(A, Bt):
     return D
 
 
-def tcec_matmul(A, B, C=None, kind=SPLIT_F16, ec=True, fk=32, main_outside=True):
-    """TCEC emulation of D = A*B (+C) with k blocks of fk."""
+def to_tf32(v):
+    """fp32 -> tf32 with ties away from zero (the reference's cvt.rna)."""
+    return np.float32(lib().orc_to_tf32(float(np.float32(v))))
+
+
+def mfma_dot(a, b, c=0.0, bf16=False):
+    """One output element of a raw MFMA in the gfx950 accumulate model: a, b hold values that are
+    exactly representable in the 16-bit type."""
+    a = np.ascontiguousarray(a, dtype=np.float32)
+    b = np.ascontiguousarray(b, dtype=np.float32)
+    assert a.shape == b.shape and a.ndim == 1
+    return np.float32(lib().orc_mfma_dot(a, b, a.size, int(bf16), float(np.float32(c))))
+
+
+def mfma_tile(type_, a_bits, b_bits, c=None):
+    """D = A*B + C of one raw MFMA in the gfx950 accumulate model; a_bits (M,K) and b_bits (K,N) are
+    uint16 bit patterns (type_ 0 half, 1 bfloat16), c (M,N) fp32 or None."""
+    a_bits = np.ascontiguousarray(a_bits).view(np.uint16)
+    b_bits = np.ascontiguousarray(b_bits).view(np.uint16)
+    M, K = a_bits.shape
+    K2, N = b_bits.shape
+    assert K == K2 and K <= 64
+    d = np.zeros((M, N), dtype=np.float32)
+    cptr = None
+    if c is not None:
+        c = np.ascontiguousarray(c, dtype=np.float32)
+        cptr = c.ctypes.data_as(_c.c_void_p)
+    lib().orc_mfma_tile(type_, M, N, K, a_bits, b_bits, cptr, d.reshape(-1))
+    return d
+
+
+def tcec_matmul(A, B, C=None, kind=SPLIT_F16, ec=True, fk=32, main_outside=True, hw_model=False):
+    """TCEC emulation of D = A*B (+C) with k blocks of fk.  hw_model: every matrix instruction in
+    the measured accumulate arithmetic of the gfx950 matrix core instead of an exact sum rounded
+    once."""
     A = np.asarray(A, dtype=np.float32)
     B = np.asarray(B, dtype=np.float32)
     m, k = A.shape
@@ -242,8 +285,8 @@ def tcec_matmul(A, B, C=None, kind=SPLIT_F16, ec=True, fk=32, main_outside=True)
     if C is not None:
         C = np.ascontiguousarray(C, dtype=np.float32)
         cptr = C.ctypes.data_as(_c.c_void_p)
-    lib().orc_tcec_matmul(m, n, k, fk, a, ar, ac, b, br, bc, cptr, D.reshape(-1), n, 1,
-                          kind, int(ec), int(main_outside))
+    lib().orc_tcec_matmul_model(m, n, k, fk, a, ar, ac, b, br, bc, cptr, D.reshape(-1), n, 1,
+                                kind, int(ec), int(main_outside), int(hw_model))
     return D
 
 

@@ -68,8 +68,11 @@ def test_sgemm_aligned_shapes(tc, orc, dev, policy, mnk):
     D = _gemm(tc, dev, A, B, policy)
     _check(orc, D, A, B, policy)
     kind, ec = POL_KIND[policy]
-    emu = orc.tcec_matmul(A, B, kind=kind, ec=ec, fk=32, main_outside=False)
-    assert np.abs(D - emu).max() <= 32 * 2.0**-24 * np.abs(emu).max()
+    # the driver's instruction sequence per output element (32 of k per step, error products
+    # before the leading one, everything chained through the matrix core) in the oracle's
+    # model of that core: same bits
+    emu = orc.tcec_matmul(A, B, kind=kind, ec=ec, fk=32, main_outside=False, hw_model=True)
+    assert np.array_equal(D.view(np.uint32), emu.view(np.uint32)), np.abs(D - emu).max()
 
 
 @pytest.mark.parametrize("policy", [0, 2])
@@ -324,6 +327,17 @@ def test_api_level_gemm_matches_driver(tc, orc, dev, type_ec):
         got = dC.cpu().numpy().T
         ref = alpha * orc.gemm_f64(A, Bt.T) + beta * C0
         _check(orc, got, A, Bt.T, policy, ref=ref, C=C0, alpha=alpha, beta=beta)
+        # the kernel is tcec::mma_sync over k steps of 32 on a zero accumulator (round-to-nearest
+        # adds of the leading product with error correction), then alpha / beta in fp32
+        emu = orc.tcec_matmul(A, Bt.T, kind=POL_KIND[policy][0], ec=bool(ec), fk=32,
+                              main_outside=bool(ec), hw_model=True)
+        if (alpha, beta) == (1.0, 0.0):
+            assert np.array_equal(got.view(np.uint32), emu.view(np.uint32)), np.abs(got - emu).max()
+        else:
+            expect = alpha * emu.astype(np.float64) + beta * C0
+            assert (np.abs(got - expect) <= 2 * 2.0**-24 * (np.abs(alpha * emu) + np.abs(beta * C0))).all()
+        # the driver chains the leading product through the matrix core instead: two roundings
+        # of the same sums
         drv = _gemm(tc, dev, A, Bt.T, policy, alpha=alpha, beta=beta, C=C0)
         assert np.abs(got - drv).max() <= 16 * 2.0**-24 * max(1.0, np.abs(ref).max())
     from wmma_extension_amd._lib import WmmaeError
@@ -441,8 +455,13 @@ def test_sgemm_randomised_sweep(tc, orc, dev):
         C = rng.uniform(-1, 1, (m, n)).astype(np.float32)
         D = _gemm(tc, dev, A, B, policy, alpha=alpha, beta=beta, C=C, ta=ta, tb=tb, ld_pad=ld_pad)
         kind, ec = POL_KIND[policy]
-        emu = orc.tcec_matmul(A, B, kind=kind, ec=ec, fk=32, main_outside=False)
+        emu = orc.tcec_matmul(A, B, kind=kind, ec=ec, fk=32, main_outside=False, hw_model=True)
         expect = alpha * emu.astype(np.float64) + beta * C
-        tol = 32 * 2.0**-24 * max(1.0, np.abs(expect).max())
-        assert np.abs(D - expect).max() <= tol, (case, m, n, k, policy, ta, tb, alpha, beta, ld_pad)
+        if tc.sgemm_path(m, n, k, 1, policy) == tc.PATH_PACKED_SPLIT_K:
+            # K slices round their partial sums
+            tol = 32 * 2.0**-24 * max(1.0, np.abs(expect).max())
+        else:
+            # same sums as the emulator; alpha and beta are applied in fp32
+            tol = 2 * 2.0**-24 * (np.abs(alpha * emu) + np.abs(beta * C)) + 2.0**-140
+        assert (np.abs(D - expect) <= tol).all(), (case, m, n, k, policy, ta, tb, alpha, beta, ld_pad)
         _check(orc, D, A, B, policy, C=C, alpha=alpha, beta=beta)

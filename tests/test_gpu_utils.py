@@ -53,11 +53,18 @@ def test_cast_matches_oracle_conversions(tc, orc, dev):
     assert np.array_equal(h, orc.split(orc.SPLIT_F16, v)[0])
     b = tc.utils_cast(1, x).cpu().numpy().view(np.uint16)
     assert np.array_equal(b, orc.split(orc.SPLIT_BF16X2, v)[0])
-    # tf32: round to nearest even at 10 mantissa bits, kept in an fp32 container
+    # tf32: 10 mantissa bits in an fp32 container, ties away from zero (cvt.rna in the reference)
     t = tc.utils_cast(2, x).cpu().numpy()
-    u = v.view(np.uint32).astype(np.uint64)
-    r = ((u + 0xFFF + ((u >> 13) & 1)) & ~np.uint64(0x1FFF)).astype(np.uint32).view(np.float32)
-    ok = np.isfinite(r)
-    assert np.array_equal(t[ok], r[ok]) and (t.view(np.uint32) & 0x1FFF == 0).all()
+    want = np.array([orc.to_tf32(e) for e in v[:4096]] + [orc.to_tf32(e) for e in special], dtype=np.float32)
+    got = np.concatenate([t[:4096], t[-special.size:]])
+    assert np.array_equal(got.view(np.uint32), want.view(np.uint32))
+    assert (t.view(np.uint32) & 0x1FFF == 0).all()
+    # in float64 over the whole sample: scale to the kept precision, floor(|x| + 1/2), scale back
+    x64 = v.astype(np.float64)
+    e = np.maximum(np.floor(np.log2(np.maximum(np.abs(x64), 2.0**-140))), -126.0)
+    ulp = np.exp2(e - 10)
+    r64 = np.sign(x64) * np.floor(np.abs(x64) / ulp + 0.5) * ulp
+    ok = np.abs(r64) < 3.4028235e38
+    assert np.array_equal(t[ok].astype(np.float64), r64[ok])
     f = tc.utils_cast(3, x).cpu().numpy()
     assert np.array_equal(f.view(np.uint32), v.view(np.uint32))

@@ -125,3 +125,43 @@ def test_split_special_values(orc):
     assert hif[7] == 65504.0 and lof[7] == 0
     # a value below half the smallest fp16 subnormal: hi = 0, lo carries it scaled
     assert hif[8] == 0.0 and abs(lof[8] / 2048 - 2.0e-8) < 2.0e-8 * 2.0**-10
+
+
+def test_to_tf32_ties_away_literals():
+    """cvt.rna.tf32.f32 of the reference (detail/common.hpp:36-48): nearest, ties away from
+    zero, low 13 bits cleared.  Bit patterns written out."""
+    from oracle import oracle as orc
+
+    def bits(u):
+        return np.array([u], dtype=np.uint32).view(np.float32)[0]
+    cases = [
+        (0x3F800000, 0x3F800000),   # 1.0
+        (0x3F800FFF, 0x3F800000),   # just below half a unit: down
+        (0x3F801000, 0x3F802000),   # exactly half, even mantissa below: away (nearest-even would stay)
+        (0x3F801001, 0x3F802000),
+        (0x3F803000, 0x3F804000),   # exactly half, odd mantissa below: up under both rules
+        (0xBF801000, 0xBF802000),   # negative tie: away from zero
+        (0xBF800FFF, 0xBF800000),
+        (0x00001000, 0x00002000),   # subnormal tie
+        (0x00000FFF, 0x00000000),
+        (0x7F7FF000, 0x7F800000),   # rounds up to infinity
+        (0x7F800000, 0x7F800000),   # inf stays
+        (0x80000000, 0x80000000),   # -0 stays
+    ]
+    for src, want in cases:
+        got = np.float32(orc.to_tf32(bits(src))).view(np.uint32)
+        assert got == want, (hex(src), hex(got), hex(want))
+
+
+def test_to_tf32_against_float64_arithmetic():
+    from oracle import oracle as orc
+    rng = np.random.default_rng(11)
+    v = rng.integers(0, 2**32, size=20000, dtype=np.uint64).astype(np.uint32).view(np.float32)
+    v = v[np.isfinite(v)]
+    x = v.astype(np.float64)
+    e = np.maximum(np.floor(np.log2(np.maximum(np.abs(x), 2.0**-140))), -126.0)
+    ulp = np.exp2(e - 10)
+    want = np.sign(x) * np.floor(np.abs(x) / ulp + 0.5) * ulp
+    got = np.array([orc.to_tf32(t) for t in v], dtype=np.float32).astype(np.float64)
+    ok = np.abs(want) < 3.4028235e38
+    assert np.array_equal(got[ok], want[ok])
