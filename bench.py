@@ -43,16 +43,51 @@ PEAK_MFMA_TFLOPS = 2500.0      # dense fp16 / bf16 MFMA, MI355X
 PEAK_HBM_GBS = 8000.0
 # workloads whose dominant kernel is bound by HBM rather than by the matrix cores
 HBM_BOUND = {"c2", "c5a", "c5a_packed"}
-# Bytes per launch of the dominant kernel that crossed the fabric side of L2, from
-# rocprofv3 --pmc FETCH_SIZE and --pmc WRITE_SIZE runs of this script (--calibrate),
-# scaled by the same counters of a 1 GiB copy (x2.000 and x1.000); see profiles/.
-MEASURED_TRAFFIC_BYTES = {
-    "c4": (75_497_800 + 1_048_580) * 1024,
-    "c3": (524_670 + 65_536) * 1024,
-    "c5a": (524_500 + 262_283) * 1024,
-    "c2": (1_048_622 + 3_276_830) * 1024,
-    "c5b": (2_100_460 + 32_768) * 1024,
+# Bytes per launch of the dominant kernel that crossed the fabric side of L2 come from two
+# rocprofv3 --pmc runs of this script (FETCH_SIZE, then WRITE_SIZE, with --calibrate), whose
+# summary under profiles/ ends in a line
+#     traffic: fetch_kib=<n> write_kib=<n> sources=<sha>
+# `sources` is the hash (below) of the kernel sources the figures were measured on: when the
+# sources have changed since, the figure is stale and `traffic` is reported as null.
+TRAFFIC_PROFILES = {
+    "c4": "tcec_gemm_kernel_c4_16384_bf16x3.md",
+    "c3": "tcec_gemm_kernel_c3_4096_f16.md",
+    "c5a": "tcec_gemm_fused_kernel_c5a_1024x256_f16.md",
+    "c5b": "tcec_gemm_kernel_c5b_1024x1024x262144_f16.md",
+    "c2": "primitive_tiles_kernel_c2_1M_tiles.md",
 }
+KERNEL_SOURCES = {
+    "c4": ["tcec_gemm_kernels.hpp"], "c3": ["tcec_gemm_kernels.hpp"], "c5b": ["tcec_gemm_kernels.hpp"],
+    "c5a": ["tcec_gemm_kernels.hpp", "tcec_gemm_fused_kernel.hpp"], "c2": ["harness_kernels.hpp"],
+}
+
+
+def kernel_sources_hash(workload):
+    import hashlib
+    h = hashlib.sha256()
+    for name in KERNEL_SOURCES.get(workload, []):
+        with open(os.path.join(ROOT, "wmma_extension_amd", "csrc", name), "rb") as f:
+            h.update(f.read())
+    return h.hexdigest()[:12]
+
+
+def measured_traffic(workload):
+    """(bytes or None, where it came from) for the workload's dominant kernel."""
+    import re
+    name = TRAFFIC_PROFILES.get(workload)
+    if name is None:
+        return None, None
+    path = os.path.join(ROOT, "profiles", name)
+    try:
+        text = open(path).read()
+    except OSError:
+        return None, None
+    m = re.search(r"traffic:\s*fetch_kib=(\d+)\s+write_kib=(\d+)\s+sources=([0-9a-f]+)", text)
+    if m is None:
+        return None, f"profiles/{name}: no traffic line"
+    if m.group(3) != kernel_sources_hash(workload):
+        return None, f"profiles/{name} was measured on other kernel sources ({m.group(3)}): stale, not reported"
+    return (int(m.group(1)) + int(m.group(2))) * 1024, f"profiles/{name} (sources {m.group(3)})"
 
 
 def make_inputs(torch, w, dev, seed):
@@ -74,21 +109,6 @@ def make_inputs(torch, w, dev, seed):
         s = torch.randint(0, 2, shape, generator=g, device=dev).to(torch.float32) * 2 - 1
         return s * x * torch.exp2(e)
     return draw(shape_a), draw(shape_b)
-
-
-def accuracy_sample(torch, orc, A, Bt, Ct, rows):
-    """max|C - C64| / max|C64| on `rows` full rows of batch 0, for TCEC and for
-    the plain fp32 loop on the same inputs."""
-    import numpy as np
-    m = A.shape[1]
-    g = torch.Generator().manual_seed(1234)
-    idx = torch.randperm(m, generator=g)[:rows].sort().values
-    a = A[0][idx.to(A.device)].cpu().numpy()
-    bt = Bt[0].cpu().numpy()
-    c = Ct[0][:, idx.to(Ct.device)].cpu().numpy().T          # (rows, n)
-    ref = orc.gemm_f64(a, bt.T)
-    c32 = orc.gemm_f32_tn(a, bt).T
-    return orc.max_rel_err(np.ascontiguousarray(c), ref), orc.max_rel_err(np.ascontiguousarray(c32), ref)
 
 
 def cpu_baseline(orc, w, target_s=15.0):
@@ -186,7 +206,8 @@ def bench_primitives(args, torch, tcec, dev, w):
         "vs_baseline": None, "dtype": "f16", "data": "synthetic",
         "config": {"workload": f"c2: {w['desc']}", "tiles": T},
         "roofline": {"bound": "hbm", "achieved": round(gbs, 1), "peak": PEAK_HBM_GBS, "unit": "GB/s",
-                     "frac": round(gbs / PEAK_HBM_GBS, 4), "traffic": MEASURED_TRAFFIC_BYTES.get("c2"),
+                     "frac": round(gbs / PEAK_HBM_GBS, 4), "traffic": measured_traffic("c2")[0],
+                     "traffic_source": measured_traffic("c2")[1],
                      "kernel": "primitive_tiles_kernel",
                      "kernel_ms": round(kernel_ms, 4), "algorithmic_bytes": nbytes},
         "tiles_per_s": round(T / (kernel_ms * 1e-3), 1),
@@ -212,49 +233,70 @@ def bench_primitives(args, torch, tcec, dev, w):
     print(json.dumps(res))
 
 
-def main():
-    ap = argparse.ArgumentParser()
-    ap.add_argument("--gpus", type=int, default=1)
-    ap.add_argument("--steps", type=int, default=None,
-                    help="timed steps; default 10 for the 16384^3 workloads and more for the short ones, so "
-                         "that the timed region lasts long enough for the clocks to settle")
-    ap.add_argument("--warmup", type=int, default=None, help="untimed steps; default 2 (20 for the short workloads)")
-    ap.add_argument("--workload", default="c4", choices=sorted(WORKLOADS))
-    ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
-    ap.add_argument("--no-accuracy", action="store_true")
-    ap.add_argument("--flags", type=int, default=0)
-    ap.add_argument("--dist", default=None, choices=["uniform", "normal", "exp", "zeros"],
-                    help="override the workload's input distribution (zeros: what the kernel reaches "
-                         "when the matrix cores are not power limited; not a valid benchmark value)")
-    ap.add_argument("--clock-trace", action="store_true",
-                    help="sample the shader clock on a second stream during the timed region and add "
-                         "its statistics to the JSON line (the matrix cores are power limited)")
-    ap.add_argument("--calibrate", action="store_true",
-                    help="after the timed region run one 1 GiB read + 1 GiB write elementwise kernel "
-                         "(the known-size copy that rocprofv3 FETCH_SIZE / WRITE_SIZE are scaled with)")
-    args = ap.parse_args()
-    if args.gpus != 1:
-        print("bench.py: this build measures one GPU only; --gpus must be 1 "
-              "(the path would shard by blocks of C or by batch entry, with no exchange)", file=sys.stderr)
-        sys.exit(2)
+def accuracy_block(torch, tcec, orc, A, Bt, Ct, rows):
+    """max|C - C64| / max|C64| on `rows` seeded full rows of batch 0 for the TCEC result and for
+    three plain fp32 products of the same rows: the oracle's sequential CPU loop, the vendor's
+    fp32 GEMM on the GPU and this library's fp32 policy (the API-level GEMM on the matrix core's
+    fp32 path).  The gate "no worse than 2x plain fp32" is reported against each."""
+    import numpy as np
+    m, k = A.shape[1], A.shape[2]
+    n = Bt.shape[1]
+    rows = min(rows, m)
+    g = torch.Generator().manual_seed(1234)
+    idx = torch.randperm(m, generator=g)[:rows].sort().values
+    a_rows = A[0][idx.to(A.device)].contiguous()                   # (rows, k)
+    a = a_rows.cpu().numpy()
+    bt = Bt[0].cpu().numpy()
+    c = Ct[0][:, idx.to(Ct.device)].cpu().numpy().T               # (rows, n)
+    ref = orc.gemm_f64(a, bt.T)
+    err = orc.max_rel_err(np.ascontiguousarray(c), ref)
+    plain = {"cpu_loop": orc.max_rel_err(np.ascontiguousarray(orc.gemm_f32_tn(a, bt).T), ref)}
+    prev = torch.backends.cuda.matmul.allow_tf32
+    torch.backends.cuda.matmul.allow_tf32 = False
+    try:
+        vend = torch.matmul(a_rows, Bt[0].t())
+        torch.cuda.synchronize()
+        plain["vendor_fp32_gemm_gpu"] = orc.max_rel_err(np.ascontiguousarray(vend.cpu().numpy()), ref)
+    finally:
+        torch.backends.cuda.matmul.allow_tf32 = prev
+    if rows % 128 == 0 and n % 128 == 0 and k % 32 == 0:
+        out = torch.empty((n, rows), dtype=torch.float32, device=A.device)
+        tcec.api_gemm(3, 0, rows, n, k, 1.0, a_rows, k, Bt[0], k, 0.0, out, rows)
+        torch.cuda.synchronize()
+        plain["fp32_policy_api_gemm_gpu"] = orc.max_rel_err(np.ascontiguousarray(out.cpu().numpy().T), ref)
+    return {
+        "max_rel_err_vs_fp64": float(f"{err:.4e}"),
+        "plain_fp32_max_rel_err_vs_fp64": float(f"{plain['cpu_loop']:.4e}"),
+        "plain_fp32_comparators": {k_: float(f"{v:.4e}") for k_, v in plain.items()},
+        "gate_2x_plain_fp32": {k_: bool(err <= 2 * v) for k_, v in plain.items()},
+        "accuracy_sample": f"{rows} seeded full rows of C (batch 0), FP64 host loop",
+    }
 
-    import torch
-    from wmma_extension_amd import _lib, tcec
-    _lib.lib()
-    dev = torch.device("cuda:0")
-    torch.cuda.set_device(dev)
-    w = dict(WORKLOADS[args.workload])
-    if args.warmup is None:
-        args.warmup = 20 if args.workload in DEFAULT_STEPS else 2
-    if args.steps is None:
-        args.steps = DEFAULT_STEPS.get(args.workload, 10)
+
+def cpu_config1(orc):
+    """The fixed CPU point: the oracle's fp32 loop at M=N=K=1024, uniform[-1,1], best of 3."""
+    import numpy as np
+    rng = np.random.default_rng(0x5EED + 1)
+    a = rng.uniform(-1, 1, (1024, 1024)).astype(np.float32)
+    b = rng.uniform(-1, 1, (1024, 1024)).astype(np.float32)
+    best = None
+    for _ in range(3):
+        t0 = time.perf_counter()
+        orc.gemm_f32_tn(a, b)
+        dt = time.perf_counter() - t0
+        best = dt if best is None else min(best, dt)
+    return {"m": 1024, "n": 1024, "k": 1024, "best_of": 3, "seconds": round(best, 5),
+            "gflops": round(2.0 * 1024 ** 3 / best / 1e9, 2)}
+
+
+def run_gemm_workload(args, torch, tcec, dev, name, steps, warmup):
+    """Times `steps` whole products of workload `name`; returns the fields of the JSON line that
+    describe it, plus the tensors the accuracy check needs."""
+    w = dict(WORKLOADS[name])
     if args.dist is not None:
         w["dist"] = args.dist
-    if w.get("kind") == "prim":
-        return bench_primitives(args, torch, tcec, dev, w)
     policy = tcec.Policy[w["policy"]]
     m, n, k, batch = w["m"], w["n"], w["k"], w["batch"]
-
     A, Bt = make_inputs(torch, w, dev, 0x5EED + 3)
     Ct = torch.empty((batch, n, m), dtype=torch.float32, device=dev)
     fused = bool(w.get("fused"))
@@ -282,18 +324,18 @@ def main():
         if ev is not None:
             ev[1].record()
 
-    for _ in range(args.warmup):
+    for _ in range(warmup):
         step()
     torch.cuda.synchronize()
     events = [(torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True))
-              for _ in range(args.steps)]
+              for _ in range(steps)]
     trace = None
     if args.clock_trace:
         # one more untimed step gives the length of the region to cover
         t0 = time.perf_counter()
         step()
         torch.cuda.synchronize()
-        est_ms = (time.perf_counter() - t0) * 1e3 * args.steps
+        est_ms = (time.perf_counter() - t0) * 1e3 * steps
         period = 10_000                                   # 100 us of the 100 MHz counter
         nsamples = int(min(50_000, (est_ms * 1.5 + 30.0) / 0.1))
         side = torch.cuda.Stream()
@@ -303,7 +345,7 @@ def main():
     if trace is None:
         torch.cuda.synchronize()
     t0 = time.perf_counter()
-    for i in range(args.steps):
+    for i in range(steps):
         step(events[i])
     if trace is not None:
         mark1 = tcec.clock_samples(1, 0)
@@ -313,17 +355,15 @@ def main():
     elapsed = time.perf_counter() - t0
     torch.cuda.synchronize()
 
-    if args.calibrate:
-        calibration_copy(torch, dev)
-
     flops = 2.0 * m * n * k * batch
-    ms_per_step = elapsed / args.steps * 1e3
-    value = flops / (elapsed / args.steps) / 1e12
-    gemm_ms = sum(e0.elapsed_time(e1) for e0, e1 in events) / args.steps
+    ms_per_step = elapsed / steps * 1e3
+    value = flops / (elapsed / steps) / 1e12
+    gemm_ms = sum(e0.elapsed_time(e1) for e0, e1 in events) / steps
     achieved = flops * w["mult"] / (gemm_ms * 1e-3) / 1e12
     bytes_min = 4.0 * (m * k + k * n + m * n) * batch
+    traffic, traffic_source = measured_traffic(name)
 
-    if args.workload in HBM_BOUND:
+    if name in HBM_BOUND:
         # packed operands in (2*terms bytes per element), C out: the GEMM kernel's own minimum
         terms = {"F16_EC": 2, "BF16X3_EC": 3, "BF16X2_EC": 2, "F16_NOEC": 1, "BF16_NOEC": 1}[w["policy"]]
         kbytes = (2.0 * terms * (m * k + k * n) + 4.0 * m * n) * batch
@@ -331,36 +371,28 @@ def main():
             kbytes = bytes_min              # fp32 A and B in, fp32 C out
         hbm = kbytes / (gemm_ms * 1e-3) / 1e9
         roofline = {"bound": "hbm", "achieved": round(hbm, 1), "peak": PEAK_HBM_GBS, "unit": "GB/s",
-                    "frac": round(hbm / PEAK_HBM_GBS, 4), "traffic": MEASURED_TRAFFIC_BYTES.get(args.workload),
+                    "frac": round(hbm / PEAK_HBM_GBS, 4), "traffic": traffic, "traffic_source": traffic_source,
                     "kernel": "tcec_gemm_fused_kernel" if fused else "tcec_gemm_kernel",
                     "kernel_ms": round(gemm_ms, 4), "algorithmic_bytes": kbytes, "mfma_frac": round(achieved / PEAK_MFMA_TFLOPS, 4)}
     else:
         roofline = {"bound": "mfma", "achieved": round(achieved, 2), "peak": PEAK_MFMA_TFLOPS,
                     "unit": "TFLOP/s", "frac": round(achieved / PEAK_MFMA_TFLOPS, 4),
-                    "traffic": MEASURED_TRAFFIC_BYTES.get(args.workload),
+                    "traffic": traffic, "traffic_source": traffic_source,
                     "kernel": "tcec_gemm_kernel", "kernel_ms": round(gemm_ms, 4),
                     "issued_flop_multiplier": w["mult"],
                     "hbm_frac_of_min_traffic": round(bytes_min / (gemm_ms * 1e-3) / 1e9 / PEAK_HBM_GBS, 4)}
     out = {
-        "metric": "TCEC SGEMM effective fp32 TFLOPS",
         "value": round(value, 3),
-        "unit": "TFLOPS",
-        "n_gpus": 1,
-        "steps": args.steps,
-        "warmup": args.warmup,
+        "steps": steps,
+        "warmup": warmup,
         "ms_per_step": round(ms_per_step, 4),
-        "higher_is_better": True,
-        "scaling": "weak",
-        "vs_baseline": None,
         "dtype": "bf16" if "BF16" in w["policy"] else "f16",
-        "data": "synthetic",
-        "config": {"workload": f"{args.workload}: {w['desc']}", "m": m, "n": n, "k": k, "batch": batch,
+        "config": {"workload": f"{name}: {w['desc']}", "m": m, "n": n, "k": k, "batch": batch,
                    "policy": w["policy"], "distribution": w["dist"], "flags": args.flags,
                    "step": ("one fused split+MFMA GEMM kernel; inputs resident in HBM" if fused else
                             "split+pack A, split+pack B, MFMA GEMM; inputs and workspace resident in HBM")},
         "roofline": roofline,
         "gemm_only_effective_tflops": round(flops / (gemm_ms * 1e-3) / 1e12, 3),
-        "fp32_vector_peak_tflops": 157.3,
     }
     if trace is not None:
         import numpy as np
@@ -381,14 +413,109 @@ def main():
                     "100 MHz counter; the timed region is delimited by two stamps on the work stream"}
     if not args.no_accuracy:
         from oracle import oracle as orc
-        rows = 64 if k >= 8192 else 256
-        err, err32 = accuracy_sample(torch, orc, A, Bt, Ct, min(rows, m))
-        out["max_rel_err_vs_fp64"] = float(f"{err:.4e}")
-        out["plain_fp32_max_rel_err_vs_fp64"] = float(f"{err32:.4e}")
-        out["accuracy_sample"] = f"{min(rows, m)} seeded full rows of C (batch 0), FP64 host loop"
+        out.update(accuracy_block(torch, tcec, orc, A, Bt, Ct, 128 if k >= 8192 else 256))
+    return out, w
+
+
+def bench_api_gemm(torch, tcec, dev, n=4096, steps=100, warmup=10):
+    """The GEMM written only against the public tcec:: device API (what a user of the headers
+    gets), fp16 hi+lo with error correction, uniform[-1,1], M=N=K=n."""
+    g = torch.Generator(device=dev)
+    g.manual_seed(0x5EED + 3)
+    A = torch.rand((n, n), generator=g, device=dev, dtype=torch.float32) * 2 - 1
+    Bt = torch.rand((n, n), generator=g, device=dev, dtype=torch.float32) * 2 - 1
+    C = torch.empty((n, n), dtype=torch.float32, device=dev)
+    for _ in range(warmup):
+        tcec.api_gemm(0, 1, n, n, n, 1.0, A, n, Bt, n, 0.0, C, n)
+    torch.cuda.synchronize()
+    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    e0.record()
+    for _ in range(steps):
+        tcec.api_gemm(0, 1, n, n, n, 1.0, A, n, Bt, n, 0.0, C, n)
+    e1.record()
+    torch.cuda.synchronize()
+    ms = e0.elapsed_time(e1) / steps
+    tf = 2.0 * n ** 3 / (ms * 1e-3) / 1e12
+    return {"kernel": "tcec_api_gemm_kernel (tcec::load_matrix_sync / mma_sync / utils::cp_async only)",
+            "workload": f"M=N=K={n}, fp16 hi+lo with EC, uniform[-1,1]", "steps": steps,
+            "ms_per_step": round(ms, 4), "value": round(tf, 2), "unit": "TFLOPS",
+            "mfma_frac": round(3 * tf / PEAK_MFMA_TFLOPS, 4)}
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=None,
+                    help="timed steps; default 80 (about 3 s) for the 16384^3 workloads and more for the short "
+                         "ones, so that the timed region lasts long enough for the clocks to settle")
+    ap.add_argument("--warmup", type=int, default=None, help="untimed steps; default 2 (20 for the short workloads)")
+    ap.add_argument("--workload", default="c4", choices=sorted(WORKLOADS))
+    ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
+    ap.add_argument("--no-accuracy", action="store_true")
+    ap.add_argument("--no-secondary", action="store_true",
+                    help="with the default workload: skip the 4096^3 half of the metric (c3) and the "
+                         "API-level GEMM figure")
+    ap.add_argument("--flags", type=int, default=0)
+    ap.add_argument("--dist", default=None, choices=["uniform", "normal", "exp", "zeros"],
+                    help="override the workload's input distribution (zeros: what the kernel reaches "
+                         "when the matrix cores are not power limited; not a valid benchmark value)")
+    ap.add_argument("--clock-trace", action="store_true",
+                    help="sample the shader clock on a second stream during the timed region and add "
+                         "its statistics to the JSON line (the matrix cores are power limited)")
+    ap.add_argument("--calibrate", action="store_true",
+                    help="after the timed region run one 1 GiB read + 1 GiB write elementwise kernel "
+                         "(the known-size copy that rocprofv3 FETCH_SIZE / WRITE_SIZE are scaled with)")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        print("bench.py: this build measures one GPU only; --gpus must be 1 "
+              "(the path would shard by blocks of C or by batch entry, with no exchange)", file=sys.stderr)
+        sys.exit(2)
+
+    import torch
+    from wmma_extension_amd import _lib, tcec
+    _lib.lib()
+    dev = torch.device("cuda:0")
+    torch.cuda.set_device(dev)
+    w = dict(WORKLOADS[args.workload])
+    if args.warmup is None:
+        args.warmup = 20 if args.workload in DEFAULT_STEPS else 2
+    if args.steps is None:
+        args.steps = DEFAULT_STEPS.get(args.workload, 80)
+    if w.get("kind") == "prim":
+        if args.dist is not None:
+            w["dist"] = args.dist
+        return bench_primitives(args, torch, tcec, dev, w)
+
+    main_out, w = run_gemm_workload(args, torch, tcec, dev, args.workload, args.steps, args.warmup)
+    if args.calibrate:
+        calibration_copy(torch, dev)
+    out = {
+        "metric": "TCEC SGEMM effective fp32 TFLOPS",
+        "value": main_out.pop("value"),
+        "unit": "TFLOPS",
+        "n_gpus": 1,
+        "steps": main_out.pop("steps"),
+        "warmup": main_out.pop("warmup"),
+        "ms_per_step": main_out.pop("ms_per_step"),
+        "higher_is_better": True,
+        "scaling": "weak",
+        "vs_baseline": None,
+        "dtype": main_out.pop("dtype"),
+        "data": "synthetic",
+    }
+    out.update(main_out)
+    out["fp32_vector_peak_tflops"] = 157.3
+    if args.workload == "c4" and not args.no_secondary and args.dist is None:
+        # the other half of the metric (4096^3, fp16 hi+lo) and the drop-in API's own GEMM
+        torch.cuda.empty_cache()
+        sec, _ = run_gemm_workload(args, torch, tcec, dev, "c3", DEFAULT_STEPS["c3"], 20)
+        sec["unit"] = "TFLOPS"
+        out["secondary"] = sec
+        out["api_level_gemm"] = bench_api_gemm(torch, tcec, dev)
     if not args.no_cpu:
         from oracle import oracle as orc
         out["cpu_baseline"] = cpu_baseline(orc, w)
+        out["cpu_baseline"]["config1_1024_cubed"] = cpu_config1(orc)
     else:
         out["cpu_baseline"] = None
     print(json.dumps(out))

@@ -337,14 +337,6 @@ int wmmae_fragment_eye(int shape, int identity, float alpha, float *out,
 int wmmae_direct_product(int elem, int terms, int from_float, const float *u,
                          const float *v, float *h, void *stream);
 
-/* Measurement aid (no counterpart in the reference): one wave writes nsamples
- * pairs out[2i] = constant-rate counter (100 MHz), out[2i+1] = shader cycle
- * counter, one pair every period_ticks of the constant counter, then ends
- * (nsamples * period_ticks <= 1e9, i.e. 10 s).  Launched on a second stream it
- * records the shader clock while other kernels run. */
-int wmmae_clock_samples(unsigned long long *out, int nsamples,
-                        long long period_ticks, void *stream);
-
 /* utils::cp_async<size> (size 4, 8 or 16 bytes per lane): 128 threads move 256
  * elements from src to dst through LDS.  mode 0: lane-linear destinations
  * (the reference's test), 1: scattered destinations, 2: every third thread
@@ -356,19 +348,21 @@ int wmmae_clock_samples(unsigned long long *out, int nsamples,
 int wmmae_utils_cp_async(int size, int mode, void *dst, const void *src,
                          void *stream);
 
+/* One wave prints (device printf, the process's stdout) a 16x16x16 half
+ * matrix_a fragment loaded from src (16x16 row-major fp32) with
+ * mtk::wmma::print_fragment, then a 32x32 TCEC accumulator filled with `base`
+ * (error part 2048*lane) with tcec::print_fragment: a title line and one line
+ * per lane each.  type 0..2, ec as in wmmae_tcec_mma_tile.
+ * Replaces: test/primitive/print_fragment.cu (detail/print.hpp,
+ * tcec/detail/print.hpp:11-55). */
+int wmmae_print_fragment(int type, int ec, const float *src, float base,
+                         void *stream);
+
 /* out[i] = utils::cast<DST>(in[i]); dst_type 0 half, 1 bfloat16 (out: 16-bit
  * patterns), 2 tf32, 3 float (out: fp32).
  * Replaces: test/utils/cast.cu:1-6 (utils::cast, utils.hpp:21-26). */
 int wmmae_utils_cast(int dst_type, const float *in, void *out, long long n,
                      void *stream);
-
-/* One raw MFMA D = A*B + C on 16-bit patterns (type 0 half, 1 bfloat16);
- * (m,n,k) one of (16,16,16), (16,16,32), (32,32,8), (32,32,16); a: m x k,
- * b: k x n, c/d: m x n, all row-major.
- * Replaces: test/primitive/mma.cu:11-45 (mma::mma_sync on one tile). */
-int wmmae_mfma_probe(int type, int m, int n, int k, float *d,
-                     const unsigned short *a, const unsigned short *b,
-                     const float *c, void *stream);
 
 #ifdef __cplusplus
 }

@@ -1,0 +1,35 @@
+/*
+ * Measurement aids of libwmmae_tcec.so that are no part of the product ABI
+ * (include/wmmae_tcec.h): they exist for the test suite and for bench.py.
+ * Same conventions: device pointers, `stream` a hipStream_t as void*, return 0
+ * or a negative wmmae_status.
+ */
+#ifndef WMMAE_TCEC_AUX_H
+#define WMMAE_TCEC_AUX_H
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+/* Measurement aid (no counterpart in the reference): one wave writes nsamples
+ * pairs out[2i] = constant-rate counter (100 MHz), out[2i+1] = shader cycle
+ * counter, one pair every period_ticks of the constant counter, then ends
+ * (nsamples * period_ticks <= 1e9, i.e. 10 s).  Launched on a second stream it
+ * records the shader clock while other kernels run. */
+int wmmae_clock_samples(unsigned long long *out, int nsamples,
+                        long long period_ticks, void *stream);
+
+/* One raw MFMA D = A*B + C on 16-bit patterns (type 0 half, 1 bfloat16);
+ * (m,n,k) one of (16,16,16), (16,16,32), (32,32,8), (32,32,16); a: m x k,
+ * b: k x n, c/d: m x n, all row-major.
+ * The instruction under the reference's test/primitive/mma.cu:11-45
+ * (mma::mma_sync on one tile), bare: the probe the oracle's model of the matrix
+ * core's accumulate arithmetic is measured and checked with. */
+int wmmae_mfma_probe(int type, int m, int n, int k, float *d,
+                     const unsigned short *a, const unsigned short *b,
+                     const float *c, void *stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* WMMAE_TCEC_AUX_H */

@@ -20,7 +20,12 @@ def h():
 
 def test_header_and_library_agree(h):
     text = open(os.path.join(ROOT, "include", "wmmae_tcec.h")).read()
+    aux = open(os.path.join(ROOT, "include", "wmmae_tcec_aux.h")).read()
     declared = set(re.findall(r"\b(wmmae_[a-z0-9_]+)\s*\(", text))
+    declared_aux = set(re.findall(r"\b(wmmae_[a-z0-9_]+)\s*\(", aux))
+    # the measurement aids live in their own header, outside the product ABI
+    assert declared_aux == {"wmmae_clock_samples", "wmmae_mfma_probe"} and not (declared & declared_aux)
+    declared |= declared_aux
     assert declared == set(_lib.EXPORTS)
     for name in declared:
         assert getattr(h, name) is not None

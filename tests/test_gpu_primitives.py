@@ -239,3 +239,25 @@ def test_gevm_identity_and_general(tc, orc, dev):
     y = tc.gevm(torch.from_numpy(x).to(dev), torch.from_numpy(_img(E, 1)).to(dev)).cpu().numpy()
     h = lambda v: v.astype(np.float16).astype(np.float64)
     assert np.abs(y - h(x) @ h(E)).max() < 1e-6
+
+
+def test_print_fragment_runs_and_prints_every_lane(dev):
+    """print_fragment of both layers in a one-wave kernel (test/primitive/print_fragment.cu):
+    run in a child process, whose stdout receives the device printf."""
+    import subprocess
+    import sys
+    code = (
+        "import torch, sys; sys.path.insert(0, %r)\n"
+        "from wmma_extension_amd import tcec\n"
+        "src = (torch.arange(256, dtype=torch.float32, device='cuda:0') / 4)\n"
+        "tcec.print_fragment(0, 1, src, 1.5)\n"
+        "torch.cuda.synchronize()\n") % os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+    out = subprocess.run([sys.executable, "-c", code], stdout=subprocess.PIPE, stderr=subprocess.PIPE,
+                         text=True, timeout=300)
+    assert out.returncode == 0, out.stderr[-2000:]
+    lines = [ln for ln in out.stdout.splitlines() if ln.strip()]
+    assert lines[0] == "prim_a = " and lines[65] == "tcec_acc = " and len(lines) == 130
+    # lane 0 of the matrix_a fragment holds row 0, k = 0..3 of the tile: 0, 0.25, 0.5, 0.75
+    assert lines[1].split() == ["+0.000e+00", "+2.500e-01", "+5.000e-01", "+7.500e-01"]
+    # lane 5 of the accumulator: 16 elements "(main)+(error / 2048)" = (1.5)+(5)
+    assert lines[66 + 5].split() == ["(+1.500e+00)+(+5.000e+00)"] * 16

@@ -56,6 +56,7 @@ EXPORTS = [
     "wmmae_direct_product",
     "wmmae_clock_samples",
     "wmmae_utils_cp_async",
+    "wmmae_print_fragment",
     "wmmae_utils_cast",
     "wmmae_mfma_probe",
 ]
@@ -137,6 +138,7 @@ _SIGNATURES = {
     "wmmae_direct_product": (_i, [_i, _i, _i, _vp, _vp, _vp, _vp]),
     "wmmae_clock_samples": (_i, [_vp, _i, _ll, _vp]),
     "wmmae_utils_cp_async": (_i, [_i, _i, _vp, _vp, _vp]),
+    "wmmae_print_fragment": (_i, [_i, _i, _vp, _c.c_float, _vp]),
     "wmmae_utils_cast": (_i, [_i, _vp, _vp, _ll, _vp]),
     "wmmae_mfma_probe": (_i, [_i, _i, _i, _i, _vp, _vp, _vp, _vp, _vp]),
 }

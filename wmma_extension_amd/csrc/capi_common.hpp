@@ -3,6 +3,7 @@
 // include/wmmae_tcec.h).
 #pragma once
 #include <wmmae_tcec.h>
+#include <wmmae_tcec_aux.h>
 
 #include <algorithm>
 #include <atomic>

@@ -168,6 +168,72 @@ inline int device_cus() {
   return prop.multiProcessorCount;
 }
 
+// ------------------------------------------------ fitted cost parameters
+// Every number the path and tile choices below are made with, in one place.
+// All are fits to measurements on MI355X (256 compute units, one box of the
+// pool each; the boxes differ by 3 to 5 % in what they sustain under the power
+// limit).  The estimates have one form: launch cost + rounds of tiles over the
+// compute units x (k stages of 32 x time per stage + time per tile), bounded
+// below by the bytes moved.
+namespace fit {
+// -- packed GEMM, time of one k stage of one tile, by stored terms (1, 2, 3).
+//    Sweep: 216 products, m = n = 512 .. 2048, k = 512 .. 4096, each run with
+//    1, 2, 3, 4, 6 and 8 K slices; the slice count chosen with them is within
+//    0.7 % of the best measured one on average (1.9 % on 120 random products
+//    with m, n = 64 .. 2900, k = 400 .. 32000, 1 .. 100 entries, 1 .. 32
+//    slices forced).
+constexpr double kStage256x128[3] = {0.8e-6, 1.0e-6, 1.0e-6}; // (no 3-term 256x128 kernel)
+constexpr double kStage128x128[3] = {0.45e-6, 0.6e-6, 0.99e-6};
+constexpr double kStage64x64 = 0.25e-6;
+constexpr double kTileOverhead = 7e-6;    // pipeline fill + epilogue of a tile
+constexpr double kFoldLaunch = 6e-6;      // the pass that adds the K slices
+constexpr double kFoldBytesPerS = 3e12;   // ... reads and writes its planes at
+constexpr double kSplitMustBeat = 0.95;   // a split has to win by 5 %
+// -- tile choice, cost of a tile in units of one 128x128 tile.  Sweep: both
+//    tiles forced on 124 products, 1024^2 .. 8192^2, k = 256 .. 4096, some
+//    batched: the choice is within 0.4 % of the faster tile on average.
+constexpr double kUnits256x128 = 2.0;
+constexpr double kUnits128x128 = 1.2;     // one and two terms (1.0 with three)
+constexpr double kUnits64x64 = 0.4;
+// -- K slices for a partly empty last round: slices, pipeline refills, fold.
+//    Sweep: 126 products, 2304^2 .. 8192^2, k = 2048 .. 8192, two policies.
+constexpr double kTailOverhead = 0.2;
+// -- single-kernel (fused) or packed path.  Sweep: 573 products measured with
+//    either path forced, m = n = 384 .. 4096, k = 64 .. 8192, 1 .. 256 entries,
+//    three policies (median error of either estimate 5 %; the choice costs
+//    0.8 % against always taking the faster path; refitted once after the tile
+//    rule changed: 0.7 % over 577 products).  Rows: one, two, three terms.
+struct PathRates {
+  double launch, stage, tile, bytes_per_s; // seconds, seconds, seconds, B/s
+  double split_bytes_per_s;                // packed path only
+};
+constexpr PathRates kFused[3] = {{5.0e-6, 0.76e-6, 3.0e-6, 5.0e12, 0.},
+                                 {5.0e-6, 1.11e-6, 3.0e-6, 5.0e12, 0.},
+                                 {5.0e-6, 1.41e-6, 3.1e-6, 5.0e12, 0.}};
+constexpr PathRates kPacked[3] = {{8.9e-6, 0.31e-6, 2.0e-6, 5.0e12, 6.6e12},
+                                  {6.5e-6, 0.50e-6, 3.8e-6, 3.6e12, 5.6e12},
+                                  {8.8e-6, 0.99e-6, 3.4e-6, 3.4e12, 5.9e12}};
+// the single kernel's 64x64 tile against its 128x128 tile (1024^3: 41 -> 27 us)
+constexpr double kFusedSmallTileTime = 0.65; // whole tile, latency-bound sizes
+constexpr double kFusedSmallStage = 0.33, kFusedSmallTile = 0.5;
+// 4-byte instead of 16-byte requests: 114 random products with k % 4 != 0 ran
+// at 0.55 of the packed path's speed in the median
+constexpr double kFusedNarrowRequests = 2.5;
+} // namespace fit
+
+// XCDs (chiplets with an L2 of their own) behind the current device.  HIP does
+// not report them; a gfx950 XCD has 32 active compute units in every partition
+// mode (SPX 256 = 8 x 32, DPX 128, QPX 64, CPX 32), so the count follows from
+// the compute units.  Consecutive workgroup ids go round-robin over the XCDs;
+// the kernels' XCD-aware item lists are written for eight of them and are used
+// only then (other counts take the plain shared list: same results, tiles not
+// grouped by L2).
+inline int device_xcds() {
+  const int cus = device_cus();
+  return cus % 32 == 0 ? cus / 32 : 1;
+}
+constexpr int kKernelXcds = 8; // the constant XCDS of the kernels' item lists
+
 // Number of K slices of every tile, when the 256x128 output tiles cannot fill
 // half the chip.  For every candidate (at most 32 slices of at least 6 stages)
 // the GEMM's time is estimated the way gemm_by_size will run it: the tile that
@@ -201,20 +267,22 @@ inline double split_time(const int terms, const int m, const int n,
   double stage_time, rounds;
   const double r_big = static_cast<double>(ceil_div(big, cus));
   const double r_mid = static_cast<double>(ceil_div(mid, cus));
-  if (big_tile_candidate(terms, mid, stages) && r_big * 2.0 <= r_mid * 1.2) {
-    stage_time = terms == 1 ? 0.8e-6 : 1.0e-6; // 256x128
+  if (big_tile_candidate(terms, mid, stages) &&
+      r_big * fit::kUnits256x128 <= r_mid * fit::kUnits128x128) {
+    stage_time = fit::kStage256x128[terms - 1];
     rounds = r_big;
   } else if (mid >= cus || (m > 64 && n > 64)) {
-    stage_time = terms == 1 ? 0.45e-6 : terms == 2 ? 0.6e-6 : 0.99e-6; // 128x128
+    stage_time = fit::kStage128x128[terms - 1];
     rounds = r_mid;
   } else {
-    stage_time = 0.25e-6; // 64x64
+    stage_time = fit::kStage64x64;
     rounds = static_cast<double>(
         ceil_div(ceil_div(m, 64) * ceil_div(n, 64) * batch * z, cus));
   }
-  double t = rounds * (stages * stage_time + 7e-6);
+  double t = rounds * (stages * stage_time + fit::kTileOverhead);
   if (z > 1)
-    t += 6e-6 + static_cast<double>(z + 1) * m * n * batch * 4.0 / 3e12;
+    t += fit::kFoldLaunch + static_cast<double>(z + 1) * m * n * batch * 4.0 /
+                                fit::kFoldBytesPerS;
   return t;
 }
 inline int choose_splits(const int terms, const int m, const int n, const int k,
@@ -224,7 +292,7 @@ inline int choose_splits(const int terms, const int m, const int n, const int k,
   if (tiles * 2 > device_cus())
     return 1;
   int best = 1;
-  double t_best = 0.95 * split_time(terms, m, n, batch, kt, 1);
+  double t_best = fit::kSplitMustBeat * split_time(terms, m, n, batch, kt, 1);
   for (int s = 2; s <= 32 && s * 6 <= kt; s++) {
     if (ceil_div(kt, ceil_div(kt, s)) != s)
       continue; // the same slices as a smaller count
@@ -269,7 +337,7 @@ inline double rounds_cost(const long long tiles, const long long resident,
     return full_rounds;
   if (!tail_allowed || t.slices < 2)
     return full_rounds + 1.0;
-  return full_rounds + 1.0 / t.slices + 0.2; // slices, pipeline refills, fold
+  return full_rounds + 1.0 / t.slices + fit::kTailOverhead;
 }
 
 // Deepest LDS ring (at most 4 stages) that fits the 160 KiB of a compute unit.
@@ -324,7 +392,8 @@ int launch_gemm(const GemmArgs &g) {
   const long long resident = static_cast<long long>(device_cus()) * per_cu;
   int grid = static_cast<int>(std::min(items, resident));
   int entry_per_xcd = 0;
-  if (zdim > 1 && resident >= 8 && resident % 8 == 0) {
+  const bool eight_xcds = device_xcds() == kKernelXcds;
+  if (zdim > 1 && eight_xcds && resident >= 8 && resident % 8 == 0) {
     // split-K: eight runs of the item list, one per XCD, so that an XCD holds
     // as few K slices as possible; the grid is padded to whole runs
     entry_per_xcd = 2;
@@ -335,7 +404,7 @@ int launch_gemm(const GemmArgs &g) {
   // (an XCD that owns one entry more than the others must not cost more
   // rounds than the shared list would take: 9 entries of 128 tiles are 8
   // rounds on the XCD with two entries, 5 on the shared list)
-  const bool by_xcd = resident >= 8 && resident % 8 == 0;
+  const bool by_xcd = eight_xcds && resident >= 8 && resident % 8 == 0;
   const long long owned_rounds =
       by_xcd ? ceil_div(static_cast<long long>(tiles_m) * tiles_n *
                             ceil_div(g.batch, 8),
@@ -421,10 +490,12 @@ template <class MT, int TERMS, bool RN> int gemm_by_size(const GemmArgs &g) {
       // time in units of one 128x128 tile: rounds * tile cost
       const bool tail_ok = g.batch == 1 && z == 1 && g.c_ptrs == nullptr &&
                            g.tail_ws != nullptr;
-      const double t_big = rounds_cost(big, cus, KT, tail_ok) * 2.0;
+      const double t_big =
+          rounds_cost(big, cus, KT, tail_ok) * fit::kUnits256x128;
       // (a 128x128 tile measured at 1.2 to 1.25 times half a 256x128 tile in
       // runs of two to eight rounds, 1.05 in long ones)
-      const double t_mid = rounds_cost(mid, cus, KT, tail_ok) * 1.2;
+      const double t_mid =
+          rounds_cost(mid, cus, KT, tail_ok) * fit::kUnits128x128;
       if (t_big <= t_mid)
         return launch_gemm<MT, TERMS, 256, 128, 2, 2, RN>(g);
     }
@@ -479,7 +550,7 @@ template <class T, int TERMS, int BM, int BN> int launch_fused(FusedArgs f) {
   const long long all_tiles =
       static_cast<long long>(p.batch) * p.tiles_per_batch;
   p.grouped =
-      p.batch >= 8 &&
+      device_xcds() == kKernelXcds && p.batch >= 8 &&
       ceil_div(ceil_div(p.batch, 8) * p.tiles_per_batch, per_xcd_max) * 100 <=
           ceil_div(all_tiles, 8ll * per_xcd_max) * 115;
   long long per_xcd = p.grouped
@@ -504,7 +575,8 @@ inline bool fused_small_tiles(const int m, const int n, const int batch) {
   const long long tiles128 = ceil_div(m, 128) * ceil_div(n, 128) * batch;
   const long long tiles64 = ceil_div(m, 64) * ceil_div(n, 64) * batch;
   return (m <= 64 && n <= 64) ||
-         (tiles128 < cus && 0.65 * static_cast<double>(ceil_div(tiles64, cus)) <
+         (tiles128 < cus && fit::kFusedSmallTileTime *
+                                    static_cast<double>(ceil_div(tiles64, cus)) <
                                 static_cast<double>(ceil_div(tiles128, cus)));
 }
 template <class T, int TERMS> int fused_by_size(const FusedArgs &f) {
@@ -541,10 +613,6 @@ int fused_dispatch(const int policy, const FusedArgs &f) {
 // 256 entries, one to three terms; median error of either estimate 5 %, the
 // choice costs 0.8 % over always taking the faster path).  K-heavy products
 // that want K slices stay on the packed path.
-struct PathRates {
-  double launch, stage, tile, bytes_per_s; // seconds, seconds, seconds, B/s
-  double split_bytes_per_s;                // packed path only
-};
 // fused_vec: the fused kernel can request 16 bytes per lane from both
 // operands (k contiguous, k and the strides multiples of 4, aligned bases).
 // Without that it issues four times as many requests and ran at 0.55 of the
@@ -563,15 +631,7 @@ inline bool use_fused(const int m, const int n, const int k, const int batch,
     return false;
   if (!fused_vec && k > 96)
     return false;
-  static const PathRates fused_rates[3] = {
-      {5.0e-6, 0.76e-6, 3.0e-6, 5.0e12, 0.},
-      {5.0e-6, 1.11e-6, 3.0e-6, 5.0e12, 0.},
-      {5.0e-6, 1.41e-6, 3.1e-6, 5.0e12, 0.}};
-  static const PathRates packed_rates[3] = {
-      {8.9e-6, 0.31e-6, 2.0e-6, 5.0e12, 6.6e12},
-      {6.5e-6, 0.50e-6, 3.8e-6, 3.6e12, 5.6e12},
-      {8.8e-6, 0.99e-6, 3.4e-6, 3.4e12, 5.9e12}};
-  const PathRates &f = fused_rates[terms - 1], &p = packed_rates[terms - 1];
+  const fit::PathRates &f = fit::kFused[terms - 1], &p = fit::kPacked[terms - 1];
   const long long cus = device_cus();
   const double kt = static_cast<double>(ceil_div(k, 32));
   const double c_bytes = 4.0 * m * n * batch;
@@ -586,9 +646,11 @@ inline bool use_fused(const int m, const int n, const int k, const int batch,
   const double f_rounds =
       static_cast<double>(ceil_div(small ? tiles64 : tiles128, cus));
   const double t_fused =
-      f.launch + std::max(f_rounds * (kt * f.stage * (fused_vec ? 1.0 : 2.5) *
-                                          (small ? 0.33 : 1.0) +
-                                      f.tile * (small ? 0.5 : 1.0)),
+      f.launch +
+      std::max(f_rounds * (kt * f.stage *
+                               (fused_vec ? 1.0 : fit::kFusedNarrowRequests) *
+                               (small ? fit::kFusedSmallStage : 1.0) +
+                           f.tile * (small ? fit::kFusedSmallTile : 1.0)),
                           (c_bytes + 4.0 * ab) / f.bytes_per_s);
 
   // packed path: rounds in units of one 128x128 tile as gemm_by_size counts
@@ -597,12 +659,13 @@ inline bool use_fused(const int m, const int n, const int k, const int batch,
   double units;
   const double r128 = static_cast<double>(ceil_div(tiles128, cus));
   if (big_tile_candidate(terms, tiles128, static_cast<int>(kt)) &&
-      2.0 * static_cast<double>(ceil_div(tiles256, cus)) <= 1.2 * r128)
-    units = 2.0 * static_cast<double>(ceil_div(tiles256, cus));
+      fit::kUnits256x128 * static_cast<double>(ceil_div(tiles256, cus)) <=
+          fit::kUnits128x128 * r128)
+    units = fit::kUnits256x128 * static_cast<double>(ceil_div(tiles256, cus));
   else if (tiles128 >= cus || (m > 64 && n > 64))
-    units = r128 * (terms <= 2 ? 1.2 : 1.0);
+    units = r128 * (terms <= 2 ? fit::kUnits128x128 : 1.0);
   else
-    units = 0.4 * static_cast<double>(ceil_div(tiles64, cus));
+    units = fit::kUnits64x64 * static_cast<double>(ceil_div(tiles64, cus));
   const double t_packed =
       p.launch + (4.0 + 2.0 * terms) * ab / p.split_bytes_per_s +
       std::max(units * (kt * p.stage + p.tile), c_bytes / p.bytes_per_s);

@@ -470,6 +470,28 @@ int wmmae_utils_cp_async(const int size, const int mode, void *const dst,
   return launch_status();
 }
 
+int wmmae_print_fragment(const int type, const int ec, const float *const src,
+                         const float base, void *const stream) {
+  if (!src)
+    return WMMAE_STATUS_NULL_POINTER;
+  if (type == 3 || !type_ec_supported(type, ec))
+    return WMMAE_STATUS_NOT_SUPPORTED;
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  return with_type(type, [&](auto tt) -> int {
+    using T = typename decltype(tt)::type;
+    if constexpr (std::is_same<T, float>::value)
+      return WMMAE_STATUS_NOT_SUPPORTED;
+    else
+      return with_ec(ec, [&](auto te) -> int {
+        using EC = typename decltype(te)::type;
+        using P = typename harness_policy<T, EC, 16, 16, 32>::type;
+        hipLaunchKernelGGL((wmmae_harness::print_fragment_kernel<T, P>), dim3(1),
+                           dim3(64), 0, s, src, base);
+        return launch_status();
+      });
+  });
+}
+
 int wmmae_utils_cast(const int dst_type, const float *const in, void *const out,
                      const long long n, void *const stream) {
   if (!in || !out)

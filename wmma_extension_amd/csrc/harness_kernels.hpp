@@ -40,6 +40,8 @@
 //   cp_async_kernel         : utils::cp_async global -> LDS copies
 //                             (reference: test/utils/cp_async.cu:15-25)
 //   cast_kernel             : utils::cast (reference: test/utils/cast.cu)
+//   print_fragment_kernel   : print_fragment of a primitive and a TCEC fragment
+//                             (reference: test/primitive/print_fragment.cu)
 #pragma once
 #include <wmma_extension/operators.hpp>
 #include <wmma_extension/tcec/complex.hpp>
@@ -762,6 +764,29 @@ __global__ void __launch_bounds__(128)
     cpa::wait_all();
     out(128 + t, &smem[1][t * W]);
   }
+}
+
+// print_fragment of both layers, one wave: a 16x16x16 half matrix_a fragment
+// loaded from `src` (16x16 row-major) and a 32x32 TCEC accumulator filled
+// with `base` whose error part is set to 2048 * lane (printed divided by the
+// split's scale).  Output goes to the process's stdout through device printf.
+// (reference: detail/print.hpp / tcec/detail/print.hpp:11-55, used by
+// test/primitive/print_fragment.cu)
+template <class T, class Policy>
+__global__ void __launch_bounds__(64)
+    print_fragment_kernel(const float *const src, const float base) {
+  w::fragment<w::matrix_a, 16, 16, 16, w::half, w::row_major> fa;
+  w::load_matrix_sync(fa, src, 16);
+  w::print_fragment(fa, "prim_a");
+  using F = tcec::fragment<w::accumulator, 32, 32, 32, T, void, Policy>;
+  F frag;
+  tcec::fill_fragment(frag, base);
+  if constexpr (F::num_terms >= 2) {
+    const unsigned lane = w::detail::common::get_lane_id();
+    for (unsigned i = 0; i < F::num_elements; i++)
+      frag.dx(i) = 2048.f * static_cast<float>(lane);
+  }
+  tcec::print_fragment(frag, "tcec_acc");
 }
 
 // utils::cast<DST>(in[i]) for DST = half, bfloat16 (16-bit patterns out),

@@ -347,6 +347,15 @@ def utils_cp_async(size, mode, src):
     return dst
 
 
+def print_fragment(type_, ec, src, base):
+    """Device printf of a primitive and a TCEC fragment (one wave) to the process's stdout."""
+    _need_cuda(src)
+    if src.dtype != torch.float32 or src.numel() < 256:
+        raise ValueError("src: 256 float32 values required")
+    st = _lib.lib().wmmae_print_fragment(type_, int(ec), _ptr(src), float(base), _stream())
+    _lib.check(st, "wmmae_print_fragment")
+
+
 def utils_cast(dst_type, x):
     """x: fp32 CUDA tensor -> int16 bit patterns (dst_type 0 half, 1 bfloat16) or fp32 (2 tf32, 3 float)."""
     _need_cuda(x)
