@@ -36,9 +36,11 @@ WORKLOADS = {
                        desc="strided-batched TCEC SGEMM, 1024 x 256^3, through packed operands"),
     "c5b": dict(m=1024, n=1024, k=262144, batch=1, policy="F16_EC", dist="normal", mult=3,
                 desc="K-heavy TCEC SGEMM, M=N=1024, K=262144"),
+    "api": dict(kind="api", m=4096, n=4096, k=4096, dist="uniform",
+                desc="GEMM written against the public tcec:: device API only, fp16 hi+lo with EC, M=N=K=4096"),
 }
 # a timed region of a few milliseconds is measured while the power management still ramps
-DEFAULT_STEPS = {"c3": 200, "c5a": 400, "c5a_packed": 200, "c5b": 50, "c2": 100}
+DEFAULT_STEPS = {"c3": 200, "c5a": 400, "c5a_packed": 200, "c5b": 50, "c2": 100, "api": 200}
 PEAK_MFMA_TFLOPS = 2500.0      # dense fp16 / bf16 MFMA, MI355X
 PEAK_HBM_GBS = 8000.0
 # workloads whose dominant kernel is bound by HBM rather than by the matrix cores
@@ -485,6 +487,19 @@ def main():
         if args.dist is not None:
             w["dist"] = args.dist
         return bench_primitives(args, torch, tcec, dev, w)
+    if w.get("kind") == "api":
+        r = bench_api_gemm(torch, tcec, dev, w["m"], args.steps, args.warmup)
+        print(json.dumps({
+            "metric": "TCEC SGEMM effective fp32 TFLOPS", "value": r["value"], "unit": "TFLOPS", "n_gpus": 1,
+            "steps": args.steps, "warmup": args.warmup, "ms_per_step": r["ms_per_step"],
+            "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "f16", "data": "synthetic",
+            "config": {"workload": f"api: {w['desc']}"},
+            "roofline": {"bound": "mfma", "achieved": round(3 * r["value"], 2), "peak": PEAK_MFMA_TFLOPS,
+                         "unit": "TFLOP/s", "frac": r["mfma_frac"], "traffic": None,
+                         "kernel": "tcec_api_gemm_kernel", "kernel_ms": r["ms_per_step"],
+                         "issued_flop_multiplier": 3},
+            "cpu_baseline": None}))
+        return
 
     main_out, w = run_gemm_workload(args, torch, tcec, dev, args.workload, args.steps, args.warmup)
     if args.calibrate:

@@ -308,31 +308,23 @@ __global__ void __launch_bounds__(64 * NW)
         for (int x = 0; x < 8; x++)
           v[q][x] = x < left ? v[q][x] : 0.f;
       }
-      // the split of split_traits<T>, two elements at a time so that the
-      // packed conversions are used: t0 = RN16(v), t1 = RN16((v - t0) * scale),
-      // t2 = RN16((v - t0) - t1)
-      typedef S s2_t __attribute__((ext_vector_type(2)));
-      typedef float f2_t __attribute__((ext_vector_type(2)));
+      // the split of split_traits<T>, four elements at a time in the form
+      // that uses the packed conversions (and for fp16 the mixed-precision
+      // fma): t0 = RN16(v), t1 = RN16((v - t0) * scale), t2 = RN16((v - t0) - t1)
+      S term[3][8];
+#pragma unroll
+      for (int x = 0; x < 8; x += 4) {
+        const mtk::wmma::tcec::detail::f32x4_t vv = {v[q][x], v[q][x + 1],
+                                                     v[q][x + 2], v[q][x + 3]};
+        mtk::wmma::tcec::detail::split4<T>(vv, &term[0][x], &term[1][x],
+                                           &term[2][x]);
+      }
       ab_vec t[3];
 #pragma unroll
-      for (int x = 0; x < 8; x += 2) {
-        const f2_t vv = {v[q][x], v[q][x + 1]};
-        const s2_t h0 = __builtin_convertvector(vv, s2_t);
-        f2_t r = vv - __builtin_convertvector(h0, f2_t);
-        if constexpr (traits::scale != 1.f)
-          r *= traits::scale;
-        const s2_t h1 = __builtin_convertvector(r, s2_t);
-        s2_t h2 = h1;
-        if constexpr (traits::num_terms >= 3)
-          h2 = __builtin_convertvector(r - __builtin_convertvector(h1, f2_t),
-                                       s2_t);
-        t[0][x] = h0[0];
-        t[0][x + 1] = h0[1];
-        t[1][x] = h1[0];
-        t[1][x + 1] = h1[1];
-        t[2][x] = h2[0];
-        t[2][x + 1] = h2[1];
-      }
+      for (int c = 0; c < TERMS; c++)
+#pragma unroll
+        for (int x = 0; x < 8; x++)
+          t[c][x] = term[c][x];
 #pragma unroll
       for (int c = 0; c < TERMS; c++)
         frag[((buf * NRB + rbl) * TERMS + c) * 64 + lane] =
