@@ -96,11 +96,7 @@ template <int N> __device__ __forceinline__ void wait_vmcnt_at_most() {
   asm volatile("s_waitcnt vmcnt(%0)" ::"n"(N > 63 ? 63 : N) : "memory");
 }
 
-// ABLATE (tuning only, 0 in the library): bit 0 drops the global->LDS requests,
-// bit 1 the conversion, bit 2 the MFMAs, bit 3 the per-stage barrier, bit 4 the
-// stores of C; bit 6 replaces the result by per-phase cycle counts (written
-// over C).
-template <class T, int TERMS, int BM, int BN, int ABLATE = 0,
+template <class T, int TERMS, int BM, int BN,
           int NW = FusedConfig<TERMS, BM, BN>::NWAVES>
 __global__ void __launch_bounds__(64 * NW)
     tcec_gemm_fused_kernel(const FusedParams p) {
@@ -220,8 +216,6 @@ __global__ void __launch_bounds__(64 * NW)
   };
   // VEC: std::true_type for 16-byte requests (both operands), else 4-byte ones
   auto issue = [&](auto VEC, const int ks, const int slot) __attribute__((always_inline)) {
-    if constexpr ((ABLATE & 1) != 0)
-      return;
 #pragma unroll
     for (int q = 0; q < NQ; q++) {
       const int rbl = wave + NW * q;
@@ -274,11 +268,7 @@ __global__ void __launch_bounds__(64 * NW)
       const int rbl = wave + NW * q;
       const unsigned char *const src =
           lds_raw + slot * Cfg::RAW_STAGE_BYTES + rbl * 2048;
-      if constexpr ((ABLATE & 2) != 0) {
-#pragma unroll
-        for (int x = 0; x < 8; x++)
-          v[q][x] = 0.f;
-      } else if constexpr (decltype(VEC)::value) {
+      if constexpr (decltype(VEC)::value) {
         const f32x4 lo = *reinterpret_cast<const f32x4 *>(src + vec_off_lo);
         const f32x4 hi = *reinterpret_cast<const f32x4 *>(src + vec_off_hi);
 #pragma unroll
@@ -296,8 +286,6 @@ __global__ void __launch_bounds__(64 * NW)
   // conversion, second half: split and write the terms of k stage `ks` into
   // fragment buffer `buf`
   auto split_store = [&](const int ks, const int buf, float (&v)[NQ][8]) __attribute__((always_inline)) {
-    if constexpr ((ABLATE & 2) != 0)
-      return;
 #pragma unroll
     for (int q = 0; q < NQ; q++) {
       const int rbl = wave + NW * q;
@@ -332,10 +320,7 @@ __global__ void __launch_bounds__(64 * NW)
     }
   };
   auto mfma = [](const ab_vec x, const ab_vec y, const f32x4 z) -> f32x4 {
-    if constexpr ((ABLATE & 4) != 0)
-      return z + f32x4{static_cast<float>(x[0]), static_cast<float>(y[0]), 0.f,
-                       0.f};
-    else if constexpr (std::is_same<S, _Float16>::value)
+    if constexpr (std::is_same<S, _Float16>::value)
       return __builtin_amdgcn_mfma_f32_16x16x32_f16(x, y, z, 0, 0, 0);
     else
       return __builtin_amdgcn_mfma_f32_16x16x32_bf16(x, y, z, 0, 0, 0);
@@ -463,20 +448,6 @@ __global__ void __launch_bounds__(64 * NW)
     // every wave has stage 0 in registers before anybody overwrites its buffer
     asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");
 
-    // tuning only (ABLATE bit 6): shader-clock time spent per phase, written to C
-    unsigned long long prof[6] = {0, 0, 0, 0, 0, 0};
-    unsigned long long stamp = 0;
-    auto tick = [&](const int phase) __attribute__((always_inline)) {
-      if constexpr ((ABLATE & 64) != 0) {
-        __builtin_amdgcn_sched_barrier(0);
-        const unsigned long long now = __builtin_amdgcn_s_memtime();
-        if (phase >= 0)
-          prof[phase] += now - stamp;
-        stamp = now;
-        __builtin_amdgcn_sched_barrier(0);
-      }
-    };
-
     // The k loop of a tile is a loop of its own so that the accumulators are
     // touched by nothing but MFMAs inside it (they stay in AGPRs); the stream
     // of requests and conversions runs on across the tile boundary.
@@ -486,14 +457,11 @@ __global__ void __launch_bounds__(64 * NW)
       clear_acc();
       for (int cur_ks = 0; cur_ks < num_k; cur_ks++, s++) {
         const int buf = s & 1;
-        tick(-1);
         // refill the slot that stage s+1 has left (it was converted last
         // iteration): it is the one before slot_conv
         issue(VEC, req_ks, slot_conv == 0 ? NRAW - 1 : slot_conv - 1);
         advance_request();
-        tick(0);
         wait_oldest_stage(VEC); // stage s+2 (past the end: a redundant tail stage)
-        tick(1);
         load_raw(VEC, slot_conv, v);
 
         auto sweep = [&](f32x4(&acc)[MT_][NT_], const int ta, const int tb) __attribute__((always_inline)) {
@@ -504,7 +472,10 @@ __global__ void __launch_bounds__(64 * NW)
               acc[i][j] = mfma(a[ta][i], b[tb][j], acc[i][j]);
         };
         auto multiply = [&]() __attribute__((always_inline)) {
-          // same products and order as tcec_gemm_kernel
+          // same products and, per accumulator, the same order as
+          // tcec_gemm_kernel.  (That kernel's tile-major issue order, a
+          // tile's products back to back, was measured here too: this kernel
+          // is not limited by the matrix core's power and ran 7 % slower.)
           if constexpr (TERMS >= 3) {
             sweep(acc_err, 2, 0);
             sweep(acc_err, 0, 2);
@@ -533,32 +504,16 @@ __global__ void __launch_bounds__(64 * NW)
         const bool matrix_first = NW < 8 || wave < NW / 2;
         if (matrix_first)
           multiply();
-        tick(2);
         // stage s+2 over the buffer of stage s, which every wave took into
         // registers before the last barrier
         split_store(conv_ks, buf, v);
-        tick(3);
         if (!matrix_first)
           multiply();
         advance_conv();
         slot_conv = slot_conv + 1 == NRAW ? 0 : slot_conv + 1;
-        if constexpr ((ABLATE & 8) == 0)
-          asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");
-        tick(4);
+        asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");
       }
-      tick(-1);
-      if constexpr ((ABLATE & 16) == 0)
-        store_tile(cur_tile);
-      else if (acc_main[0][0][0] == 123.456f) // keep the accumulators alive
-        store_tile(cur_tile);
-      tick(5);
-    }
-    if constexpr ((ABLATE & 64) != 0) {
-      asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
-      if (lane == 0)
-        for (int i = 0; i < 6; i++)
-          reinterpret_cast<unsigned long long *>(
-              p.C)[(blockIdx.x * NW + wave) * 8 + i] = prof[i];
+      store_tile(cur_tile);
     }
   };
   if (vec_a && vec_b)

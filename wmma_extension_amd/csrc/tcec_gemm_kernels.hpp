@@ -319,12 +319,6 @@ __global__ void __launch_bounds__(256)
 //
 // C is column major (element (i,j) at C[i + j*ldc]); an accumulator lane owns
 // four consecutive rows of one column, i.e. one 16-byte store.
-//
-// ABLATE (tuning only, 0 in the library): bit 0 drops the global->LDS requests
-// of the main loop, bit 1 its LDS reads, bit 2 its barriers, bit 3 the wait
-// for the requests, bit 4 the MFMAs, bit 5 makes every block read tile (0,0),
-// bit 7 drops every fourth request, bit 8 every fourth LDS read.
-// Results are then wrong; the variants exist to time the remaining parts.
 // --------------------------------------------------------------------------
 template <class MT, int TERMS, int BM, int BN, int WGM, int WGN, int NSTAGE,
           bool RN_MAIN>
@@ -347,7 +341,7 @@ struct GemmConfig {
 };
 
 template <class MT, int TERMS, int BM, int BN, int WGM, int WGN, int NSTAGE,
-          bool RN_MAIN, int ABLATE = 0>
+          bool RN_MAIN>
 __global__ void __launch_bounds__(WGM *WGN * 64)
     tcec_gemm_kernel(const u32x4 *__restrict__ Ap, const u32x4 *__restrict__ Bp,
                      float *__restrict__ C, const int M, const int N,
@@ -452,8 +446,6 @@ __global__ void __launch_bounds__(WGM *WGN * 64)
     }
     tile_of<(BM > BN ? 4u : 8u)>(pid, num_tiles, tiles_m, tiles_n,
                                  !entry_per_xcd, it.tm, it.tn);
-    if constexpr ((ABLATE & 32) != 0)
-      it.tm = it.tn = 0;
     return it;
   };
   // Split-K: with `partial` set, slice z covers split_stages k stages from
@@ -573,11 +565,12 @@ __global__ void __launch_bounds__(WGM *WGN * 64)
   // In-place accumulate, written as inline assembly so that every accumulator
   // stays in one fixed accumulation register for the whole K loop (with the
   // largest tile the accumulators fill the register file exactly, and the
-  // register allocator otherwise shuffles them every iteration).  Used only
-  // when a sweep has at least eight tiles: dependent MFMAs on one accumulator
-  // are then at least eight 16-cycle instructions apart, beyond any software
-  // wait state the matrix core needs; smaller wave tiles use the builtin and
-  // leave the hazards to the compiler.
+  // register allocator otherwise shuffles them every iteration).  The only
+  // dependence between the MFMAs of a step is an MFMA whose accumulator is
+  // the destination of the one just before it, same shape and same
+  // registers, which the matrix core takes back to back without software
+  // wait states (the compiler emits none for the builtin either).  Small wave
+  // tiles use the builtin.
   constexpr bool USE_ASM = MT_ * NT_ >= 8;
   auto mfma_acc = [](f32x4 &z, const ab_vec x, const ab_vec y) {
     if constexpr (std::is_same<MT, _Float16>::value)
@@ -619,25 +612,17 @@ __global__ void __launch_bounds__(WGM *WGN * 64)
     }
   };
 
-  // MFMAs of one step in issue order: the error products (smallest first) and
-  // then the main product; every product sweeps all tiles before the next one
-  // starts, so consecutive MFMAs never depend on each other.
+  // MFMAs of one step in issue order: tile after tile, and for every tile the
+  // error products (smallest first) and then the main product.
   constexpr int NPROD = TERMS == 1 ? 1 : (TERMS == 2 ? 3 : 6);
   constexpr int NTILE = MT_ * NT_;
   constexpr int NMFMA = NPROD * NTILE;
   // LDS read r of the next stage goes out after MFMA number (r+1)*SPAN/NFRAG:
   // the reads are spread over the first three quarters of the step (the LGKM
   // counter only tracks 15 outstanding operations)
-#ifndef WMMAE_TUNE_SPAN_NUM
-#define WMMAE_TUNE_SPAN_NUM 3
-#define WMMAE_TUNE_SPAN_DEN 4
-#endif
   // MFMA after which the last request of a step goes out
   constexpr int N_ADVANCE = (NMFMA * (CPW - 1)) / CPW;
-  constexpr int SPAN =
-      (NMFMA * WMMAE_TUNE_SPAN_NUM) / WMMAE_TUNE_SPAN_DEN > 0
-          ? (NMFMA * WMMAE_TUNE_SPAN_NUM) / WMMAE_TUNE_SPAN_DEN
-          : 1;
+  constexpr int SPAN = (NMFMA * 3) / 4 > 0 ? (NMFMA * 3) / 4 : 1;
 
   // One pipeline step: multiply the fragments of stage st (already in
   // registers) while the fragments of stage st+1 are read from LDS and stage
@@ -657,29 +642,32 @@ __global__ void __launch_bounds__(WGM *WGN * 64)
     int r_base = rbuf * (NCH * 1024);
     asm volatile("" : "+s"(w_base), "+s"(r_base));
     // own loads of the next stage landed; own LDS reads of this stage finished
-    if constexpr ((ABLATE & 4) == 0) {
-      // the requests of the stage read next are older than those of the
-      // NSTAGE-2 stages after it (the branch sits before the barrier, where
-      // the wave waits anyway)
-      if (skip_waits > 0)
-        skip_waits--;
-      else
-        asm volatile("s_waitcnt vmcnt(%0)" ::"n"((ABLATE & 8)
-                                                     ? 63
-                                                     : CPW * (NSTAGE - 2))
-                     : "memory");
-      asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");
-    }
+    // the requests of the stage read next are older than those of the
+    // NSTAGE-2 stages after it (the branch sits before the barrier, where
+    // the wave waits anyway)
+    if (skip_waits > 0)
+      skip_waits--;
+    else
+      asm volatile("s_waitcnt vmcnt(%0)" ::"n"(CPW * (NSTAGE - 2)) : "memory");
+    asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");
 
     static_for<0, NMFMA>([&](auto N_) {
       constexpr int n = decltype(N_)::value;
-      constexpr int p = n / NTILE;
-      // tiles in serpentine order: consecutive MFMAs share the A fragment
-      // along a row of tiles and the B fragment at the turn (fewer operand
-      // bits change between instructions; measured 1 % faster under the
-      // power limit)
-      constexpr int i = (n % NTILE) / NT_;
-      constexpr int j = (i % 2) ? NT_ - 1 - n % NT_ : n % NT_;
+      // Tile-major order: the products of one tile follow each other (the
+      // error products chained through its error accumulator, then the main
+      // product), tiles in serpentine order so that neighbouring tiles share
+      // the A fragment along a row and the B fragment at the turn.  Each
+      // accumulator sees the same sequence of products as in a product-major
+      // sweep, so the result bits do not depend on this choice; a chain of
+      // MFMAs on one accumulator costs the matrix core less power than the
+      // same MFMAs spread over many accumulators, and under the power limit
+      // that is time (16384^3, three bf16 terms: 35.0 -> 33.1 ms; 4096^3 fp16:
+      // 0.289 -> 0.280 ms).  The hardware supports back-to-back dependent
+      // MFMAs of one shape on one destination without wait states.
+      constexpr int p = n % NPROD;
+      constexpr int tile = n / NPROD;
+      constexpr int i = tile / NT_;
+      constexpr int j = (i % 2) ? NT_ - 1 - tile % NT_ : tile % NT_;
       // (term of A, term of B) of product p
       constexpr int ta =
           TERMS == 1   ? 0
@@ -692,9 +680,7 @@ __global__ void __launch_bounds__(WGM *WGN * 64)
                                                            : p == 4   ? 1
                                                                       : 0);
       constexpr bool is_main = p == NPROD - 1;
-      if constexpr ((ABLATE & 16) != 0) {
-        // tuning: no matrix work at all
-      } else if constexpr (is_main && RN_MAIN) {
+      if constexpr (is_main && RN_MAIN) {
         acc_main[i][j] +=
             mfma(cur.a[0][i], cur.b[0][j], f32x4{0.f, 0.f, 0.f, 0.f});
       } else if constexpr (USE_ASM) {
@@ -709,9 +695,7 @@ __global__ void __launch_bounds__(WGM *WGN * 64)
       constexpr int qlo = (n * CPW + NMFMA - 1) / NMFMA;
       constexpr int qhi = ((n + 1) * CPW + NMFMA - 1) / NMFMA;
       static_for<qlo, (qhi < CPW ? qhi : CPW)>([&](auto Q) {
-        if constexpr ((ABLATE & 1) == 0 &&
-                      !((ABLATE & 128) != 0 && decltype(Q)::value % 4 == 3))
-          issue_chunk(w_base, Q);
+        issue_chunk(w_base, Q);
         __builtin_amdgcn_sched_barrier(0);
       });
       // all requests of this step are out: move the cursor on while the
@@ -724,9 +708,7 @@ __global__ void __launch_bounds__(WGM *WGN * 64)
       constexpr int lo = n == 0 ? 0 : reads_due(n, SPAN, NFRAG);
       constexpr int hi = n + 1 == NMFMA ? NFRAG : reads_due(n + 1, SPAN, NFRAG);
       static_for<lo, hi>([&](auto R_) {
-        if constexpr ((ABLATE & 2) == 0 &&
-                      !((ABLATE & 256) != 0 && decltype(R_)::value % 4 == 3))
-          read_frag(nxt, r_base, R_);
+        read_frag(nxt, r_base, R_);
         __builtin_amdgcn_sched_barrier(0);
       });
     });
