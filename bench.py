@@ -57,8 +57,12 @@ TRAFFIC_PROFILES = {
     "c5a": "tcec_gemm_fused_kernel_c5a_1024x256_f16.md",
     "c5b": "tcec_gemm_kernel_c5b_1024x1024x262144_f16.md",
     "c2": "primitive_tiles_kernel_c2_1M_tiles.md",
+    "api": "tcec_api_gemm_kernel_api_4096_f16.md",
 }
 KERNEL_SOURCES = {
+    "api": ["tcec_api_gemm_kernel.hpp", "include/wmma_extension/tcec/tcec.hpp",
+            "include/wmma_extension/tcec/detail/split.hpp", "include/wmma_extension/utils.hpp",
+            "include/wmma_extension/wmma_extension.hpp", "include/wmma_extension/detail/mfma.hpp"],
     "c4": ["tcec_gemm_kernels.hpp"], "c3": ["tcec_gemm_kernels.hpp"], "c5b": ["tcec_gemm_kernels.hpp"],
     "c5a": ["tcec_gemm_kernels.hpp", "tcec_gemm_fused_kernel.hpp"], "c2": ["harness_kernels.hpp"],
 }
@@ -68,7 +72,8 @@ def kernel_sources_hash(workload):
     import hashlib
     h = hashlib.sha256()
     for name in KERNEL_SOURCES.get(workload, []):
-        with open(os.path.join(ROOT, "wmma_extension_amd", "csrc", name), "rb") as f:
+        path = os.path.join(ROOT, name) if "/" in name else os.path.join(ROOT, "wmma_extension_amd", "csrc", name)
+        with open(path, "rb") as f:
             h.update(f.read())
     return h.hexdigest()[:12]
 
@@ -489,14 +494,17 @@ def main():
         return bench_primitives(args, torch, tcec, dev, w)
     if w.get("kind") == "api":
         r = bench_api_gemm(torch, tcec, dev, w["m"], args.steps, args.warmup)
+        if args.calibrate:
+            calibration_copy(torch, dev)
+        traffic, traffic_source = measured_traffic("api")
         print(json.dumps({
             "metric": "TCEC SGEMM effective fp32 TFLOPS", "value": r["value"], "unit": "TFLOPS", "n_gpus": 1,
             "steps": args.steps, "warmup": args.warmup, "ms_per_step": r["ms_per_step"],
             "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "f16", "data": "synthetic",
             "config": {"workload": f"api: {w['desc']}"},
             "roofline": {"bound": "mfma", "achieved": round(3 * r["value"], 2), "peak": PEAK_MFMA_TFLOPS,
-                         "unit": "TFLOP/s", "frac": r["mfma_frac"], "traffic": None,
-                         "kernel": "tcec_api_gemm_kernel", "kernel_ms": r["ms_per_step"],
+                         "unit": "TFLOP/s", "frac": r["mfma_frac"], "traffic": traffic,
+                         "traffic_source": traffic_source, "kernel": "tcec_api_gemm_kernel", "kernel_ms": r["ms_per_step"],
                          "issued_flop_multiplier": 3},
             "cpu_baseline": None}))
         return

@@ -13,6 +13,7 @@
 // wave64-collective; `sync` arguments are accepted and ignored because a wave
 // runs in lock step.
 #pragma once
+#include "detail/functions.hpp"
 #include "detail/policy.hpp"
 #include "detail/split.hpp"
 
@@ -42,6 +43,28 @@ WMMAE_HD unsigned mem_offset(const unsigned i, const unsigned j,
   else
     return (j + n_offset) + (i + m_offset) * ldm;
 }
+
+// The same offsets as function objects under the reference's name
+// (tcec/detail/common.hpp:32-63): from the mem_index a foreach callback
+// receives for a frag_m x frag_n sub-block, or from a position (i, j).
+template <int frag_m, int frag_n, class Layout> struct compute_mem_offset {
+  WMMAE_HD unsigned operator()(const unsigned mem_index, const unsigned ldm,
+                               const unsigned m_offset,
+                               const unsigned n_offset) const {
+    constexpr unsigned lead =
+        std::is_same<Layout, col_major>::value ? frag_m : frag_n;
+    const unsigned major = mem_index / lead, minor = mem_index % lead;
+    if constexpr (std::is_same<Layout, col_major>::value)
+      return mem_offset<Layout>(minor, major, ldm, m_offset, n_offset);
+    else
+      return mem_offset<Layout>(major, minor, ldm, m_offset, n_offset);
+  }
+  WMMAE_HD unsigned operator()(const unsigned i, const unsigned j,
+                               const unsigned ldm, const unsigned m_offset,
+                               const unsigned n_offset) const {
+    return mem_offset<Layout>(i, j, ldm, m_offset, n_offset);
+  }
+};
 } // namespace detail
 
 template <class Use, int m, int n, int k, class T, class Layout = void,

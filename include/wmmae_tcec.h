@@ -298,7 +298,10 @@ int wmmae_tcec_mma_complex(int type, int ec, float *d, const float *a,
  * store_matrix_sync.  elem: 0 half, 1 bfloat16, 2 float; shape: 0 16x16x16,
  * 1 16x16x32, 2 32x32x8, 3 32x32x16 (float: shapes 0 and 2); a (M x K),
  * b (K x N), c, d (M x N): fp32 images, dense, *_col = 1 for column major;
- * c may be NULL.  Replaces: test/primitive/mma.cu:11-45. */
+ * c may be NULL.  shape + 8: the same MMA through the policy-dispatched
+ * function objects of tcec::detail (reference:
+ * include/wmma_extension/tcec/detail/functions.hpp:10-348, compute_mem_offset
+ * of tcec/detail/common.hpp:32-63).  Replaces: test/primitive/mma.cu:11-45. */
 int wmmae_primitive_mma(int elem, int shape, float *d, const float *a,
                         const float *b, const float *c, int a_col, int b_col,
                         int c_col, int d_col, void *stream);

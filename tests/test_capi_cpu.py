@@ -169,6 +169,8 @@ def test_primitive_entries_reject_bad_arguments_on_the_host(h):
     p = ctypes.c_void_p(64)
     assert h.wmmae_primitive_mma(3, 0, p, p, p, p, 0, 0, 0, 0, None) == -1
     assert h.wmmae_primitive_mma(0, 4, p, p, p, p, 0, 0, 0, 0, None) == -1
+    assert h.wmmae_primitive_mma(0, 12, p, p, p, p, 0, 0, 0, 0, None) == -1    # 8 + shape: wrappers
+    assert h.wmmae_primitive_mma(2, 9, p, p, p, p, 0, 0, 0, 0, None) == -4
     assert h.wmmae_primitive_mma(2, 1, p, p, p, p, 0, 0, 0, 0, None) == -4     # fp32 has no 16x16x32
     assert h.wmmae_primitive_mma(0, 0, None, p, p, p, 0, 0, 0, 0, None) == -2
     assert h.wmmae_foreach_ec(p, None, p, None) == -2

@@ -184,6 +184,14 @@ def test_primitive_mma_all_shapes(tc, orc, dev, elem, shape):
         D = d.reshape(n, m).T if d_col else d.reshape(m, n)
         ref = orc.gemm_f64(A, B) + (C if with_c else 0)
         assert orc.max_rel_err(D, ref) < 16 * eps, (a_col, b_col, c_col, d_col, with_c)
+        # the same MMA through tcec::detail's foreach(_ij)_wrapper + compute_mem_offset,
+        # load_matrix_sync_wrapper / fill_fragment_wrapper, mma_sync_wrapper and
+        # store_matrix_sync_wrapper (tcec/detail/functions.hpp:10-348): same bits
+        dw = tc.primitive_mma(elem, shape, torch.from_numpy(_img(A, a_col)).to(dev),
+                              torch.from_numpy(_img(B, b_col)).to(dev),
+                              None if C is None else torch.from_numpy(_img(C, c_col)).to(dev),
+                              a_col, b_col, c_col, d_col, wrappers=True).cpu().numpy()
+        assert np.array_equal(d.view(np.uint32), dw.view(np.uint32)), (a_col, b_col, c_col, d_col, with_c)
 
 
 @pytest.mark.parametrize("shape", [0, 2])

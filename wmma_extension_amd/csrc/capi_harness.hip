@@ -296,12 +296,14 @@ int wmmae_tcec_mma_complex(const int type, const int ec, float *const d,
   });
 }
 
-int wmmae_primitive_mma(const int elem, const int shape, float *const d,
+int wmmae_primitive_mma(const int elem, const int shape_arg, float *const d,
                         const float *const a, const float *const b,
                         const float *const c, const int a_col, const int b_col,
                         const int c_col, const int d_col, void *const stream) {
   if (!d || !a || !b)
     return WMMAE_STATUS_NULL_POINTER;
+  const bool wrappers = shape_arg >= 8; // + 8: tcec::detail function objects
+  const int shape = wrappers ? shape_arg - 8 : shape_arg;
   if (elem < 0 || elem > 2 || shape < 0 || shape > 3)
     return WMMAE_STATUS_INVALID_VALUE;
   if (elem == 2 && shape != 0 && shape != 2)
@@ -320,18 +322,20 @@ int wmmae_primitive_mma(const int elem, const int shape, float *const d,
         using T = typename decltype(tt)::type;
         switch (shape) {
         case 0:
-          return go(wmmae_harness::primitive_mma_kernel<T, 16, 16, 16, AL, BL>);
+          return wrappers ? go(wmmae_harness::wrapper_mma_kernel<T, 16, 16, 16, AL, BL>)
+                          : go(wmmae_harness::primitive_mma_kernel<T, 16, 16, 16, AL, BL>);
         case 1:
           if constexpr (!std::is_same<T, float>::value)
-            return go(
-                wmmae_harness::primitive_mma_kernel<T, 16, 16, 32, AL, BL>);
+            return wrappers ? go(wmmae_harness::wrapper_mma_kernel<T, 16, 16, 32, AL, BL>)
+                          : go(wmmae_harness::primitive_mma_kernel<T, 16, 16, 32, AL, BL>);
           break;
         case 2:
-          return go(wmmae_harness::primitive_mma_kernel<T, 32, 32, 8, AL, BL>);
+          return wrappers ? go(wmmae_harness::wrapper_mma_kernel<T, 32, 32, 8, AL, BL>)
+                          : go(wmmae_harness::primitive_mma_kernel<T, 32, 32, 8, AL, BL>);
         default:
           if constexpr (!std::is_same<T, float>::value)
-            return go(
-                wmmae_harness::primitive_mma_kernel<T, 32, 32, 16, AL, BL>);
+            return wrappers ? go(wmmae_harness::wrapper_mma_kernel<T, 32, 32, 16, AL, BL>)
+                          : go(wmmae_harness::primitive_mma_kernel<T, 32, 32, 16, AL, BL>);
           break;
         }
         return static_cast<int>(WMMAE_STATUS_NOT_SUPPORTED);

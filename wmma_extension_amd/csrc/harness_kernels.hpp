@@ -25,6 +25,7 @@
 //   tcec_mma_complex_kernel : one-wave complex D = A*B (+C) through fragment_complex
 //                             (reference: test/tcec/mma_complex.cu:22-101)
 //   primitive_mma_kernel    : mma::load_matrix_sync -> mma_sync -> mma::store_matrix_sync
+//   wrapper_mma_kernel      : the same through the tcec::detail function objects
 //                             (reference: test/primitive/mma.cu:11-45)
 //   foreach_ec_kernel       : A, dA, B, dB built through foreach, three MMAs
 //                             (reference: test/primitive/foreach.cu:24-80)
@@ -490,6 +491,55 @@ __global__ void __launch_bounds__(64)
   mma::mma_sync(fd, fa, fb, fc);
   mma::store_matrix_sync(d, fd, d_col ? M : N,
                          d_col ? w::mem_col_major : w::mem_row_major);
+}
+
+// --------------------------------------------------------------------------
+// The same MMA through the policy-dispatched function objects of
+// tcec::detail (foreach_ij_wrapper and foreach_wrapper with
+// compute_mem_offset for the operands, load_matrix_sync_wrapper or
+// fill_fragment_wrapper for C, mma_sync_wrapper, store_matrix_sync_wrapper).
+// float operands take the fp32 policy, whose sub-fragments hold floats.
+// --------------------------------------------------------------------------
+template <class T, int M, int N, int K, class AL, class BL>
+__global__ void __launch_bounds__(64)
+    wrapper_mma_kernel(float *const d, const float *const a,
+                       const float *const b, const float *const c,
+                       const int c_col, const int d_col) {
+  namespace td = tcec::detail;
+  using Op = typename std::conditional<std::is_same<T, float>::value,
+                                       tcec::op_simt, tcec::op_mfma>::type;
+  using P = tcec::Policy<Op, tcec::with_ec, M, N, K>;
+  td::policy_fragment_t<w::matrix_a, T, AL, P> fa;
+  td::policy_fragment_t<w::matrix_b, T, BL, P> fb;
+  td::policy_fragment_t<w::accumulator, float, void, P> fc, fd;
+  using ET = typename decltype(fa)::element_type;
+  td::fill_zero_wrapper<w::matrix_a, T, AL, P>{}(fa);
+  td::fill_zero_wrapper<w::matrix_b, T, BL, P>{}(fb);
+  const unsigned lda = std::is_same<AL, w::col_major>::value ? M : K;
+  const unsigned ldb = std::is_same<BL, w::col_major>::value ? K : N;
+  td::foreach_ij_wrapper<w::matrix_a, T, AL, P>{}(
+      [&](const unsigned *list, const unsigned count, const unsigned i,
+          const unsigned j) {
+        const unsigned off = td::compute_mem_offset<M, K, AL>{}(i, j, lda, 0u, 0u);
+        for (unsigned f = 0; f < count; f++)
+          fa.x[list[f]] = w::detail::common::cast<ET>(a[off]);
+      });
+  td::foreach_wrapper<w::matrix_b, T, BL, P>{}(
+      [&](const unsigned *list, const unsigned count,
+          const unsigned mem_index) {
+        const unsigned off =
+            td::compute_mem_offset<K, N, BL>{}(mem_index, ldb, 0u, 0u);
+        for (unsigned f = 0; f < count; f++)
+          fb.x[list[f]] = w::detail::common::cast<ET>(b[off]);
+      });
+  if (c != nullptr)
+    td::load_matrix_sync_wrapper<w::accumulator, float, void, P>{}(
+        fc, c, c_col ? M : N, c_col ? w::mem_col_major : w::mem_row_major);
+  else
+    td::fill_fragment_wrapper<w::accumulator, float, void, P, float>{}(fc, 0.f);
+  td::mma_sync_wrapper<T, AL, BL, float, P>{}(fd, fa, fb, fc);
+  td::store_matrix_sync_wrapper<float, P>{}(
+      d, fd, d_col ? M : N, d_col ? w::mem_col_major : w::mem_row_major);
 }
 
 // --------------------------------------------------------------------------

@@ -414,11 +414,14 @@ def clock_samples(nsamples, period_ticks, stream=None, device="cuda:0"):
 PRIMITIVE_SHAPES = {0: (16, 16, 16), 1: (16, 16, 32), 2: (32, 32, 8), 3: (32, 32, 16)}
 
 
-def primitive_mma(elem, shape, a, b, c, a_col, b_col, c_col, d_col, d=None):
+def primitive_mma(elem, shape, a, b, c, a_col, b_col, c_col, d_col, d=None, wrappers=False):
     """a, b, c: flat fp32 CUDA images of the operands in the given layouts; returns flat d
-    (written into `d` when the caller passes one, e.g. a view at an odd offset)."""
+    (written into `d` when the caller passes one, e.g. a view at an odd offset).
+    wrappers=True runs the same MMA through the tcec::detail function objects."""
     _need_cuda(a, b, c, d)
     m, n, _ = PRIMITIVE_SHAPES[shape]
+    if wrappers:
+        shape += 8
     if d is None:
         d = torch.full((m * n,), float("nan"), dtype=torch.float32, device=a.device)
     assert d.numel() == m * n and d.is_contiguous()
