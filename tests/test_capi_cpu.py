@@ -212,7 +212,7 @@ def test_slice_counts_the_estimates_choose():
         assert out.value % (m * n * batch * 4) == 0
         return out.value // (m * n * batch * 4)
     assert planes(0, 1024, 1024, 262144) == 8
-    assert planes(2, 1024, 1024, 262144) == 4
+    assert planes(2, 1024, 1024, 262144) == 8    # three terms: 256x128 tiles too, one slice per XCD
     assert planes(0, 1024, 1024, 4096) == 4
     assert planes(0, 1280, 1280, 4096) == 5      # 250 tiles of 256x128: one round
     assert planes(0, 512, 512, 1024) == 5

@@ -182,7 +182,7 @@ namespace fit {
 //    0.7 % of the best measured one on average (1.9 % on 120 random products
 //    with m, n = 64 .. 2900, k = 400 .. 32000, 1 .. 100 entries, 1 .. 32
 //    slices forced).
-constexpr double kStage256x128[3] = {0.8e-6, 1.0e-6, 1.0e-6}; // (no 3-term 256x128 kernel)
+constexpr double kStage256x128[3] = {0.8e-6, 1.0e-6, 1.82e-6};
 constexpr double kStage128x128[3] = {0.45e-6, 0.6e-6, 0.99e-6};
 constexpr double kStage64x64 = 0.25e-6;
 constexpr double kTileOverhead = 7e-6;    // pipeline fill + epilogue of a tile
@@ -193,8 +193,21 @@ constexpr double kSplitMustBeat = 0.95;   // a split has to win by 5 %
 //    tiles forced on 124 products, 1024^2 .. 8192^2, k = 256 .. 4096, some
 //    batched: the choice is within 0.4 % of the faster tile on average.
 constexpr double kUnits256x128 = 2.0;
-constexpr double kUnits128x128 = 1.2;     // one and two terms (1.0 with three)
+constexpr double kUnits128x128 = 1.2;     // one and two terms
+//    Three terms (sweep: both tiles forced on 36 products, 1024^2 .. 8192^2,
+//    k = 1024 .. 5000, some batched or rectangular: a round of 256x128 tiles
+//    costs 1.8 rounds of 128x128 tiles, so the large tile wins when it halves
+//    the rounds, 8 to 14 %, and loses otherwise, 3 % at 7 -> 4 rounds, 17 to
+//    20 % at 3 -> 2).
+constexpr double kUnits256x128Terms3 = 1.8;
+constexpr double kUnits128x128Terms3 = 1.0;
 constexpr double kUnits64x64 = 0.4;
+constexpr double units256x128(const int terms) {
+  return terms == 3 ? kUnits256x128Terms3 : kUnits256x128;
+}
+constexpr double units128x128(const int terms) {
+  return terms == 3 ? kUnits128x128Terms3 : kUnits128x128;
+}
 // -- K slices for a partly empty last round: slices, pipeline refills, fold.
 //    Sweep: 126 products, 2304^2 .. 8192^2, k = 2048 .. 8192, two policies.
 constexpr double kTailOverhead = 0.2;
@@ -255,7 +268,7 @@ constexpr int kKernelXcds = 8; // the constant XCDS of the kernels' item lists
 // round of 256x128 tiles instead had cost 2 %, up to 13 % at 2560^2 .. 2816^2.)
 inline bool big_tile_candidate(const int terms, const long long mid,
                                const int kt) {
-  return terms <= 2 && mid > device_cus() && !(terms == 1 && kt <= 32);
+  return mid > device_cus() && !(terms == 1 && kt <= 32);
 }
 inline double split_time(const int terms, const int m, const int n,
                          const int batch, const int kt, const int slices) {
@@ -268,7 +281,7 @@ inline double split_time(const int terms, const int m, const int n,
   const double r_big = static_cast<double>(ceil_div(big, cus));
   const double r_mid = static_cast<double>(ceil_div(mid, cus));
   if (big_tile_candidate(terms, mid, stages) &&
-      r_big * fit::kUnits256x128 <= r_mid * fit::kUnits128x128) {
+      r_big * fit::units256x128(terms) <= r_mid * fit::units128x128(terms)) {
     stage_time = fit::kStage256x128[terms - 1];
     rounds = r_big;
   } else if (mid >= cus || (m > 64 && n > 64)) {
@@ -484,18 +497,18 @@ template <class MT, int TERMS, bool RN> int gemm_by_size(const GemmArgs &g) {
       ceil_div(g.m, 128) * ceil_div(g.n, 128) * g.batch * z;
   // (not with the separate fp32 adds of RN: their temporaries do not fit the
   // register file next to the large tile's accumulators)
-  if constexpr (TERMS <= 2 && !RN) {
+  if constexpr (!RN) {
     const int KT = packed_k_tiles(g.k);
     if (big_tile_candidate(TERMS, mid, static_cast<int>(ceil_div(KT, z)))) {
       // time in units of one 128x128 tile: rounds * tile cost
       const bool tail_ok = g.batch == 1 && z == 1 && g.c_ptrs == nullptr &&
                            g.tail_ws != nullptr;
       const double t_big =
-          rounds_cost(big, cus, KT, tail_ok) * fit::kUnits256x128;
+          rounds_cost(big, cus, KT, tail_ok) * fit::units256x128(TERMS);
       // (a 128x128 tile measured at 1.2 to 1.25 times half a 256x128 tile in
       // runs of two to eight rounds, 1.05 in long ones)
       const double t_mid =
-          rounds_cost(mid, cus, KT, tail_ok) * fit::kUnits128x128;
+          rounds_cost(mid, cus, KT, tail_ok) * fit::units128x128(TERMS);
       if (t_big <= t_mid)
         return launch_gemm<MT, TERMS, 256, 128, 2, 2, RN>(g);
     }
@@ -654,16 +667,17 @@ inline bool use_fused(const int m, const int n, const int k, const int batch,
                           (c_bytes + 4.0 * ab) / f.bytes_per_s);
 
   // packed path: rounds in units of one 128x128 tile as gemm_by_size counts
-  // them (a 256x128 tile 2.0, a 128x128 tile 1.2 for one and two terms, a
-  // 64x64 tile 0.4)
+  // them (a 256x128 tile 2.0 and a 128x128 tile 1.2 for one and two terms,
+  // 1.8 and 1.0 for three, a 64x64 tile 0.4)
   double units;
   const double r128 = static_cast<double>(ceil_div(tiles128, cus));
   if (big_tile_candidate(terms, tiles128, static_cast<int>(kt)) &&
-      fit::kUnits256x128 * static_cast<double>(ceil_div(tiles256, cus)) <=
-          fit::kUnits128x128 * r128)
-    units = fit::kUnits256x128 * static_cast<double>(ceil_div(tiles256, cus));
+      fit::units256x128(terms) * static_cast<double>(ceil_div(tiles256, cus)) <=
+          fit::units128x128(terms) * r128)
+    units = fit::units256x128(terms) *
+            static_cast<double>(ceil_div(tiles256, cus));
   else if (tiles128 >= cus || (m > 64 && n > 64))
-    units = r128 * (terms <= 2 ? fit::kUnits128x128 : 1.0);
+    units = r128 * fit::units128x128(terms);
   else
     units = fit::kUnits64x64 * static_cast<double>(ceil_div(tiles64, cus));
   const double t_packed =

@@ -34,6 +34,7 @@ typedef float f32x4 __attribute__((ext_vector_type(4)));
 constexpr int kChunkRows = 16; // rows per packed chunk (MFMA M / N)
 constexpr int kChunkK = 32;    // k per packed chunk (MFMA K) = one pipeline stage
 
+template <int I> using ic = std::integral_constant<int, I>;
 // Compile-time loop: f(std::integral_constant<int, I>) for I in [B, E).
 template <int B, int E, class F>
 __device__ __forceinline__ void static_for(F &&f) {
@@ -302,7 +303,13 @@ __global__ void __launch_bounds__(256)
 //             registers, stage s+1 is being read from LDS into the second
 //             fragment set and stages s+2 .. s+NSTAGE are in flight from
 //             HBM/L2, which is what covers memory latency with a single
-//             workgroup per compute unit.
+//             workgroup per compute unit.  The 256x128 tile with three terms
+//             (72 KiB a stage, a ring of two; 144 registers of fragments a
+//             stage) keeps one copy of the A fragments and refills a tile
+//             row's registers for the next stage right after that row's
+//             MFMAs have been issued (GemmConfig::RECYCLE_A): a quarter fewer
+//             L2 -> LDS bytes and LDS reads per MFMA than the 128x128 tile,
+//             16384^3 32.5 -> 29.5 ms.
 //   RN_MAIN : accumulate the leading product with fp32 adds outside the
 //             matrix core (the reference's mma_rn_sync, tcec/tcec.hpp:673-694)
 //             instead of chaining it through the MFMA accumulator.  The gfx950
@@ -333,6 +340,11 @@ struct GemmConfig {
   static constexpr int NCH = CH_A + CH_B;
   static constexpr int CPW = NCH / NW; // chunks each wave requests per stage
   static constexpr int LDS_BYTES = NSTAGE * NCH * 1024;
+  // Two sets of operand fragments (the stage being multiplied and the next
+  // one) must fit the 256 vector registers beside the accumulators; when they
+  // do not, the A fragments of all tile rows but the last exist once and are
+  // refilled for the next stage as soon as their tile row has been issued.
+  static constexpr bool RECYCLE_A = 2 * TERMS * (MT_ + NT_) * 4 > 256;
   static_assert(NCH % NW == 0, "chunks must divide evenly over the waves");
   static_assert(WM % 16 == 0 && WN % 16 == 0, "wave tile must be MFMA tiles");
   static_assert(NSTAGE >= 2 && NSTAGE <= 4, "ring depth");
@@ -476,11 +488,12 @@ __global__ void __launch_bounds__(WGM *WGN * 64)
   // per row block serves them through the instruction's immediate offset.
   // Which row blocks: w, w + NW, w + 2 NW, ... with one or two terms (the
   // waves then ask for neighbouring row blocks at the same time; batched
-  // 1024x1024x256 measured 276 against 258 effective TFLOPS), w*RPW ..
-  // w*RPW + RPW-1 with three terms (16384^3: 240 against 219).
+  // 1024x1024x256 measured 276 against 258 effective TFLOPS) and for the
+  // three-term 256x128 tile (16384^3: 29.5 against 30.0 ms), w*RPW ..
+  // w*RPW + RPW-1 for the three-term 128x128 tile (16384^3: 240 against 219).
   constexpr unsigned STAGE_BYTES = CH_PER_RB * 1024u; // one stage of a row block
   constexpr int RPW = CPW / CH_PER_RB;                // row blocks per wave
-  constexpr bool STRIDED_RB = TERMS <= 2;
+  constexpr bool STRIDED_RB = TERMS <= 2 || Cfg::RECYCLE_A;
   constexpr int RB_STEP = STRIDED_RB ? Cfg::NW : 1; // between a wave's row blocks
   static_assert(CPW % CH_PER_RB == 0, "a wave requests whole row blocks");
   unsigned long long gsrc[RPW];
@@ -589,14 +602,28 @@ __global__ void __launch_bounds__(WGM *WGN * 64)
       return __builtin_amdgcn_mfma_f32_16x16x32_bf16(x, y, z, 0, 0, 0);
   };
 
-  // Operand fragments of one stage: TERMS chunks per 16-row block.
+  // Operand fragments of one stage: TERMS chunks per 16-row block.  With
+  // RECYCLE_A a Frags holds the B fragments and the A fragments of the last
+  // tile row only; the other tile rows' A fragments live once, in a_once.
+  constexpr bool RECYCLE = Cfg::RECYCLE_A;
   struct Frags {
-    ab_vec a[TERMS][MT_];
+    ab_vec a[TERMS][RECYCLE ? 1 : MT_];
     ab_vec b[TERMS][NT_];
+  };
+  ab_vec a_once[TERMS][RECYCLE ? MT_ - 1 : 1];
+  auto a_frag = [&](const Frags &f, auto T_, auto I_) -> const ab_vec & {
+    constexpr int t = decltype(T_)::value, i = decltype(I_)::value;
+    if constexpr (!RECYCLE)
+      return f.a[t][i];
+    else if constexpr (i < MT_ - 1)
+      return a_once[t][i];
+    else
+      return f.a[t][0];
   };
   constexpr int NFRAG = TERMS * (MT_ + NT_);
   // fragment IDX of a stage (compile-time index, so that every fragment is a
-  // fixed register): B fragments first, then A
+  // fixed register): B fragments first, then A (RECYCLE: A's last tile row
+  // first, then rows 0 .. MT_-2)
   auto read_frag = [&](Frags &f, const int r_base, auto IDX) {
     constexpr int r = decltype(IDX)::value;
     const u32x4 *const stage =
@@ -606,9 +633,18 @@ __global__ void __launch_bounds__(WGM *WGN * 64)
       const u32x4 *const sb = stage + (CH_A + wn * NT_ * CH_PER_RB) * 64;
       f.b[t][j] = __builtin_bit_cast(ab_vec, sb[(j * CH_PER_RB + t) * 64]);
     } else {
-      constexpr int i = (r - TERMS * NT_) / TERMS, t = (r - TERMS * NT_) % TERMS;
+      constexpr int ra = r - TERMS * NT_, t = ra % TERMS;
+      constexpr int i = !RECYCLE ? ra / TERMS
+                                 : (ra < TERMS ? MT_ - 1 : ra / TERMS - 1);
       const u32x4 *const sa = stage + (wm * MT_ * CH_PER_RB) * 64;
-      f.a[t][i] = __builtin_bit_cast(ab_vec, sa[(i * CH_PER_RB + t) * 64]);
+      const ab_vec v =
+          __builtin_bit_cast(ab_vec, sa[(i * CH_PER_RB + t) * 64]);
+      if constexpr (!RECYCLE)
+        f.a[t][i] = v;
+      else if constexpr (i < MT_ - 1)
+        a_once[t][i] = v;
+      else
+        f.a[t][0] = v;
     }
   };
 
@@ -620,9 +656,28 @@ __global__ void __launch_bounds__(WGM *WGN * 64)
   // LDS read r of the next stage goes out after MFMA number (r+1)*SPAN/NFRAG:
   // the reads are spread over the first three quarters of the step (the LGKM
   // counter only tracks 15 outstanding operations)
+  // The requests of a step are spread over the whole step; with a ring of two
+  // stages they must have landed when the next step begins and go out in the
+  // step's first half (16384^3, three terms, 256x128 tile, requests within the
+  // first 1/8, 1/4, 1/3, 1/2, 2/3, 3/4, 5/6 of the step and over all of it:
+  // 33.1, 31.4, 30.3, 29.4, 29.3, 30.6, 31.3, 32.8 ms).
+    constexpr int REQ_SPAN = NSTAGE == 2 ? (NMFMA / 2 > 0 ? NMFMA / 2 : 1) : NMFMA;
   // MFMA after which the last request of a step goes out
-  constexpr int N_ADVANCE = (NMFMA * (CPW - 1)) / CPW;
+  constexpr int N_ADVANCE = (REQ_SPAN * (CPW - 1)) / CPW;
   constexpr int SPAN = (NMFMA * 3) / 4 > 0 ? (NMFMA * 3) / 4 : 1;
+  // RECYCLE: MFMA after which read r of the next stage goes out.  The B
+  // fragments and A's last tile row (separate registers) during the first tile
+  // row; the A fragments of tile row i, which overwrite the current stage's,
+  // right after the last MFMA of that row has been issued (the matrix core
+  // has taken its operands by then; the LDS data arrives much later).
+  constexpr int ROW_MFMA = NT_ * NPROD;
+  constexpr int FIRST_READS = TERMS * (NT_ + 1);
+  constexpr auto recycle_slot = [](const int r) constexpr {
+    return r < FIRST_READS
+               ? (r * ROW_MFMA) / FIRST_READS
+               : ((r - FIRST_READS) / TERMS + 1) * ROW_MFMA +
+                     2 * ((r - FIRST_READS) % TERMS);
+  };
 
   // One pipeline step: multiply the fragments of stage st (already in
   // registers) while the fragments of stage st+1 are read from LDS and stage
@@ -681,20 +736,22 @@ __global__ void __launch_bounds__(WGM *WGN * 64)
                                                                       : 0);
       constexpr bool is_main = p == NPROD - 1;
       if constexpr (is_main && RN_MAIN) {
-        acc_main[i][j] +=
-            mfma(cur.a[0][i], cur.b[0][j], f32x4{0.f, 0.f, 0.f, 0.f});
+        acc_main[i][j] += mfma(a_frag(cur, ic<0>{}, ic<i>{}), cur.b[0][j],
+                               f32x4{0.f, 0.f, 0.f, 0.f});
       } else if constexpr (USE_ASM) {
-        mfma_acc(is_main ? acc_main[i][j] : acc_err[i][j], cur.a[ta][i],
-                 cur.b[tb][j]);
+        mfma_acc(is_main ? acc_main[i][j] : acc_err[i][j],
+                 a_frag(cur, ic<ta>{}, ic<i>{}), cur.b[tb][j]);
       } else if constexpr (is_main) {
-        acc_main[i][j] = mfma(cur.a[ta][i], cur.b[tb][j], acc_main[i][j]);
+        acc_main[i][j] = mfma(a_frag(cur, ic<ta>{}, ic<i>{}), cur.b[tb][j],
+                              acc_main[i][j]);
       } else {
-        acc_err[i][j] = mfma(cur.a[ta][i], cur.b[tb][j], acc_err[i][j]);
+        acc_err[i][j] = mfma(a_frag(cur, ic<ta>{}, ic<i>{}), cur.b[tb][j],
+                             acc_err[i][j]);
       }
       // global->LDS requests due after this MFMA
-      constexpr int qlo = (n * CPW + NMFMA - 1) / NMFMA;
-      constexpr int qhi = ((n + 1) * CPW + NMFMA - 1) / NMFMA;
-      static_for<qlo, (qhi < CPW ? qhi : CPW)>([&](auto Q) {
+      constexpr int qlo = (n * CPW + REQ_SPAN - 1) / REQ_SPAN;
+      constexpr int qhi = ((n + 1) * CPW + REQ_SPAN - 1) / REQ_SPAN;
+      static_for<(qlo < CPW ? qlo : CPW), (qhi < CPW ? qhi : CPW)>([&](auto Q) {
         issue_chunk(w_base, Q);
         __builtin_amdgcn_sched_barrier(0);
       });
@@ -705,12 +762,22 @@ __global__ void __launch_bounds__(WGM *WGN * 64)
         __builtin_amdgcn_sched_barrier(0);
       }
       // LDS reads due after this MFMA
-      constexpr int lo = n == 0 ? 0 : reads_due(n, SPAN, NFRAG);
-      constexpr int hi = n + 1 == NMFMA ? NFRAG : reads_due(n + 1, SPAN, NFRAG);
-      static_for<lo, hi>([&](auto R_) {
-        read_frag(nxt, r_base, R_);
-        __builtin_amdgcn_sched_barrier(0);
-      });
+      if constexpr (RECYCLE) {
+        static_for<0, NFRAG>([&](auto R_) {
+          if constexpr (recycle_slot(decltype(R_)::value) == n) {
+            read_frag(nxt, r_base, R_);
+            __builtin_amdgcn_sched_barrier(0);
+          }
+        });
+      } else {
+        constexpr int lo = n == 0 ? 0 : reads_due(n, SPAN, NFRAG);
+        constexpr int hi =
+            n + 1 == NMFMA ? NFRAG : reads_due(n + 1, SPAN, NFRAG);
+        static_for<lo, hi>([&](auto R_) {
+          read_frag(nxt, r_base, R_);
+          __builtin_amdgcn_sched_barrier(0);
+        });
+      }
     });
   };
 
