@@ -63,11 +63,14 @@ def test_xcd_owned_batch_entries_equal_single_entry_calls(tc, orc, dev, policy, 
 
 
 @pytest.mark.parametrize("policy", [0, 1, 2, 3, 4])
-@pytest.mark.parametrize("shape", [(4096, 4096, 96, 1), (2048, 3000, 40, 3), (4096, 2048, 1024, 2)])
+@pytest.mark.parametrize("shape", [(4096, 4096, 96, 1), (2048, 3000, 40, 3), (4096, 2048, 1024, 2),
+                                   (4096, 4096, 32, 1), (4096, 4096, 64, 1), (4096, 4096, 160, 1)])
 def test_persistent_shared_list_equals_column_blocks(tc, orc, dev, policy, shape):
     """Few entries, short K loops, more tiles than resident workgroups: persistent
     workgroups on one list.  The same product from column blocks of 512 columns of B
-    (few enough tiles for one workgroup each) has to agree bit for bit."""
+    (few enough tiles for one workgroup each) has to agree bit for bit.  The whole products
+    take the 256x128 tile (with three terms: one copy of the A fragments and a ring of two
+    stages), the column blocks the 128x128 tile; 1, 2, 3, 5 and 32 stages per item."""
     m, n, k, batch = shape
     A = _uniform((batch, m, k), 400 + k, dev)
     B = _uniform((batch, n, k), 500 + k, dev)
