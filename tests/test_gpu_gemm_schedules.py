@@ -94,22 +94,24 @@ def test_persistent_shared_list_equals_column_blocks(tc, orc, dev, policy, shape
         _fp64_check(orc, A[0], B[0], C[0], policy)
 
 
-def test_one_workgroup_per_item_for_long_k(tc, orc, dev):
+@pytest.mark.parametrize("policy,slabs", [(0, 2), (2, 2), (2, 4)])
+def test_one_workgroup_per_item_for_long_k(tc, orc, dev, policy, slabs):
     """Many tiles with 64 or more stages each and a single entry: one workgroup per item.
-    Rows of A in two halves give the same bits."""
+    Rows of A in two halves (the 256x128 tile again) or, with three terms, in four slabs
+    of 1024 rows (256 tiles of 128x128: the smaller tile) give the same bits."""
     m, n, k = 4096, 4096, 2048 + 32
     A = _uniform((1, m, k), 7, dev)
     B = _uniform((1, n, k), 8, dev)
-    pa, _ = _pack(tc, 0, A, dev)
-    pb, _ = _pack(tc, 0, B, dev)
+    pa, _ = _pack(tc, policy, A, dev)
+    pb, _ = _pack(tc, policy, B, dev)
     C = torch.zeros((n, m), dtype=torch.float32, device=dev)
-    tc.gemm_packed(0, m, n, k, 1.0, pa, pb, 0.0, C, m)
+    tc.gemm_packed(policy, m, n, k, 1.0, pa, pb, 0.0, C, m)
     ref = torch.zeros((n, m), dtype=torch.float32, device=dev)
-    half = m // 2
-    rb_bytes = ((k + 31) // 32) * 2 * 1024
-    for r0 in (0, half):
-        # rows r0 .. r0+half of C: the column-major slab starts at element r0 of every column
-        tc.gemm_packed(0, half, n, k, 1.0, pa[(r0 // 16) * rb_bytes:], pb, 0.0,
+    part = m // slabs
+    rb_bytes = ((k + 31) // 32) * TERMS[policy] * 1024
+    for r0 in range(0, m, part):
+        # rows r0 .. r0+part of C: the column-major slab starts at element r0 of every column
+        tc.gemm_packed(policy, part, n, k, 1.0, pa[(r0 // 16) * rb_bytes:], pb, 0.0,
                        ref.view(-1)[r0:], m)
     torch.cuda.synchronize()
     assert torch.equal(C, ref)
