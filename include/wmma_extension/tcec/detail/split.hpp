@@ -86,6 +86,37 @@ template <> struct split_traits<float> {
 //   bf16 : v_cvt_pk_bf16_f32 pairs, residuals by fp32 subtraction
 typedef float f32x2_t __attribute__((ext_vector_type(2)));
 typedef float f32x4_t __attribute__((ext_vector_type(4)));
+// split2: two values -> pairs of terms (h0 leading, h1 residual, h2 second
+// residual; the pairs beyond the split's number of terms are left alone)
+template <class T, class S = typename split_traits<T>::storage,
+          class S2 = S __attribute__((ext_vector_type(2)))>
+WMMAE_D void split2(const f32x2_t vv, S2 &h0, S2 &h1, S2 &h2) {
+  using traits = split_traits<T>;
+  static_assert(!std::is_same<S, float>::value, "16-bit terms only");
+  h0 = __builtin_convertvector(vv, S2);
+  if constexpr (traits::num_terms >= 2) {
+    f32x2_t r = {0.f, 0.f};
+    if constexpr (std::is_same<S, _Float16>::value) {
+      static_assert(traits::num_terms == 2, "two-term fp16 split");
+      const float m0 = vv[0] * traits::scale, m1 = vv[1] * traits::scale;
+      const float neg_scale = -traits::scale;
+      asm("v_fma_mixlo_f16 %0, %1, %2, %3 op_sel:[0,0,0] op_sel_hi:[1,0,0]"
+          : "=v"(h1)
+          : "v"(h0), "s"(neg_scale), "v"(m0));
+      asm("v_fma_mixhi_f16 %0, %1, %2, %3 op_sel:[1,0,0] op_sel_hi:[1,0,0]"
+          : "+v"(h1)
+          : "v"(h0), "s"(neg_scale), "v"(m1));
+    } else {
+      r = vv - __builtin_convertvector(h0, f32x2_t);
+      if constexpr (traits::scale != 1.f)
+        r *= traits::scale;
+      h1 = __builtin_convertvector(r, S2);
+    }
+    if constexpr (traits::num_terms >= 3)
+      h2 = __builtin_convertvector(r - __builtin_convertvector(h1, f32x2_t),
+                                   S2);
+  }
+}
 template <class T, class S = typename split_traits<T>::storage>
 WMMAE_D void split4(const f32x4_t v, S *const t0, S *const t1, S *const t2) {
   using traits = split_traits<T>;
@@ -97,37 +128,17 @@ WMMAE_D void split4(const f32x4_t v, S *const t0, S *const t1, S *const t2) {
     typedef S s2_t __attribute__((ext_vector_type(2)));
 #pragma unroll
     for (int e = 0; e < 4; e += 2) {
-      const f32x2_t vv = {v[e], v[e + 1]};
-      const s2_t h0 = __builtin_convertvector(vv, s2_t);
+      s2_t h0, h1, h2;
+      split2<T>(f32x2_t{v[e], v[e + 1]}, h0, h1, h2);
       t0[e] = h0[0];
       t0[e + 1] = h0[1];
       if constexpr (traits::num_terms >= 2) {
-        f32x2_t r = {0.f, 0.f};
-        s2_t h1;
-        if constexpr (std::is_same<S, _Float16>::value) {
-          static_assert(traits::num_terms == 2, "two-term fp16 split");
-          const float m0 = vv[0] * traits::scale, m1 = vv[1] * traits::scale;
-          const float neg_scale = -traits::scale;
-          asm("v_fma_mixlo_f16 %0, %1, %2, %3 op_sel:[0,0,0] op_sel_hi:[1,0,0]"
-              : "=v"(h1)
-              : "v"(h0), "s"(neg_scale), "v"(m0));
-          asm("v_fma_mixhi_f16 %0, %1, %2, %3 op_sel:[1,0,0] op_sel_hi:[1,0,0]"
-              : "+v"(h1)
-              : "v"(h0), "s"(neg_scale), "v"(m1));
-        } else {
-          r = vv - __builtin_convertvector(h0, f32x2_t);
-          if constexpr (traits::scale != 1.f)
-            r *= traits::scale;
-          h1 = __builtin_convertvector(r, s2_t);
-        }
         t1[e] = h1[0];
         t1[e + 1] = h1[1];
-        if constexpr (traits::num_terms >= 3) {
-          const s2_t h2 = __builtin_convertvector(
-              r - __builtin_convertvector(h1, f32x2_t), s2_t);
-          t2[e] = h2[0];
-          t2[e + 1] = h2[1];
-        }
+      }
+      if constexpr (traits::num_terms >= 3) {
+        t2[e] = h2[0];
+        t2[e + 1] = h2[1];
       }
     }
   }

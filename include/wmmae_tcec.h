@@ -66,6 +66,16 @@ typedef enum {
 #define WMMAE_FLAG_RN_MAIN 1 /* accumulate the leading product with fp32 adds
                                 outside the matrix core (the reference's
                                 mma_rn_sync, tcec/tcec.hpp:640-706) */
+/* wmmae_tcec_sgemm*: take this path instead of the one the time estimates
+ * choose (at most one of the three; WMMAE_STATUS_NOT_SUPPORTED when the
+ * arguments do not allow it).  No counterpart in the reference, whose harness
+ * fixes one kernel configuration at compile time. */
+#define WMMAE_FLAG_PATH_PACKED 2 /* split pass + GEMM on packed operands */
+#define WMMAE_FLAG_PATH_FUSED 4  /* the single kernel for small products */
+#define WMMAE_FLAG_PATH_DIRECT 8 /* the packed path's GEMM kernel splitting the
+                                    fp32 operands itself: needs op(A) and op(B)
+                                    with k contiguous ('T','N'), k % 32 == 0, a
+                                    policy of one or two terms, no RN_MAIN */
 
 /* Text for a wmmae_status value.  (No counterpart in the reference: its
  * harness aborts through WMMAE_CUDA_CHECK_ERROR, test/tcec/utils.hpp:11-20.) */
@@ -94,8 +104,12 @@ int wmmae_query(int what, long long *out);
  * 16 bytes at a time) are split inside the GEMM
  * kernel (as the reference's bgemm_kernel splits at fragment load,
  * batch_gemm.cu:196-386): they use no workspace, allocate nothing and ignore
- * the workspace arguments.  Both paths give the same bits as long as no K
- * slices are made (those add the partial sums' rounding). */
+ * the workspace arguments.  Batches of medium-sized matrices and K-heavy
+ * products with k contiguous in both operands run the packed path's GEMM
+ * kernel on the fp32 operands directly (it splits them on their way into LDS):
+ * no packed copy; the workspace then only holds K slices.  All paths give the
+ * same bits as long as no K slices are made (those add the partial sums'
+ * rounding). */
 int wmmae_tcec_sgemm_workspace_bytes(int m, int n, int k, int batch, int policy,
                                      size_t *bytes);
 
@@ -103,7 +117,10 @@ int wmmae_tcec_sgemm_workspace_bytes(int m, int n, int k, int batch, int policy,
  * reference, whose harness fixes one kernel configuration at compile time,
  * batch_gemm.cu:408-431, 659): *path = 0 the single kernel that splits the
  * operands on the fly (no workspace), 1 packed operands in the workspace,
- * 2 packed operands and K slices (when the workspace has room for them).
+ * 2 packed operands and K slices (when the workspace has room for them),
+ * 3 the packed path's GEMM kernel loading and splitting the fp32 operands
+ * itself (no packed operands), 4 the same with K slices.  3 and 4 assume
+ * k contiguous in both operands ('T','N'); other layouts take 1 and 2.
  * The answer assumes operands the single kernel can read 16 bytes at a time
  * (k the contiguous direction, k and the leading dimensions multiples of 4,
  * 16-byte aligned bases); other operands with k > 96 take path 1 where this

@@ -76,7 +76,12 @@ def test_sgemm_argument_validation(h):
     assert _sgemm(h, m=-1) == -1
     assert _sgemm(h, k=-5) == -1
     assert _sgemm(h, policy=7) == -1
-    assert _sgemm(h, flags=4) == -1
+    assert _sgemm(h, flags=16) == -1
+    assert _sgemm(h, flags=2 | 8) == -1         # at most one path flag
+    assert _sgemm(h, flags=8, k=48, lda=48, ldb=48) == -4    # direct path: k % 32 == 0
+    assert _sgemm(h, flags=8, ta=b"N") == -4               # ... and k contiguous
+    assert _sgemm(h, flags=8 | 1) == -4                      # ... and no RN_MAIN
+    assert _sgemm(h, flags=8, policy=2) == -4                # ... and at most two terms
     assert _sgemm(h, alpha=False) == -2
     assert _sgemm(h, beta=False) == -2
     assert _sgemm(h, A=0) == -2
@@ -178,15 +183,17 @@ def test_primitive_entries_reject_bad_arguments_on_the_host(h):
 
 
 def test_sgemm_path_query_on_the_baseline_workloads():
-    """wmmae_tcec_sgemm_path needs no GPU: the batched 256^3 products take the single kernel,
-    4096^3 and 16384^3 packed operands, the K-heavy product K slices; bad arguments are
-    turned down."""
+    """wmmae_tcec_sgemm_path needs no GPU: the batched 256^3 products and the K-heavy
+    product (with K slices) take the GEMM kernel that splits the fp32 operands itself,
+    4096^3 and 16384^3 packed operands, small batched products and the round-to-nearest
+    variant the single kernel; bad arguments are turned down."""
     import ctypes
     from wmma_extension_amd import _lib
     h = _lib.lib()
     out = ctypes.c_int(-1)
-    for args, want in (((256, 256, 256, 1024, 0, 0), 0), ((4096, 4096, 4096, 1, 0, 0), 1),
-                       ((16384, 16384, 16384, 1, 2, 0), 1), ((1024, 1024, 262144, 1, 0, 0), 2),
+    for args, want in (((256, 256, 256, 1024, 0, 0), 3), ((4096, 4096, 4096, 1, 0, 0), 1),
+                       ((16384, 16384, 16384, 1, 2, 0), 1), ((1024, 1024, 262144, 1, 0, 0), 4),
+                       ((1024, 1024, 262144, 1, 2, 0), 2), ((128, 128, 128, 1024, 0, 0), 0),
                        ((512, 512, 1024, 256, 0, 1), 0), ((512, 512, 1024, 256, 1, 1), 1)):
         assert h.wmmae_tcec_sgemm_path(*args, ctypes.byref(out)) == 0
         assert out.value == want, args

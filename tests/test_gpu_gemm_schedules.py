@@ -227,13 +227,15 @@ def test_random_blas_arguments_against_fp64(tc, dev):
     """100 seeded calls of the strided-batched entry point the way a BLAS user makes them:
     both transposes of both operands, padded leading dimensions, alpha and beta other than
     1 and 0, the round-to-nearest flag, with and without a caller's workspace, shapes drawn
-    so that all three paths (fused, packed, packed with K slices) are taken.  Each result is
+    so that all paths (fused, packed, packed with K slices, direct with and without K
+    slices) are taken.  Each result is
     compared with alpha * op(A) op(B) + beta * C in FP64, and the padding rows of C
     (ldc > m) must keep their bytes."""
     import random
     rnd = random.Random(77)
     bound = {0: 4e-6, 2: 4e-6, 1: 3e-3, 3: 3e-4, 4: 3e-2}
-    paths = [0, 0, 0]
+    paths = [0, 0, 0, 0, 0]
+    forced_direct = 0
     for case in range(100):
         policy = rnd.choice([0, 0, 2, 2, 1, 3, 4])
         batch = rnd.choice([1, 1, 1, 1, 2, 3, 9])
@@ -250,6 +252,9 @@ def test_random_blas_arguments_against_fp64(tc, dev):
             else:
                 k = max(1, k // 2)
         ta, tb = rnd.choice("NT"), rnd.choice("NT")
+        readable = rnd.random() < 0.35  # what the direct kernel can read: 'T','N', k % 32 == 0
+        if readable:
+            ta, tb, k = "T", "N", max(32, k // 32 * 32)
         # column-major storage: A holds ra x ca elements, ra contiguous, in columns of lda
         ra, ca = (m, k) if ta == "N" else (k, m)
         rb, cb = (k, n) if tb == "N" else (n, k)
@@ -260,6 +265,9 @@ def test_random_blas_arguments_against_fp64(tc, dev):
         alpha = rnd.choice([1.0, 1.0, -0.5, 2.25])
         beta = rnd.choice([0.0, 0.0, 1.0, -1.5])
         flags = rnd.choice([0, 0, 0, tc.FLAG_RN_MAIN]) if policy in (0, 2) else 0
+        if readable and policy != 2 and flags == 0 and rnd.random() < 0.7:
+            flags = tc.FLAG_PATH_DIRECT                       # else the estimates decide
+            forced_direct += 1
         a_cm = A[:, :, :ra].double()                          # [entry, column, row]
         b_cm = B[:, :, :rb].double()
         op_a = a_cm.transpose(1, 2) if ta == "N" else a_cm    # (entry, m, k)
@@ -278,5 +286,5 @@ def test_random_blas_arguments_against_fp64(tc, dev):
         tag = (case, policy, flags, batch, ta + tb, m, n, k, lda, ldb, ldc, alpha, beta, ws is not None)
         assert err < bound[policy], (tag, err)
         assert torch.equal(C[:, :, m:], C0[:, :, m:]), tag
-        paths[tc.sgemm_path(m, n, k, batch, policy, flags)] += 1
-    assert min(paths) >= 10, paths
+        paths[tc.sgemm_path(m, n, k, batch, policy, flags & tc.FLAG_RN_MAIN)] += 1
+    assert min(paths[:3]) >= 10 and forced_direct >= 10, (paths, forced_direct)

@@ -145,6 +145,10 @@ struct GemmArgs {
   float *tail_ws;
   size_t tail_ws_bytes;
   hipStream_t stream;
+  // fp32 operands for the kernel variant that splits them itself (a and b are
+  // null then)
+  bool is_direct = false;
+  wmmae_gemm::DirectSource direct = {};
 };
 
 // Compute units of the current device, looked up once per device.
@@ -226,6 +230,17 @@ constexpr PathRates kFused[3] = {{5.0e-6, 0.76e-6, 3.0e-6, 5.0e12, 0.},
 constexpr PathRates kPacked[3] = {{8.9e-6, 0.31e-6, 2.0e-6, 5.0e12, 6.6e12},
                                   {6.5e-6, 0.50e-6, 3.8e-6, 3.6e12, 5.6e12},
                                   {8.8e-6, 0.99e-6, 3.4e-6, 3.4e12, 5.9e12}};
+// -- the packed path's GEMM kernel reading and splitting the fp32 operands
+//    itself (256x128 tiles only; rows: one, two terms).  Sweep: 45 products
+//    run on this path and on the estimated one of the other two (the
+//    reference harness's grid m = n = 512, 1024, k = 128 .. 16384, 256
+//    entries; single and batched products of other shapes, four policies): a
+//    k stage of a 256x128 tile takes 0.8 / 1.56 us (packed operands: 0.5 /
+//    1.0 us), a tile 6 us on top.
+constexpr PathRates kDirect[2] = {{6.0e-6, 0.40e-6, 3.0e-6, 5.0e12, 0.},
+                                  {6.0e-6, 0.78e-6, 3.0e-6, 5.0e12, 0.}};
+// with K slices: the GEMM's time against the same kernel on packed operands
+constexpr double kDirectSliceRatio[2] = {1.5, 1.56};
 // the single kernel's 64x64 tile against its 128x128 tile (1024^3: 41 -> 27 us)
 constexpr double kFusedSmallTileTime = 0.65; // whole tile, latency-bound sizes
 constexpr double kFusedSmallStage = 0.33, kFusedSmallTile = 0.5;
@@ -360,12 +375,14 @@ constexpr int ring_depth(const int bm, const int bn, const int terms) {
   return fit > 4 ? 4 : fit;
 }
 
-template <class MT, int TERMS, int BM, int BN, int WGM, int WGN, bool RN>
+template <class MT, int TERMS, int BM, int BN, int WGM, int WGN, bool RN,
+          bool DIRECT = false>
 int launch_gemm(const GemmArgs &g) {
-  constexpr int NSTAGE = ring_depth(BM, BN, TERMS);
-  using Cfg = wmmae_gemm::GemmConfig<MT, TERMS, BM, BN, WGM, WGN, NSTAGE, RN>;
-  auto kernel =
-      wmmae_gemm::tcec_gemm_kernel<MT, TERMS, BM, BN, WGM, WGN, NSTAGE, RN>;
+  constexpr int NSTAGE = DIRECT ? 2 : ring_depth(BM, BN, TERMS);
+  using Cfg =
+      wmmae_gemm::GemmConfig<MT, TERMS, BM, BN, WGM, WGN, NSTAGE, RN, DIRECT>;
+  auto kernel = wmmae_gemm::tcec_gemm_kernel<MT, TERMS, BM, BN, WGM, WGN,
+                                             NSTAGE, RN, DIRECT>;
   static std::atomic<unsigned long long> lds_allowed{0};
   WMMAE_HIP_TRY(allow_dynamic_lds(reinterpret_cast<const void *>(kernel),
                                   Cfg::LDS_BYTES, lds_allowed));
@@ -458,7 +475,7 @@ int launch_gemm(const GemmArgs &g) {
                      g.stride_c, split_stages,
                      zdim > 1 ? g.partial : static_cast<float *>(nullptr),
                      g.c_ptrs, g.batch, zdim, entry_per_xcd, tail_begin,
-                     tail.stages, g.tail_ws);
+                     tail.stages, g.tail_ws, g.direct);
   int st = launch_status();
   if (st == WMMAE_STATUS_SUCCESS && tail_begin != 0xffffffffu) {
     hipLaunchKernelGGL((wmmae_gemm::reduce_tail_kernel<BM, BN>),
@@ -495,6 +512,10 @@ template <class MT, int TERMS, bool RN> int gemm_by_size(const GemmArgs &g) {
       ceil_div(g.m, 256) * ceil_div(g.n, 128) * g.batch * z;
   const long long mid =
       ceil_div(g.m, 128) * ceil_div(g.n, 128) * g.batch * z;
+  if constexpr (TERMS <= 2 && !RN) {
+    if (g.is_direct)
+      return launch_gemm<MT, TERMS, 256, 128, 2, 2, RN, true>(g);
+  }
   // (not with the separate fp32 adds of RN: their temporaries do not fit the
   // register file next to the large tile's accumulators)
   if constexpr (!RN) {
@@ -632,18 +653,46 @@ int fused_dispatch(const int policy, const FusedArgs &f) {
 // packed path's speed in the median over 114 random products with k % 4 != 0
 // (faster than the packed path in one of them, by 10 %, at k = 77), so such
 // products take the packed path unless k is very short.
-inline bool use_fused(const int m, const int n, const int k, const int batch,
-                      const int flags, const int terms, const int policy,
-                      const bool fused_vec = true) {
+// The third path, "direct": the packed path's GEMM kernel (256x128 tiles)
+// loading the fp32 operands itself and splitting them on their way into LDS.
+// No packed copy and no split pass, at 1.5 times the time per k stage; it wins
+// where an operand element is used by few tiles (batches of small and medium
+// matrices, K-heavy products).  It needs k contiguous in both operands, k a
+// multiple of 32 and at most two terms; same bits as the packed path.
+enum class Path { Fused, Packed, Direct };
+constexpr int kPathFlags =
+    WMMAE_FLAG_PATH_PACKED | WMMAE_FLAG_PATH_FUSED | WMMAE_FLAG_PATH_DIRECT;
+constexpr int kAllFlags = WMMAE_FLAG_RN_MAIN | kPathFlags;
+inline bool one_path_at_most(const int flags) {
+  const int f = flags & kPathFlags;
+  return (f & (f - 1)) == 0;
+}
+inline Path choose_path(const int m, const int n, const int k, const int batch,
+                        const int flags, const int terms, const int policy,
+                        const bool fused_vec, const bool direct_ok) {
   // (the round-to-nearest flag with a policy that has no such variant is
   // turned down by the packed path's dispatch)
   const bool rn_unsupported =
       (flags & WMMAE_FLAG_RN_MAIN) != 0 && policy != WMMAE_POLICY_F16_EC &&
       policy != WMMAE_POLICY_BF16X3_EC;
-  if (k <= 0 || rn_unsupported || choose_splits(terms, m, n, k, batch) != 1)
-    return false;
-  if (!fused_vec && k > 96)
-    return false;
+  if (k <= 0 || rn_unsupported)
+    return Path::Packed;
+  const int splits = choose_splits(terms, m, n, k, batch);
+  if (splits != 1) {
+    // K slices: the split pass against the slower stages of the direct kernel
+    if (!direct_ok)
+      return Path::Packed;
+    const fit::PathRates &pk = fit::kPacked[terms - 1];
+    const double ab = (static_cast<double>(m) + n) * k * batch;
+    const double gemm = split_time(terms, m, n, batch,
+                                   static_cast<int>(ceil_div(k, 32)), splits);
+    const double t_packed =
+        pk.launch + (4.0 + 2.0 * terms) * ab / pk.split_bytes_per_s + gemm;
+    const double t_direct =
+        fit::kDirect[terms - 1].launch + gemm * fit::kDirectSliceRatio[terms - 1];
+    return t_direct < t_packed ? Path::Direct : Path::Packed;
+  }
+  const bool fused_allowed = fused_vec || k <= 96;
   const fit::PathRates &f = fit::kFused[terms - 1], &p = fit::kPacked[terms - 1];
   const long long cus = device_cus();
   const double kt = static_cast<double>(ceil_div(k, 32));
@@ -683,7 +732,31 @@ inline bool use_fused(const int m, const int n, const int k, const int batch,
   const double t_packed =
       p.launch + (4.0 + 2.0 * terms) * ab / p.split_bytes_per_s +
       std::max(units * (kt * p.stage + p.tile), c_bytes / p.bytes_per_s);
-  return t_fused < t_packed;
+  double t_best = t_packed;
+  Path best = Path::Packed;
+  if (fused_allowed && t_fused < t_best) {
+    t_best = t_fused;
+    best = Path::Fused;
+  }
+  if (direct_ok) {
+    const fit::PathRates &d = fit::kDirect[terms - 1];
+    const double t_direct =
+        d.launch +
+        std::max(fit::kUnits256x128 *
+                     static_cast<double>(ceil_div(tiles256, cus)) *
+                     (kt * d.stage + d.tile),
+                 (c_bytes + 4.0 * ab) / d.bytes_per_s);
+    if (t_direct < t_best)
+      best = Path::Direct;
+  }
+  return best;
+}
+// what the direct kernel needs of a product (the operands' k strides are 1)
+inline bool direct_possible(const int k, const int terms, const int flags,
+                            const long long a_rs, const long long b_rs) {
+  return k > 0 && k % 32 == 0 && terms <= 2 &&
+         (flags & WMMAE_FLAG_RN_MAIN) == 0 && a_rs < (1 << 24) &&
+         b_rs < (1 << 24);
 }
 
 inline bool is_n(const char t) { return t == 'N' || t == 'n'; }
@@ -802,6 +875,29 @@ int pack_impl(const int policy, const int rows, const int k,
                        static_cast<hipStream_t>(stream));
 }
 
+// split-K, or K slices for a partly empty last round, only when the caller
+// supplied room for the slices
+void plan_k_slices(GemmArgs &g, void *const workspace,
+                   const size_t workspace_bytes) {
+  g.splits = choose_splits(g.terms, g.m, g.n, g.k, g.batch);
+  g.partial = nullptr;
+  g.tail_ws = nullptr;
+  g.tail_ws_bytes = 0;
+  const bool ws_usable =
+      workspace != nullptr && reinterpret_cast<uintptr_t>(workspace) % 16 == 0;
+  if (g.splits > 1 && ws_usable &&
+      workspace_bytes >=
+          static_cast<size_t>(g.splits) * g.batch * g.m * g.n * 4u) {
+    g.partial = static_cast<float *>(workspace);
+  } else {
+    g.splits = 1;
+    if (ws_usable) {
+      g.tail_ws = static_cast<float *>(workspace);
+      g.tail_ws_bytes = workspace_bytes;
+    }
+  }
+}
+
 int gemm_packed_impl(const int policy, const int m, const int n, const int k,
                      const float *const alpha, const void *const packed_a,
                      const void *const packed_b, const float *const beta,
@@ -854,23 +950,7 @@ int gemm_packed_impl(const int policy, const int m, const int n, const int k,
   g.batch = batch;
   g.terms = p.terms;
   g.stream = static_cast<hipStream_t>(stream);
-  // split-K only when the caller supplied room for the slices
-  g.splits = choose_splits(p.terms, m, n, k, batch);
-  g.partial = nullptr;
-  g.tail_ws = nullptr;
-  g.tail_ws_bytes = 0;
-  const bool ws_usable =
-      workspace != nullptr && reinterpret_cast<uintptr_t>(workspace) % 16 == 0;
-  if (g.splits > 1 && ws_usable &&
-      workspace_bytes >= static_cast<size_t>(g.splits) * batch * m * n * 4u) {
-    g.partial = static_cast<float *>(workspace);
-  } else {
-    g.splits = 1;
-    if (ws_usable) {
-      g.tail_ws = static_cast<float *>(workspace);
-      g.tail_ws_bytes = workspace_bytes;
-    }
-  }
+  plan_k_slices(g, workspace, workspace_bytes);
   return gemm_dispatch(policy, flags, g);
 }
 
@@ -887,7 +967,7 @@ int sgemm_impl(const char transa, const char transb, const int m, const int n,
   PolicyInfo p;
   if ((!is_n(transa) && !is_t(transa)) || (!is_n(transb) && !is_t(transb)) ||
       m < 0 || n < 0 || k < 0 || batch < 0 || !policy_info(policy, p) ||
-      (flags & ~WMMAE_FLAG_RN_MAIN) != 0)
+      (flags & ~kAllFlags) != 0 || !one_path_at_most(flags))
     return WMMAE_STATUS_INVALID_VALUE;
   if (alpha == nullptr || beta == nullptr)
     return WMMAE_STATUS_NULL_POINTER;
@@ -914,7 +994,66 @@ int sgemm_impl(const char transa, const char transb, const int m, const int n,
                      (a_ptrs != nullptr || (aligned16(A) && stride_a % 4 == 0));
   const bool vec_b = b_ks == 1 && k % 4 == 0 && b_rs % 4 == 0 &&
                      (b_ptrs != nullptr || (aligned16(B) && stride_b % 4 == 0));
-  if (use_fused(m, n, k, batch, flags, p.terms, policy, vec_a && vec_b)) {
+  const bool direct_ok = a_ks == 1 && b_ks == 1 &&
+                         direct_possible(k, p.terms, flags, a_rs, b_rs);
+  const int rn = flags & WMMAE_FLAG_RN_MAIN;
+  Path path = choose_path(m, n, k, batch, rn, p.terms, policy, vec_a && vec_b,
+                          direct_ok);
+  if ((flags & WMMAE_FLAG_PATH_DIRECT) != 0) {
+    if (!direct_ok)
+      return WMMAE_STATUS_NOT_SUPPORTED;
+    path = Path::Direct;
+  } else if ((flags & WMMAE_FLAG_PATH_FUSED) != 0) {
+    if (k <= 0 || (rn != 0 && policy != WMMAE_POLICY_F16_EC &&
+                   policy != WMMAE_POLICY_BF16X3_EC))
+      return WMMAE_STATUS_NOT_SUPPORTED;
+    path = Path::Fused;
+  } else if ((flags & WMMAE_FLAG_PATH_PACKED) != 0) {
+    path = Path::Packed;
+  }
+  if (path == Path::Direct) {
+    // the planes of the K slices are the only workspace this path uses
+    size_t bytes_c = 0;
+    wmmae_tcec_gemm_packed_workspace_bytes(policy, m, n, k, batch, &bytes_c);
+    hipStream_t s = static_cast<hipStream_t>(stream);
+    void *ws = workspace;
+    size_t ws_bytes = workspace_bytes;
+    bool own = false;
+    if (ws == nullptr) {
+      if (bytes_c > 0) {
+        WMMAE_HIP_TRY(hipMallocAsync(&ws, bytes_c, s));
+        ws_bytes = bytes_c;
+        own = true;
+      }
+    } else if (reinterpret_cast<uintptr_t>(ws) % 16 != 0) {
+      return WMMAE_STATUS_MISALIGNED;
+    }
+    GemmArgs g;
+    g.a = nullptr;
+    g.b = nullptr;
+    g.c = C;
+    g.c_ptrs = c_ptrs;
+    g.m = m;
+    g.n = n;
+    g.k = k;
+    g.ldc = ldc;
+    g.stride_c = stride_c;
+    g.alpha = *alpha;
+    g.beta = *beta;
+    g.inv_scale = p.inv_scale;
+    g.batch = batch;
+    g.terms = p.terms;
+    g.stream = s;
+    g.is_direct = true;
+    g.direct = wmmae_gemm::DirectSource{A,    B,    a_ptrs,   b_ptrs,
+                                        a_rs, b_rs, stride_a, stride_b};
+    plan_k_slices(g, ws, ws_bytes);
+    int st = gemm_dispatch(policy, 0, g);
+    if (own && hipFreeAsync(ws, s) != hipSuccess && st == WMMAE_STATUS_SUCCESS)
+      st = WMMAE_STATUS_RUNTIME_ERROR;
+    return st;
+  }
+  if (path == Path::Fused) {
     if (batch > (1 << 26)) // tile indices are 32-bit
       return WMMAE_STATUS_NOT_SUPPORTED;
     FusedArgs f;
@@ -994,7 +1133,8 @@ int sgemm_impl(const char transa, const char transb, const int m, const int n,
   }
   if (st == WMMAE_STATUS_SUCCESS)
     st = gemm_packed_impl(policy, m, n, k, alpha, pa, pb, beta, C, c_ptrs, ldc,
-                          stride_c, batch, flags, pc, bytes_c, stream);
+                          stride_c, batch, flags & WMMAE_FLAG_RN_MAIN, pc, bytes_c,
+                          stream);
   if (own) {
     if (hipFreeAsync(workspace, s) != hipSuccess &&
         st == WMMAE_STATUS_SUCCESS)
@@ -1076,13 +1216,19 @@ int wmmae_tcec_sgemm_path(const int m, const int n, const int k,
   if (m < 0 || n < 0 || k < 0 || batch < 0 || !policy_info(policy, p) ||
       (flags & ~WMMAE_FLAG_RN_MAIN) != 0)
     return WMMAE_STATUS_INVALID_VALUE;
-  if (use_fused(m, n, k, batch, flags, p.terms, policy))
+  const bool slices = m > 0 && n > 0 && k > 0 && batch > 0 &&
+                      choose_splits(p.terms, m, n, k, batch) > 1;
+  switch (choose_path(m, n, k, batch, flags, p.terms, policy, true,
+                      direct_possible(k, p.terms, flags, 1, 1))) {
+  case Path::Fused:
     *path = 0;
-  else
-    *path = (m > 0 && n > 0 && k > 0 && batch > 0 &&
-             choose_splits(p.terms, m, n, k, batch) > 1)
-                ? 2
-                : 1;
+    break;
+  case Path::Direct:
+    *path = slices ? 4 : 3;
+    break;
+  default:
+    *path = slices ? 2 : 1;
+  }
   return WMMAE_STATUS_SUCCESS;
 }
 

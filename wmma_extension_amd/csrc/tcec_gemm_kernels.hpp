@@ -43,6 +43,11 @@ __device__ __forceinline__ void static_for(F &&f) {
     static_for<B + 1, E>(f);
   }
 }
+// Row permutation of k group q (0..3) of a chunk written by the DIRECT
+// variant of tcec_gemm_kernel.
+__host__ __device__ constexpr unsigned direct_swizzle(const unsigned q) {
+  return 12u * (q & 1u) ^ 4u * (q >> 1);
+}
 // Number of LDS reads that have been issued once `count` MFMAs of a step are
 // out: read r is due after MFMA number (r+1)*span/nfrag.
 __host__ __device__ constexpr int reads_due(const int count, const int span,
@@ -327,8 +332,19 @@ __global__ void __launch_bounds__(256)
 // C is column major (element (i,j) at C[i + j*ldc]); an accumulator lane owns
 // four consecutive rows of one column, i.e. one 16-byte store.
 // --------------------------------------------------------------------------
+// fp32 operands of the DIRECT variant of tcec_gemm_kernel, which splits them
+// itself: op(A) as m rows of k contiguous floats (row i at A + i*lda), op(B)
+// as n rows of k contiguous floats (row j at B + j*ldb); batch entry y at
+// base + y*bs or, when the pointer arrays are set, at ptrs[y].
+struct DirectSource {
+  const float *A, *B;
+  const float *const *a_ptrs, *const *b_ptrs;
+  long long lda, ldb;
+  long long a_bs, b_bs;
+};
+
 template <class MT, int TERMS, int BM, int BN, int WGM, int WGN, int NSTAGE,
-          bool RN_MAIN>
+          bool RN_MAIN, bool DIRECT = false>
 struct GemmConfig {
   static constexpr int NW = WGM * WGN;
   static constexpr int NTHREADS = NW * 64;
@@ -344,7 +360,11 @@ struct GemmConfig {
   // one) must fit the 256 vector registers beside the accumulators; when they
   // do not, the A fragments of all tile rows but the last exist once and are
   // refilled for the next stage as soon as their tile row has been issued.
-  static constexpr bool RECYCLE_A = 2 * TERMS * (MT_ + NT_) * 4 > 256;
+  // (DIRECT needs room for the fp32 values in flight as well.)
+  static constexpr bool RECYCLE_A =
+      2 * TERMS * (MT_ + NT_) * 4 > (DIRECT ? 128 : 256);
+  static_assert(!DIRECT || (NSTAGE == 2 && TERMS <= 2),
+                "DIRECT: two LDS buffers, one or two terms");
   static_assert(NCH % NW == 0, "chunks must divide evenly over the waves");
   static_assert(WM % 16 == 0 && WN % 16 == 0, "wave tile must be MFMA tiles");
   static_assert(NSTAGE >= 2 && NSTAGE <= 4, "ring depth");
@@ -353,7 +373,7 @@ struct GemmConfig {
 };
 
 template <class MT, int TERMS, int BM, int BN, int WGM, int WGN, int NSTAGE,
-          bool RN_MAIN>
+          bool RN_MAIN, bool DIRECT = false>
 __global__ void __launch_bounds__(WGM *WGN * 64)
     tcec_gemm_kernel(const u32x4 *__restrict__ Ap, const u32x4 *__restrict__ Bp,
                      float *__restrict__ C, const int M, const int N,
@@ -368,8 +388,8 @@ __global__ void __launch_bounds__(WGM *WGN * 64)
                      float *const *__restrict__ c_ptrs, const int batches,
                      const int splits, const int entry_per_xcd,
                      const unsigned tail_begin, const int tail_stages,
-                     float *__restrict__ tail_partial) {
-  using Cfg = GemmConfig<MT, TERMS, BM, BN, WGM, WGN, NSTAGE, RN_MAIN>;
+                     float *__restrict__ tail_partial, const DirectSource ds) {
+  using Cfg = GemmConfig<MT, TERMS, BM, BN, WGM, WGN, NSTAGE, RN_MAIN, DIRECT>;
   typedef MT ab_vec __attribute__((ext_vector_type(8)));
   constexpr int NCH = Cfg::NCH, CH_A = Cfg::CH_A, CPW = Cfg::CPW;
   constexpr int MT_ = Cfg::MT_, NT_ = Cfg::NT_;
@@ -491,12 +511,19 @@ __global__ void __launch_bounds__(WGM *WGN * 64)
   // 1024x1024x256 measured 276 against 258 effective TFLOPS) and for the
   // three-term 256x128 tile (16384^3: 29.5 against 30.0 ms), w*RPW ..
   // w*RPW + RPW-1 for the three-term 128x128 tile (16384^3: 240 against 219).
-  constexpr unsigned STAGE_BYTES = CH_PER_RB * 1024u; // one stage of a row block
+  // DIRECT: the sources are fp32 rows instead (gsrc[g]: first row of the row
+  // block at the cursor's k) and a stage is 32 floats further along the rows.
+  // A row block is fetched by two loads of eight rows each, eight lanes to a
+  // row (one whole 128-byte line; lane l: row l/8 or 8 + l/8, clamped to the
+  // operand's last row, floats 4*(l%8) .. +3: voff[g][0..1]).
+  constexpr unsigned STAGE_BYTES =
+      DIRECT ? 32u * 4u : CH_PER_RB * 1024u;          // one stage of a row block
   constexpr int RPW = CPW / CH_PER_RB;                // row blocks per wave
   constexpr bool STRIDED_RB = TERMS <= 2 || Cfg::RECYCLE_A;
   constexpr int RB_STEP = STRIDED_RB ? Cfg::NW : 1; // between a wave's row blocks
   static_assert(CPW % CH_PER_RB == 0, "a wave requests whole row blocks");
   unsigned long long gsrc[RPW];
+  unsigned voff[DIRECT ? RPW : 1][2];
   unsigned lane_off = lane * 16u;
   int req_item = 0, req_st = 0, req_stages = 0;
   auto set_sources = [&](const int i) {
@@ -506,6 +533,35 @@ __global__ void __launch_bounds__(WGM *WGN * 64)
         partial != nullptr || it.tail >= 0
             ? static_cast<long long>(it.z) * slice_stages(it)
             : 0;
+    if constexpr (DIRECT) {
+      // the pointer arrays are read with scalar loads (constant address space)
+      typedef const float *const __attribute__((address_space(4))) *ptr_array_t;
+      const float *const Ab = ds.a_ptrs != nullptr
+                                  ? ((ptr_array_t)ds.a_ptrs)[it.batch]
+                                  : ds.A + it.batch * ds.a_bs;
+      const float *const Bb = ds.b_ptrs != nullptr
+                                  ? ((ptr_array_t)ds.b_ptrs)[it.batch]
+                                  : ds.B + it.batch * ds.b_bs;
+#pragma unroll
+      for (int g = 0; g < RPW; g++) {
+        const int r = STRIDED_RB ? wave + Cfg::NW * g : wave * RPW + g;
+        const bool is_a = r < RBM;
+        const int last = (is_a ? M : N) - 1;
+        int row0 = is_a ? it.tm * BM + 16 * r : it.tn * BN + 16 * (r - RBM);
+        row0 = row0 < last ? row0 : last;
+        const long long ld = is_a ? ds.lda : ds.ldb;
+        gsrc[g] = reinterpret_cast<unsigned long long>(
+            (is_a ? Ab : Bb) + row0 * ld + first_stage * 32);
+        asm volatile("" : "+s"(gsrc[g]));
+#pragma unroll
+        for (int h = 0; h < 2; h++) {
+          int mine = row0 + 8 * h + static_cast<int>(lane >> 3);
+          mine = (mine < last ? mine : last) - row0;
+          voff[g][h] = static_cast<unsigned>(mine * ld) * 4u + 16u * (lane & 7u);
+        }
+      }
+      return;
+    }
 #pragma unroll
     for (int g = 0; g < RPW; g++) {
       // row block inside the stage: A's, then B's
@@ -575,6 +631,91 @@ __global__ void __launch_bounds__(WGM *WGN * 64)
         16, (q % CH_PER_RB) * 1024, 0);
   };
 
+  // DIRECT: what a wave does per stage for each of its RPW row blocks instead
+  // of the requests above.  A lane's eight floats (four from each of the two
+  // loads of a row block) stay in registers from the load to the split one
+  // step later:
+  //   load_rb  : the lane's floats of row block g at the cursor's stage
+  //   split_rb : pair P of them -> one register of each term
+  //   write_rb : the terms as 8-byte halves of the 16-byte fragment positions
+  //              of the stage image in LDS, where the packed operands would
+  //              have been copied to
+  using SplitTag = typename std::conditional<std::is_same<MT, _Float16>::value,
+                                             mtk::wmma::half,
+                                             mtk::wmma::bfloat16>::type;
+  typedef MT s2_t __attribute__((ext_vector_type(2)));
+  float raw[DIRECT ? RPW : 1][8];
+  unsigned term[2][4];
+  auto load_rb = [&](auto G) {
+    constexpr int g = decltype(G)::value;
+    // 16-byte loads; the address need only be a float's (global memory is
+    // accessed in unaligned mode), so any leading dimension and base work
+    typedef f32x4 __attribute__((aligned(4))) f32x4_u;
+    typedef const __attribute__((address_space(1))) f32x4_u *vec_ptr;
+    const auto *const p =
+        reinterpret_cast<const __attribute__((address_space(1))) char *>(
+            gsrc[g]);
+    // (the offsets are redefined in place so that each address is formed here,
+    // as the instruction's scalar base + 32-bit lane offset, and not hoisted
+    // into vector register pairs)
+    asm volatile("" : "+v"(voff[g][0]), "+v"(voff[g][1]));
+    const f32x4 lo = *reinterpret_cast<vec_ptr>(p + voff[g][0]);
+    const f32x4 hi = *reinterpret_cast<vec_ptr>(p + voff[g][1]);
+#pragma unroll
+    for (int x = 0; x < 4; x++) {
+      raw[g][x] = lo[x];
+      raw[g][4 + x] = hi[x];
+    }
+  };
+  auto split_rb = [&](auto G, auto P) {
+    constexpr int g = decltype(G)::value, q = decltype(P)::value;
+    s2_t h0, h1, h2;
+    mtk::wmma::tcec::detail::split2<SplitTag>(
+        mtk::wmma::tcec::detail::f32x2_t{raw[g][2 * q], raw[g][2 * q + 1]}, h0,
+        h1, h2);
+    term[0][q] = __builtin_bit_cast(unsigned, h0);
+    if constexpr (TERMS >= 2)
+      term[1][q] = __builtin_bit_cast(unsigned, h1);
+  };
+  // A lane's four values of a load are half of a fragment position (row r,
+  // k group q = k/8 of the stage): position r + 16*q of the chunk, stored at
+  // 16-byte slot 16*q + (r ^ swz(q)), swz = 0, 12, 4, 8.  The lanes of a
+  // load that hold the same row differ in q; without the permutation their
+  // 8-byte writes fall on the same banks (measured at 8192^3: bank-conflict
+  // cycles 6.1e8 with slots in position order, 4.1e8 with a rotation by 4*q,
+  // 2.0e8 with this one; the 16-byte fragment reads, lane = position, stay
+  // conflict free).
+  typedef unsigned u32x2 __attribute__((ext_vector_type(2)));
+  unsigned woff[2];
+#pragma unroll
+  for (int h = 0; h < 2; h++) {
+    const unsigned r = 8u * h + (lane >> 3), q = (lane & 7u) >> 1;
+    woff[h] = 256u * q + 16u * (r ^ direct_swizzle(q)) + 8u * (lane & 1u);
+  }
+  auto write_rb = [&](const int w_base, auto G) {
+    constexpr int g = decltype(G)::value;
+#pragma unroll
+    for (int t = 0; t < TERMS; t++)
+#pragma unroll
+      for (int h = 0; h < 2; h++)
+        *reinterpret_cast<u32x2 *>(lds_raw + w_base +
+                                   g * RB_STEP * CH_PER_RB * 1024 + t * 1024 +
+                                   woff[h]) =
+            u32x2{term[t][2 * h], term[t][2 * h + 1]};
+  };
+  // micro-operation U of a step's RPW * 6 (per row block: four pairs to
+  // split, the writes, the loads of the stage after)
+  constexpr int NUOP = RPW * 6;
+  auto direct_uop = [&](const int w_base, auto U) {
+    constexpr int u = decltype(U)::value, g = u / 6, o = u % 6;
+    if constexpr (o < 4)
+      split_rb(ic<g>{}, ic<o>{});
+    else if constexpr (o == 4)
+      write_rb(w_base, ic<g>{});
+    else
+      load_rb(ic<g>{});
+  };
+
   // In-place accumulate, written as inline assembly so that every accumulator
   // stays in one fixed accumulation register for the whole K loop (with the
   // largest tile the accumulators fill the register file exactly, and the
@@ -621,13 +762,17 @@ __global__ void __launch_bounds__(WGM *WGN * 64)
       return f.a[t][0];
   };
   constexpr int NFRAG = TERMS * (MT_ + NT_);
+  // 16-byte slot of this lane's fragment inside a chunk: the lane itself, or
+  // with DIRECT the permuted slot the chunks were written with
+  const unsigned frag_slot =
+      DIRECT ? (lane & 48u) + ((lane & 15u) ^ direct_swizzle(lane >> 4)) : lane;
   // fragment IDX of a stage (compile-time index, so that every fragment is a
   // fixed register): B fragments first, then A (RECYCLE: A's last tile row
   // first, then rows 0 .. MT_-2)
   auto read_frag = [&](Frags &f, const int r_base, auto IDX) {
     constexpr int r = decltype(IDX)::value;
     const u32x4 *const stage =
-        reinterpret_cast<const u32x4 *>(lds_raw + r_base) + lane;
+        reinterpret_cast<const u32x4 *>(lds_raw + r_base) + frag_slot;
     if constexpr (r < TERMS * NT_) {
       constexpr int j = r / TERMS, t = r % TERMS;
       const u32x4 *const sb = stage + (CH_A + wn * NT_ * CH_PER_RB) * 64;
@@ -700,10 +845,15 @@ __global__ void __launch_bounds__(WGM *WGN * 64)
     // the requests of the stage read next are older than those of the
     // NSTAGE-2 stages after it (the branch sits before the barrier, where
     // the wave waits anyway)
-    if (skip_waits > 0)
-      skip_waits--;
-    else
-      asm volatile("s_waitcnt vmcnt(%0)" ::"n"(CPW * (NSTAGE - 2)) : "memory");
+    // (DIRECT: the stage read next was written to LDS by the waves
+    // themselves during the last step; the barrier publishes it)
+    if constexpr (!DIRECT) {
+      if (skip_waits > 0)
+        skip_waits--;
+      else
+        asm volatile("s_waitcnt vmcnt(%0)" ::"n"(CPW * (NSTAGE - 2))
+                     : "memory");
+    }
     asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");
 
     static_for<0, NMFMA>([&](auto N_) {
@@ -748,18 +898,35 @@ __global__ void __launch_bounds__(WGM *WGN * 64)
         acc_err[i][j] = mfma(a_frag(cur, ic<ta>{}, ic<i>{}), cur.b[tb][j],
                              acc_err[i][j]);
       }
-      // global->LDS requests due after this MFMA
-      constexpr int qlo = (n * CPW + REQ_SPAN - 1) / REQ_SPAN;
-      constexpr int qhi = ((n + 1) * CPW + REQ_SPAN - 1) / REQ_SPAN;
-      static_for<(qlo < CPW ? qlo : CPW), (qhi < CPW ? qhi : CPW)>([&](auto Q) {
-        issue_chunk(w_base, Q);
-        __builtin_amdgcn_sched_barrier(0);
-      });
-      // all requests of this step are out: move the cursor on while the
-      // remaining MFMAs run
-      if constexpr (n == N_ADVANCE) {
-        advance_request();
-        __builtin_amdgcn_sched_barrier(0);
+      if constexpr (DIRECT) {
+        // split the stage after next (loaded during the last step) into the
+        // buffer the current stage has left, load the stage after that: the
+        // micro-operations spread evenly over the step
+        constexpr int ulo = (n * NUOP + NMFMA - 1) / NMFMA;
+        constexpr int uhi = ((n + 1) * NUOP + NMFMA - 1) / NMFMA;
+        static_for<ulo, (uhi < NUOP ? uhi : NUOP)>([&](auto U) {
+          direct_uop(w_base, U);
+          __builtin_amdgcn_sched_barrier(0);
+        });
+        if constexpr (n == NMFMA - 1) {
+          advance_request();
+          __builtin_amdgcn_sched_barrier(0);
+        }
+      } else {
+        // global->LDS requests due after this MFMA
+        constexpr int qlo = (n * CPW + REQ_SPAN - 1) / REQ_SPAN;
+        constexpr int qhi = ((n + 1) * CPW + REQ_SPAN - 1) / REQ_SPAN;
+        static_for<(qlo < CPW ? qlo : CPW), (qhi < CPW ? qhi : CPW)>(
+            [&](auto Q) {
+              issue_chunk(w_base, Q);
+              __builtin_amdgcn_sched_barrier(0);
+            });
+        // all requests of this step are out: move the cursor on while the
+        // remaining MFMAs run
+        if constexpr (n == N_ADVANCE) {
+          advance_request();
+          __builtin_amdgcn_sched_barrier(0);
+        }
       }
       // LDS reads due after this MFMA
       if constexpr (RECYCLE) {
@@ -846,14 +1013,27 @@ __global__ void __launch_bounds__(WGM *WGN * 64)
   // ---- prologue: request the first NSTAGE stages of the stream, fetch the
   // first stage's fragments
   set_sources(0);
-#pragma unroll
-  for (int s = 0; s < NSTAGE; s++) {
-    static_for<0, CPW>([&](auto Q) { issue_chunk(wave_base(s), Q); });
-    advance_request();
-  }
   Frags f0, f1;
-  asm volatile("s_waitcnt vmcnt(%0)\n\ts_barrier" ::"n"(CPW * (NSTAGE - 1))
-               : "memory");
+  if constexpr (DIRECT) {
+    // stages 0 and 1 of the stream into the two LDS buffers, stage 2 into
+    // the registers
+    static_for<0, RPW>([&](auto G) { load_rb(G); });
+    advance_request();
+#pragma unroll
+    for (int s = 0; s < 2; s++) {
+      static_for<0, NUOP>([&](auto U) { direct_uop(wave_base(s), U); });
+      advance_request();
+    }
+    asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");
+  } else {
+#pragma unroll
+    for (int s = 0; s < NSTAGE; s++) {
+      static_for<0, CPW>([&](auto Q) { issue_chunk(wave_base(s), Q); });
+      advance_request();
+    }
+    asm volatile("s_waitcnt vmcnt(%0)\n\ts_barrier" ::"n"(CPW * (NSTAGE - 1))
+                 : "memory");
+  }
   static_for<0, NFRAG>([&](auto R_) { read_frag(f0, 0, R_); });
 
   // ---- items; the stage loop is unrolled by two so that the fragment sets

@@ -24,6 +24,9 @@ class Policy(enum.IntEnum):
 
 
 FLAG_RN_MAIN = 1
+FLAG_PATH_PACKED = 2    # take this path instead of the estimated one
+FLAG_PATH_FUSED = 4
+FLAG_PATH_DIRECT = 8
 
 TYPE_HALF, TYPE_BF16, TYPE_TF32 = 0, 1, 2
 USE_A, USE_B, USE_ACC = 0, 1, 2
