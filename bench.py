@@ -2,8 +2,11 @@
 """Benchmark of the TCEC SGEMM hot path on one MI355X.
 
 One "step" = one full product C = A*B on synthetic seeded fp32 inputs that are
-already resident in HBM: split+pack of A, split+pack of B, MFMA GEMM (the
-workspace for the packed operands is allocated once, outside the timed region).
+already resident in HBM, run on the path the library's time estimates choose
+for the shape: split+pack of A, split+pack of B and the MFMA GEMM on the packed
+path (large single products, the headline workload), or the one kernel that
+splits the fp32 operands itself (batches of medium-sized matrices, K-heavy
+products).  The workspace is allocated once, outside the timed region.
 
 Prints ONE JSON line: effective fp32 TFLOPS (2*M*N*K*batch / t), the MFMA
 roofline of the GEMM kernel measured with HIP events inside the timed region,
@@ -30,21 +33,23 @@ WORKLOADS = {
     "c2": dict(kind="prim", tiles=1 << 20, dist="uniform",
                desc="fragment primitives over 1,048,576 16x16 tiles (foreach_ij fills of A/B row+col, "
                     "accumulator store, load_vector/store_vector)"),
-    "c5a": dict(m=256, n=256, k=256, batch=1024, policy="F16_EC", dist="normal", mult=3, fused=True,
-                desc="strided-batched TCEC SGEMM, 1024 x 256^3 (split inside the GEMM kernel)"),
-    "c5a_packed": dict(m=256, n=256, k=256, batch=1024, policy="F16_EC", dist="normal", mult=3,
-                       desc="strided-batched TCEC SGEMM, 1024 x 256^3, through packed operands"),
+    "c5a": dict(m=256, n=256, k=256, batch=1024, policy="F16_EC", dist="normal", mult=3,
+                desc="strided-batched TCEC SGEMM, 1024 x 256^3"),
+    "c5a_fused": dict(m=256, n=256, k=256, batch=1024, policy="F16_EC", dist="normal", mult=3, path_flag=4,
+                      desc="strided-batched TCEC SGEMM, 1024 x 256^3, forced onto the single (fused) kernel"),
+    "c5a_packed": dict(m=256, n=256, k=256, batch=1024, policy="F16_EC", dist="normal", mult=3, path_flag=2,
+                       desc="strided-batched TCEC SGEMM, 1024 x 256^3, forced through packed operands"),
     "c5b": dict(m=1024, n=1024, k=262144, batch=1, policy="F16_EC", dist="normal", mult=3,
                 desc="K-heavy TCEC SGEMM, M=N=1024, K=262144"),
     "api": dict(kind="api", m=4096, n=4096, k=4096, dist="uniform",
                 desc="GEMM written against the public tcec:: device API only, fp16 hi+lo with EC, M=N=K=4096"),
 }
 # a timed region of a few milliseconds is measured while the power management still ramps
-DEFAULT_STEPS = {"c3": 200, "c5a": 400, "c5a_packed": 200, "c5b": 50, "c2": 100, "api": 200}
+DEFAULT_STEPS = {"c3": 200, "c5a": 400, "c5a_fused": 400, "c5a_packed": 200, "c5b": 50, "c2": 100, "api": 200}
 PEAK_MFMA_TFLOPS = 2500.0      # dense fp16 / bf16 MFMA, MI355X
 PEAK_HBM_GBS = 8000.0
 # workloads whose dominant kernel is bound by HBM rather than by the matrix cores
-HBM_BOUND = {"c2", "c5a", "c5a_packed"}
+HBM_BOUND = {"c2", "c5a", "c5a_fused", "c5a_packed"}
 # Bytes per launch of the dominant kernel that crossed the fabric side of L2 come from two
 # rocprofv3 --pmc runs of this script (FETCH_SIZE, then WRITE_SIZE, with --calibrate), whose
 # summary under profiles/ ends in a line
@@ -54,7 +59,8 @@ HBM_BOUND = {"c2", "c5a", "c5a_packed"}
 TRAFFIC_PROFILES = {
     "c4": "tcec_gemm_kernel_c4_16384_bf16x3.md",
     "c3": "tcec_gemm_kernel_c3_4096_f16.md",
-    "c5a": "tcec_gemm_fused_kernel_c5a_1024x256_f16.md",
+    "c5a": "tcec_gemm_kernel_direct_c5a_1024x256_f16.md",
+    "c5a_fused": "tcec_gemm_fused_kernel_c5a_1024x256_f16.md",
     "c5b": "tcec_gemm_kernel_c5b_1024x1024x262144_f16.md",
     "c2": "primitive_tiles_kernel_c2_1M_tiles.md",
     "api": "tcec_api_gemm_kernel_api_4096_f16.md",
@@ -64,7 +70,8 @@ KERNEL_SOURCES = {
             "include/wmma_extension/tcec/detail/split.hpp", "include/wmma_extension/utils.hpp",
             "include/wmma_extension/wmma_extension.hpp", "include/wmma_extension/detail/mfma.hpp"],
     "c4": ["tcec_gemm_kernels.hpp"], "c3": ["tcec_gemm_kernels.hpp"], "c5b": ["tcec_gemm_kernels.hpp"],
-    "c5a": ["tcec_gemm_kernels.hpp", "tcec_gemm_fused_kernel.hpp"], "c2": ["harness_kernels.hpp"],
+    "c5a": ["tcec_gemm_kernels.hpp"], "c5a_fused": ["tcec_gemm_kernels.hpp", "tcec_gemm_fused_kernel.hpp"],
+    "c2": ["harness_kernels.hpp"],
 }
 
 
@@ -306,20 +313,31 @@ def run_gemm_workload(args, torch, tcec, dev, name, steps, warmup):
     m, n, k, batch = w["m"], w["n"], w["k"], w["batch"]
     A, Bt = make_inputs(torch, w, dev, 0x5EED + 3)
     Ct = torch.empty((batch, n, m), dtype=torch.float32, device=dev)
-    fused = bool(w.get("fused"))
-    if not fused:
+    # The step is the product the way the library runs it: the path its time estimates choose
+    # for the shape (a workload may force another one), inputs and workspace resident in HBM.
+    # On the packed path the two split passes and the GEMM are separate calls here, so that
+    # the events bracket the GEMM kernel alone; the other paths are one call (one kernel,
+    # plus the fold of the K slices where there are any).
+    flags = args.flags | w.get("path_flag", 0)
+    path = {2: tcec.PATH_PACKED, 4: tcec.PATH_FUSED, 8: tcec.PATH_DIRECT}.get(
+        flags & 14, tcec.sgemm_path(m, n, k, batch, policy, flags & 1))
+    packed = path in (tcec.PATH_PACKED, tcec.PATH_PACKED_SPLIT_K)
+    fused = path == tcec.PATH_FUSED
+    if packed:
         pa = torch.empty(tcec.pack_bytes(m, k, batch, policy), dtype=torch.uint8, device=dev)
         pb = torch.empty(tcec.pack_bytes(n, k, batch, policy), dtype=torch.uint8, device=dev)
         ws_bytes = tcec.gemm_packed_workspace_bytes(policy, m, n, k, batch)
         ws = torch.empty(ws_bytes, dtype=torch.uint8, device=dev) if ws_bytes else None
+    else:
+        ws_bytes = tcec.workspace_bytes(m, n, k, batch, policy)   # holds the planes of K slices
+        ws = torch.empty(ws_bytes, dtype=torch.uint8, device=dev) if ws_bytes else None
 
     def step(ev=None):
-        if fused:
-            # small products: one kernel reads fp32 A and B, splits in registers, writes C
+        if not packed:
             if ev is not None:
                 ev[0].record()
             tcec.sgemm_strided_batched("T", "N", m, n, k, 1.0, A, k, m * k, Bt, k, n * k, 0.0,
-                                       Ct, m, n * m, batch, policy, args.flags)
+                                       Ct, m, n * m, batch, policy, flags, ws)
             if ev is not None:
                 ev[1].record()
             return
@@ -327,7 +345,7 @@ def run_gemm_workload(args, torch, tcec, dev, name, steps, warmup):
         tcec.pack(policy, n, k, Bt, k, 1, pb, batch, n * k)
         if ev is not None:
             ev[0].record()
-        tcec.gemm_packed(policy, m, n, k, 1.0, pa, pb, 0.0, Ct, m, batch, n * m, args.flags, ws)
+        tcec.gemm_packed(policy, m, n, k, 1.0, pa, pb, 0.0, Ct, m, batch, n * m, flags & 1, ws)
         if ev is not None:
             ev[1].record()
 
@@ -369,23 +387,25 @@ def run_gemm_workload(args, torch, tcec, dev, name, steps, warmup):
     achieved = flops * w["mult"] / (gemm_ms * 1e-3) / 1e12
     bytes_min = 4.0 * (m * k + k * n + m * n) * batch
     traffic, traffic_source = measured_traffic(name)
+    kernel_name = ("tcec_gemm_fused_kernel" if fused else
+                   "tcec_gemm_kernel" if packed else "tcec_gemm_kernel (DIRECT: fp32 operands split in the kernel)")
 
     if name in HBM_BOUND:
         # packed operands in (2*terms bytes per element), C out: the GEMM kernel's own minimum
         terms = {"F16_EC": 2, "BF16X3_EC": 3, "BF16X2_EC": 2, "F16_NOEC": 1, "BF16_NOEC": 1}[w["policy"]]
         kbytes = (2.0 * terms * (m * k + k * n) + 4.0 * m * n) * batch
-        if fused:
+        if not packed:
             kbytes = bytes_min              # fp32 A and B in, fp32 C out
         hbm = kbytes / (gemm_ms * 1e-3) / 1e9
         roofline = {"bound": "hbm", "achieved": round(hbm, 1), "peak": PEAK_HBM_GBS, "unit": "GB/s",
                     "frac": round(hbm / PEAK_HBM_GBS, 4), "traffic": traffic, "traffic_source": traffic_source,
-                    "kernel": "tcec_gemm_fused_kernel" if fused else "tcec_gemm_kernel",
+                    "kernel": kernel_name,
                     "kernel_ms": round(gemm_ms, 4), "algorithmic_bytes": kbytes, "mfma_frac": round(achieved / PEAK_MFMA_TFLOPS, 4)}
     else:
         roofline = {"bound": "mfma", "achieved": round(achieved, 2), "peak": PEAK_MFMA_TFLOPS,
                     "unit": "TFLOP/s", "frac": round(achieved / PEAK_MFMA_TFLOPS, 4),
                     "traffic": traffic, "traffic_source": traffic_source,
-                    "kernel": "tcec_gemm_kernel", "kernel_ms": round(gemm_ms, 4),
+                    "kernel": kernel_name, "kernel_ms": round(gemm_ms, 4),
                     "issued_flop_multiplier": w["mult"],
                     "hbm_frac_of_min_traffic": round(bytes_min / (gemm_ms * 1e-3) / 1e9 / PEAK_HBM_GBS, 4)}
     out = {
@@ -396,11 +416,17 @@ def run_gemm_workload(args, torch, tcec, dev, name, steps, warmup):
         "dtype": "bf16" if "BF16" in w["policy"] else "f16",
         "config": {"workload": f"{name}: {w['desc']}", "m": m, "n": n, "k": k, "batch": batch,
                    "policy": w["policy"], "distribution": w["dist"], "flags": args.flags,
-                   "step": ("one fused split+MFMA GEMM kernel; inputs resident in HBM" if fused else
-                            "split+pack A, split+pack B, MFMA GEMM; inputs and workspace resident in HBM")},
+                   "path": {0: "fused", 1: "packed", 2: "packed + K slices", 3: "direct",
+                            4: "direct + K slices"}[path],
+                   "step": ("split+pack A, split+pack B, MFMA GEMM; inputs and workspace resident in HBM"
+                            if packed else
+                            "one wmmae_tcec_sgemm_strided_batched call (one kernel splits the fp32 operands "
+                            "and multiplies; plus the fold of K slices if any); inputs resident in HBM")},
         "roofline": roofline,
         "gemm_only_effective_tflops": round(flops / (gemm_ms * 1e-3) / 1e12, 3),
     }
+    if path in (tcec.PATH_PACKED_SPLIT_K, tcec.PATH_DIRECT_SPLIT_K):
+        roofline["kernel_ms_covers"] = "the GEMM kernel and the fold of its K slices (the events bracket the call)"
     if trace is not None:
         import numpy as np
         tr = trace.cpu().numpy()

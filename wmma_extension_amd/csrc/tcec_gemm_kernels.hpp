@@ -990,11 +990,18 @@ __global__ void __launch_bounds__(WGM *WGN * 64)
         if constexpr (TERMS >= 2)
           v += acc_err[i][j] * inv_scale;
         v *= a_out;
-        float *const dst = Cb + row + static_cast<long long>(col) * ld_out;
+        // (every destination is device memory: global-memory instructions, not
+        // generic ones, which would also count as LDS operations and make the
+        // compiler drain both memory counters before the next step's first
+        // dependent instruction)
+        typedef __attribute__((address_space(1))) float gfloat;
+        typedef __attribute__((address_space(1))) f32x4 gf32x4;
+        gfloat *const dst =
+            (gfloat *)(Cb + row + static_cast<long long>(col) * ld_out);
         if (vec_out && row + 3 < M) {
           if (b_out != 0.f)
-            v += b_out * *reinterpret_cast<const f32x4 *>(dst);
-          *reinterpret_cast<f32x4 *>(dst) = v;
+            v += b_out * *reinterpret_cast<const gf32x4 *>(dst);
+          *reinterpret_cast<gf32x4 *>(dst) = v;
         } else {
 #pragma unroll
           for (int x = 0; x < 4; x++) {
@@ -1067,7 +1074,12 @@ __global__ void __launch_bounds__(WGM *WGN * 64)
     // depend on those requests skip their counted wait.  The no-ops cover the
     // matrix core's write-to-VALU-read distance for the last accumulate
     // instructions, which the compiler cannot see.
-    asm volatile("s_waitcnt vmcnt(0)\n\ts_nop 15\n\ts_nop 15" ::: "memory");
+    // (DIRECT: the loads in flight fill registers, which the compiler tracks
+    // itself; they need not have landed here.)
+    if constexpr (DIRECT)
+      asm volatile("s_nop 15\n\ts_nop 15" ::: "memory");
+    else
+      asm volatile("s_waitcnt vmcnt(0)\n\ts_nop 15\n\ts_nop 15" ::: "memory");
     skip_waits = NSTAGE - 1;
     store_item(it);
   }

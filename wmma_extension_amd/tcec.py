@@ -106,7 +106,7 @@ def workspace_bytes(m, n, k, batch=1, policy=Policy.F16_EC):
     return out.value
 
 
-PATH_FUSED, PATH_PACKED, PATH_PACKED_SPLIT_K = 0, 1, 2
+PATH_FUSED, PATH_PACKED, PATH_PACKED_SPLIT_K, PATH_DIRECT, PATH_DIRECT_SPLIT_K = 0, 1, 2, 3, 4
 
 
 def sgemm_path(m, n, k, batch=1, policy=Policy.F16_EC, flags=0):
