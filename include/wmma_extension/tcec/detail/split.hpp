@@ -86,35 +86,77 @@ template <> struct split_traits<float> {
 //   bf16 : v_cvt_pk_bf16_f32 pairs, residuals by fp32 subtraction
 typedef float f32x2_t __attribute__((ext_vector_type(2)));
 typedef float f32x4_t __attribute__((ext_vector_type(4)));
+// split2 in single instructions, for callers that place them themselves (the
+// GEMM kernel that splits its own operands issues them one at a time between
+// its matrix instructions):
+//   split2_lead     : the leading terms                        (one instruction)
+//   split2_prep<E>  : what the residual of element E is rounded from - half:
+//                     the value times the scale (the mixed-precision fma
+//                     subtracts); bf16: the fp32 residual, scaled (one / two)
+//   split2_resid_lo : half: the residual term of element 0 into the low half
+//                     of a register; bf16: nothing               (one / none)
+//   split2_resid_hi : the finished pair of residual terms        (one)
+template <class T, class S = typename split_traits<T>::storage,
+          class S2 = S __attribute__((ext_vector_type(2)))>
+WMMAE_D S2 split2_lead(const f32x2_t vv) {
+  static_assert(!std::is_same<S, float>::value, "16-bit terms only");
+  return __builtin_convertvector(vv, S2);
+}
+template <class T, int E, class S = typename split_traits<T>::storage,
+          class S2 = S __attribute__((ext_vector_type(2)))>
+WMMAE_D float split2_prep(const float v, const S2 h0) {
+  using traits = split_traits<T>;
+  if constexpr (std::is_same<S, _Float16>::value) {
+    return v * traits::scale;
+  } else {
+    float r = v - static_cast<float>(h0[E]);
+    if constexpr (traits::scale != 1.f)
+      r *= traits::scale;
+    return r;
+  }
+}
+template <class T, class S = typename split_traits<T>::storage,
+          class S2 = S __attribute__((ext_vector_type(2)))>
+WMMAE_D S2 split2_resid_lo(const S2 h0, const float p0) {
+  using traits = split_traits<T>;
+  S2 h1 = {};
+  if constexpr (std::is_same<S, _Float16>::value) {
+    static_assert(traits::num_terms == 2, "two-term fp16 split");
+    const float neg_scale = -traits::scale;
+    asm("v_fma_mixlo_f16 %0, %1, %2, %3 op_sel:[0,0,0] op_sel_hi:[1,0,0]"
+        : "=v"(h1)
+        : "v"(h0), "s"(neg_scale), "v"(p0));
+  }
+  return h1;
+}
+template <class T, class S = typename split_traits<T>::storage,
+          class S2 = S __attribute__((ext_vector_type(2)))>
+WMMAE_D S2 split2_resid_hi(S2 h1, const S2 h0, const float p0, const float p1) {
+  using traits = split_traits<T>;
+  if constexpr (std::is_same<S, _Float16>::value) {
+    const float neg_scale = -traits::scale;
+    asm("v_fma_mixhi_f16 %0, %1, %2, %3 op_sel:[1,0,0] op_sel_hi:[1,0,0]"
+        : "+v"(h1)
+        : "v"(h0), "s"(neg_scale), "v"(p1));
+    return h1;
+  } else {
+    return __builtin_convertvector(f32x2_t{p0, p1}, S2);
+  }
+}
 // split2: two values -> pairs of terms (h0 leading, h1 residual, h2 second
 // residual; the pairs beyond the split's number of terms are left alone)
 template <class T, class S = typename split_traits<T>::storage,
           class S2 = S __attribute__((ext_vector_type(2)))>
 WMMAE_D void split2(const f32x2_t vv, S2 &h0, S2 &h1, S2 &h2) {
   using traits = split_traits<T>;
-  static_assert(!std::is_same<S, float>::value, "16-bit terms only");
-  h0 = __builtin_convertvector(vv, S2);
+  h0 = split2_lead<T>(vv);
   if constexpr (traits::num_terms >= 2) {
-    f32x2_t r = {0.f, 0.f};
-    if constexpr (std::is_same<S, _Float16>::value) {
-      static_assert(traits::num_terms == 2, "two-term fp16 split");
-      const float m0 = vv[0] * traits::scale, m1 = vv[1] * traits::scale;
-      const float neg_scale = -traits::scale;
-      asm("v_fma_mixlo_f16 %0, %1, %2, %3 op_sel:[0,0,0] op_sel_hi:[1,0,0]"
-          : "=v"(h1)
-          : "v"(h0), "s"(neg_scale), "v"(m0));
-      asm("v_fma_mixhi_f16 %0, %1, %2, %3 op_sel:[1,0,0] op_sel_hi:[1,0,0]"
-          : "+v"(h1)
-          : "v"(h0), "s"(neg_scale), "v"(m1));
-    } else {
-      r = vv - __builtin_convertvector(h0, f32x2_t);
-      if constexpr (traits::scale != 1.f)
-        r *= traits::scale;
-      h1 = __builtin_convertvector(r, S2);
-    }
+    const float p0 = split2_prep<T, 0>(vv[0], h0);
+    const float p1 = split2_prep<T, 1>(vv[1], h0);
+    h1 = split2_resid_hi<T>(split2_resid_lo<T>(h0, p0), h0, p0, p1);
     if constexpr (traits::num_terms >= 3)
-      h2 = __builtin_convertvector(r - __builtin_convertvector(h1, f32x2_t),
-                                   S2);
+      h2 = __builtin_convertvector(
+          f32x2_t{p0, p1} - __builtin_convertvector(h1, f32x2_t), S2);
   }
 }
 template <class T, class S = typename split_traits<T>::storage>

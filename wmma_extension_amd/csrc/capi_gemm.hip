@@ -235,12 +235,12 @@ constexpr PathRates kPacked[3] = {{8.9e-6, 0.31e-6, 2.0e-6, 5.0e12, 6.6e12},
 //    run on this path and on the estimated one of the other two (the
 //    reference harness's grid m = n = 512, 1024, k = 128 .. 16384, 256
 //    entries; single and batched products of other shapes, four policies): a
-//    k stage of a 256x128 tile takes 0.8 / 1.56 us (packed operands: 0.5 /
+//    k stage of a 256x128 tile takes 0.8 / 1.5 us (packed operands: 0.5 /
 //    1.0 us), a tile 6 us on top.
 constexpr PathRates kDirect[2] = {{6.0e-6, 0.40e-6, 3.0e-6, 5.0e12, 0.},
-                                  {6.0e-6, 0.78e-6, 3.0e-6, 5.0e12, 0.}};
+                                  {6.0e-6, 0.75e-6, 3.0e-6, 5.0e12, 0.}};
 // with K slices: the GEMM's time against the same kernel on packed operands
-constexpr double kDirectSliceRatio[2] = {1.5, 1.56};
+constexpr double kDirectSliceRatio[2] = {1.5, 1.5};
 // the single kernel's 64x64 tile against its 128x128 tile (1024^3: 41 -> 27 us)
 constexpr double kFusedSmallTileTime = 0.65; // whole tile, latency-bound sizes
 constexpr double kFusedSmallStage = 0.33, kFusedSmallTile = 0.5;

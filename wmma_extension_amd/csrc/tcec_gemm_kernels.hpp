@@ -57,6 +57,42 @@ __host__ __device__ constexpr int reads_due(const int count, const int span,
     r++;
   return r;
 }
+// MFMA of a step after which LDS read r of the next stage goes out when the A
+// fragments are recycled (GemmConfig::RECYCLE_A): the first `first_reads` (B
+// and A's last tile row, which have registers of their own) spread over the
+// first tile row's `row_mfma` MFMAs, the A fragments of tile row i right after
+// the last MFMA of that row.
+__host__ __device__ constexpr int recycled_read_slot(const int r,
+                                                     const int first_reads,
+                                                     const int row_mfma,
+                                                     const int terms) {
+  return r < first_reads ? (r * row_mfma) / first_reads
+                         : ((r - first_reads) / terms + 1) * row_mfma +
+                               2 * ((r - first_reads) % terms);
+}
+// DIRECT: number of producer micro-operations that have gone out once `n`
+// MFMAs of a step are out.  Micro-operations and LDS reads together are spread
+// evenly over the MFMAs: after every MFMA the micro-operations make up what
+// the reads due there leave of the common rate.
+__host__ __device__ constexpr int
+direct_uops_before(const int n, const bool recycle, const int nuop,
+                   const int nfrag, const int nmfma, const int span,
+                   const int first_reads, const int row_mfma, const int terms) {
+  int prev = 0;
+  for (int m = 1; m <= n; m++) {
+    int reads = 0; // issued after the MFMAs 0 .. m-1
+    if (recycle) {
+      for (int r = 0; r < nfrag; r++)
+        reads += recycled_read_slot(r, first_reads, row_mfma, terms) < m;
+    } else {
+      reads = m == nmfma ? nfrag : reads_due(m, span, nfrag);
+    }
+    int t = (m * (nuop + nfrag)) / nmfma - reads;
+    t = t < prev ? prev : t;
+    prev = t > nuop ? nuop : t;
+  }
+  return n >= nmfma ? nuop : prev;
+}
 
 // --------------------------------------------------------------------------
 // split_pack_kernel: X (fp32, element (r,k) at X[r*row_stride + k*k_stride])
@@ -635,19 +671,23 @@ __global__ void __launch_bounds__(WGM *WGN * 64)
   // of the requests above.  A lane's eight floats (four from each of the two
   // loads of a row block) stay in registers from the load to the split one
   // step later:
-  //   load_rb  : the lane's floats of row block g at the cursor's stage
-  //   split_rb : pair P of them -> one register of each term
-  //   write_rb : the terms as 8-byte halves of the 16-byte fragment positions
-  //              of the stage image in LDS, where the packed operands would
-  //              have been copied to
+  //   load_half  : the lane's four floats of half h (rows 8h .. 8h+7) of row
+  //                block g at the cursor's stage
+  //   split_step : one instruction of the split of a pair of them -> one
+  //                register of each term
+  //   write_half : the terms of a half as 8-byte halves of the 16-byte
+  //                fragment positions of the stage image in LDS, where the
+  //                packed operands would have been copied to
   using SplitTag = typename std::conditional<std::is_same<MT, _Float16>::value,
                                              mtk::wmma::half,
                                              mtk::wmma::bfloat16>::type;
   typedef MT s2_t __attribute__((ext_vector_type(2)));
   float raw[DIRECT ? RPW : 1][8];
-  unsigned term[2][4];
-  auto load_rb = [&](auto G) {
-    constexpr int g = decltype(G)::value;
+  unsigned term[2][2];
+  s2_t lead_h;     // a pair's leading terms and what its residual terms are
+  float prep_r[2]; // rounded from, between the instructions of its split
+  auto load_half = [&](auto G, auto H) {
+    constexpr int g = decltype(G)::value, h = decltype(H)::value;
     // 16-byte loads; the address need only be a float's (global memory is
     // accessed in unaligned mode), so any leading dimension and base work
     typedef f32x4 __attribute__((aligned(4))) f32x4_u;
@@ -655,27 +695,40 @@ __global__ void __launch_bounds__(WGM *WGN * 64)
     const auto *const p =
         reinterpret_cast<const __attribute__((address_space(1))) char *>(
             gsrc[g]);
-    // (the offsets are redefined in place so that each address is formed here,
+    // (the offset is redefined in place so that the address is formed here,
     // as the instruction's scalar base + 32-bit lane offset, and not hoisted
-    // into vector register pairs)
-    asm volatile("" : "+v"(voff[g][0]), "+v"(voff[g][1]));
-    const f32x4 lo = *reinterpret_cast<vec_ptr>(p + voff[g][0]);
-    const f32x4 hi = *reinterpret_cast<vec_ptr>(p + voff[g][1]);
+    // into a vector register pair)
+    asm volatile("" : "+v"(voff[g][h]));
+    const f32x4 v = *reinterpret_cast<vec_ptr>(p + voff[g][h]);
 #pragma unroll
-    for (int x = 0; x < 4; x++) {
-      raw[g][x] = lo[x];
-      raw[g][4 + x] = hi[x];
-    }
+    for (int x = 0; x < 4; x++)
+      raw[g][4 * h + x] = v[x];
   };
-  auto split_rb = [&](auto G, auto P) {
-    constexpr int g = decltype(G)::value, q = decltype(P)::value;
-    s2_t h0, h1, h2;
-    mtk::wmma::tcec::detail::split2<SplitTag>(
-        mtk::wmma::tcec::detail::f32x2_t{raw[g][2 * q], raw[g][2 * q + 1]}, h0,
-        h1, h2);
-    term[0][q] = __builtin_bit_cast(unsigned, h0);
-    if constexpr (TERMS >= 2)
-      term[1][q] = __builtin_bit_cast(unsigned, h1);
+  // instruction PH of the split of pair Q of row block G: 0 leading terms,
+  // 1 and 2 what the residuals of the pair's two values are rounded from,
+  // 3 and 4 the residual terms
+  auto split_step = [&](auto G, auto Q, auto PH) {
+    constexpr int g = decltype(G)::value, q = decltype(Q)::value,
+                  ph = decltype(PH)::value;
+    namespace sd = mtk::wmma::tcec::detail;
+    if constexpr (ph == 0) {
+      lead_h = sd::split2_lead<SplitTag>(
+          sd::f32x2_t{raw[g][2 * q], raw[g][2 * q + 1]});
+      term[0][q % 2] = __builtin_bit_cast(unsigned, lead_h);
+    } else if constexpr (TERMS >= 2 && ph == 1) {
+      prep_r[0] = sd::split2_prep<SplitTag, 0>(raw[g][2 * q], lead_h);
+    } else if constexpr (TERMS >= 2 && ph == 2) {
+      prep_r[1] = sd::split2_prep<SplitTag, 1>(raw[g][2 * q + 1], lead_h);
+    } else if constexpr (TERMS >= 2 && ph == 3) {
+      term[1][q % 2] = __builtin_bit_cast(
+          unsigned, sd::split2_resid_lo<SplitTag>(lead_h, prep_r[0]));
+    } else if constexpr (TERMS >= 2) {
+      term[1][q % 2] = __builtin_bit_cast(
+          unsigned,
+          sd::split2_resid_hi<SplitTag>(
+              __builtin_bit_cast(s2_t, term[1][q % 2]), lead_h, prep_r[0],
+              prep_r[1]));
+    }
   };
   // A lane's four values of a load are half of a fragment position (row r,
   // k group q = k/8 of the stage): position r + 16*q of the chunk, stored at
@@ -692,28 +745,33 @@ __global__ void __launch_bounds__(WGM *WGN * 64)
     const unsigned r = 8u * h + (lane >> 3), q = (lane & 7u) >> 1;
     woff[h] = 256u * q + 16u * (r ^ direct_swizzle(q)) + 8u * (lane & 1u);
   }
-  auto write_rb = [&](const int w_base, auto G) {
-    constexpr int g = decltype(G)::value;
+  auto write_half = [&](const int w_base, auto G, auto H) {
+    constexpr int g = decltype(G)::value, h = decltype(H)::value;
 #pragma unroll
     for (int t = 0; t < TERMS; t++)
-#pragma unroll
-      for (int h = 0; h < 2; h++)
-        *reinterpret_cast<u32x2 *>(lds_raw + w_base +
-                                   g * RB_STEP * CH_PER_RB * 1024 + t * 1024 +
-                                   woff[h]) =
-            u32x2{term[t][2 * h], term[t][2 * h + 1]};
+      *reinterpret_cast<u32x2 *>(lds_raw + w_base +
+                                 g * RB_STEP * CH_PER_RB * 1024 + t * 1024 +
+                                 woff[h]) = u32x2{term[t][0], term[t][1]};
   };
-  // micro-operation U of a step's RPW * 6 (per row block: four pairs to
-  // split, the writes, the loads of the stage after)
-  constexpr int NUOP = RPW * 6;
+  // A step's producer work, cut into micro-operations of one instruction each
+  // (a half's writes: one per term) so that no matrix instruction is followed
+  // by a burst of vector instructions.  The matrix pipe cannot run ahead of the
+  // wave's issue: five vector instructions after every fourth MFMA cost a bare
+  // stream of these MFMAs 15 %, the same five spread evenly nothing.  Per row
+  // block and half (the eight rows of one load): the five instructions of each
+  // of its two pairs, the writes of the half, the load of the same half of the
+  // stage after.
+  constexpr int UOPS_PER_HALF = 2 * 5 + 2;
+  constexpr int NUOP = RPW * 2 * UOPS_PER_HALF;
   auto direct_uop = [&](const int w_base, auto U) {
-    constexpr int u = decltype(U)::value, g = u / 6, o = u % 6;
-    if constexpr (o < 4)
-      split_rb(ic<g>{}, ic<o>{});
-    else if constexpr (o == 4)
-      write_rb(w_base, ic<g>{});
+    constexpr int u = decltype(U)::value, g = u / (2 * UOPS_PER_HALF),
+                  h = (u / UOPS_PER_HALF) % 2, o = u % UOPS_PER_HALF;
+    if constexpr (o < 10)
+      split_step(ic<g>{}, ic<2 * h + o / 5>{}, ic<o % 5>{});
+    else if constexpr (o == 10)
+      write_half(w_base, ic<g>{}, ic<h>{});
     else
-      load_rb(ic<g>{});
+      load_half(ic<g>{}, ic<h>{});
   };
 
   // In-place accumulate, written as inline assembly so that every accumulator
@@ -818,10 +876,7 @@ __global__ void __launch_bounds__(WGM *WGN * 64)
   constexpr int ROW_MFMA = NT_ * NPROD;
   constexpr int FIRST_READS = TERMS * (NT_ + 1);
   constexpr auto recycle_slot = [](const int r) constexpr {
-    return r < FIRST_READS
-               ? (r * ROW_MFMA) / FIRST_READS
-               : ((r - FIRST_READS) / TERMS + 1) * ROW_MFMA +
-                     2 * ((r - FIRST_READS) % TERMS);
+    return recycled_read_slot(r, FIRST_READS, ROW_MFMA, TERMS);
   };
 
   // One pipeline step: multiply the fragments of stage st (already in
@@ -902,9 +957,13 @@ __global__ void __launch_bounds__(WGM *WGN * 64)
         // split the stage after next (loaded during the last step) into the
         // buffer the current stage has left, load the stage after that: the
         // micro-operations spread evenly over the step
-        constexpr int ulo = (n * NUOP + NMFMA - 1) / NMFMA;
-        constexpr int uhi = ((n + 1) * NUOP + NMFMA - 1) / NMFMA;
-        static_for<ulo, (uhi < NUOP ? uhi : NUOP)>([&](auto U) {
+        constexpr int ulo =
+            direct_uops_before(n, RECYCLE, NUOP, NFRAG, NMFMA, SPAN,
+                               FIRST_READS, ROW_MFMA, TERMS);
+        constexpr int uhi =
+            direct_uops_before(n + 1, RECYCLE, NUOP, NFRAG, NMFMA, SPAN,
+                               FIRST_READS, ROW_MFMA, TERMS);
+        static_for<ulo, uhi>([&](auto U) {
           direct_uop(w_base, U);
           __builtin_amdgcn_sched_barrier(0);
         });
@@ -1024,7 +1083,10 @@ __global__ void __launch_bounds__(WGM *WGN * 64)
   if constexpr (DIRECT) {
     // stages 0 and 1 of the stream into the two LDS buffers, stage 2 into
     // the registers
-    static_for<0, RPW>([&](auto G) { load_rb(G); });
+    static_for<0, RPW>([&](auto G) {
+      load_half(G, ic<0>{});
+      load_half(G, ic<1>{});
+    });
     advance_request();
 #pragma unroll
     for (int s = 0; s < 2; s++) {
