@@ -660,6 +660,22 @@ int fused_dispatch(const int policy, const FusedArgs &f) {
 // matrices, K-heavy products).  It needs k contiguous in both operands, k a
 // multiple of 32 and at most two terms; same bits as the packed path.
 enum class Path { Fused, Packed, Direct };
+// the direct kernel's time without K slices: rounds of 256x128 tiles over the
+// compute units, and the bytes it moves
+struct DirectTimes {
+  double tiles, bytes;
+};
+inline DirectTimes direct_times(const int m, const int n, const int k,
+                                const int batch, const int terms) {
+  const fit::PathRates &d = fit::kDirect[terms - 1];
+  const double kt = static_cast<double>(ceil_div(k, 32));
+  const long long tiles256 = ceil_div(m, 256) * ceil_div(n, 128) * batch;
+  const double ab = (static_cast<double>(m) + n) * k * batch;
+  return {fit::kUnits256x128 *
+              static_cast<double>(ceil_div(tiles256, device_cus())) *
+              (kt * d.stage + d.tile),
+          (4.0 * m * n * batch + 4.0 * ab) / d.bytes_per_s};
+}
 constexpr int kPathFlags =
     WMMAE_FLAG_PATH_PACKED | WMMAE_FLAG_PATH_FUSED | WMMAE_FLAG_PATH_DIRECT;
 constexpr int kAllFlags = WMMAE_FLAG_RN_MAIN | kPathFlags;
@@ -739,14 +755,8 @@ inline Path choose_path(const int m, const int n, const int k, const int batch,
     best = Path::Fused;
   }
   if (direct_ok) {
-    const fit::PathRates &d = fit::kDirect[terms - 1];
-    const double t_direct =
-        d.launch +
-        std::max(fit::kUnits256x128 *
-                     static_cast<double>(ceil_div(tiles256, cus)) *
-                     (kt * d.stage + d.tile),
-                 (c_bytes + 4.0 * ab) / d.bytes_per_s);
-    if (t_direct < t_best)
+    const DirectTimes d = direct_times(m, n, k, batch, terms);
+    if (fit::kDirect[terms - 1].launch + std::max(d.tiles, d.bytes) < t_best)
       best = Path::Direct;
   }
   return best;
@@ -1046,8 +1056,12 @@ int sgemm_impl(const char transa, const char transb, const int m, const int n,
     g.stream = s;
     g.is_direct = true;
     g.direct = wmmae_gemm::DirectSource{A,    B,    a_ptrs,   b_ptrs,
-                                        a_rs, b_rs, stride_a, stride_b};
+                                        a_rs, b_rs, stride_a, stride_b, 0};
     plan_k_slices(g, ws, ws_bytes);
+    // staggered start for launches bound by their bytes (see the kernel)
+    const DirectTimes dt = direct_times(m, n, k, batch, p.terms);
+    if (g.splits <= 1 && batch >= 8 && dt.bytes > dt.tiles)
+      g.direct.stagger = 1;
     int st = gemm_dispatch(policy, 0, g);
     if (own && hipFreeAsync(ws, s) != hipSuccess && st == WMMAE_STATUS_SUCCESS)
       st = WMMAE_STATUS_RUNTIME_ERROR;
