@@ -77,6 +77,14 @@ def test_direct_path_k_slices(tc, orc, dev, policy):
     assert orc.max_rel_err(d.view(n, m).cpu().numpy().T, ref) < {0: 4e-6, 3: 2e-4}[policy]
 
 
+def test_direct_path_staggered_start(tc, dev):
+    """A launch bound by its bytes (many small matrices, two k stages a tile): the workgroups
+    of an XCD start a little apart; nothing but their timing changes."""
+    for policy in (0, 4):
+        (d, p), _, _, _ = _both(tc, dev, 256, 256, 64, 1024, policy)
+        assert torch.equal(d, p)
+
+
 def test_direct_path_pointer_arrays(tc, dev):
     """wmmae_tcec_sgemm_batched (device arrays of matrix pointers, test/tcec/batch_gemm.cu:433-443)
     with entries that are not 16-byte aligned."""
