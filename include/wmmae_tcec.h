@@ -74,7 +74,7 @@ typedef enum {
 #define WMMAE_FLAG_PATH_FUSED 4  /* the single kernel for small products */
 #define WMMAE_FLAG_PATH_DIRECT 8 /* the packed path's GEMM kernel splitting the
                                     fp32 operands itself: needs op(A) and op(B)
-                                    with k contiguous ('T','N'), k % 32 == 0, a
+                                    with k contiguous ('T','N'), k % 4 == 0, a
                                     policy of one or two terms, no RN_MAIN */
 
 /* Text for a wmmae_status value.  (No counterpart in the reference: its

@@ -77,6 +77,20 @@ def test_direct_path_k_slices(tc, orc, dev, policy):
     assert orc.max_rel_err(d.view(n, m).cpu().numpy().T, ref) < {0: 4e-6, 3: 2e-4}[policy]
 
 
+@pytest.mark.parametrize("policy", [0, 1, 3, 4])
+def test_direct_path_k_not_a_multiple_of_32(tc, orc, dev, policy):
+    """k a multiple of 4 only: the last stage of a row is shorter than 32 floats (one stage in
+    all, a few, many; K slices; rows that end at the allocation's last float)."""
+    for (m, n, k, batch) in ((256, 128, 4, 1), (300, 200, 36, 3), (520, 392, 1000, 5),
+                             (512, 384, 16388, 1), (1024, 1024, 100, 9)):
+        (d, p), A, B, _ = _both(tc, dev, m, n, k, batch, policy, seed=k)
+        assert torch.equal(d, p), (m, n, k, batch)
+    m, n, k = 300, 200, 36
+    (d, _), A, B, _ = _both(tc, dev, m, n, k, 1, policy, seed=1)
+    ref = orc.gemm_f64(A.view(m, k).cpu().numpy(), B.view(n, k).cpu().numpy().T)
+    assert orc.max_rel_err(d.view(n, m).cpu().numpy().T, ref) < {0: 4e-6, 1: 2e-3, 3: 2e-4, 4: 2e-2}[policy]
+
+
 def test_direct_path_staggered_start(tc, dev):
     """A launch bound by its bytes (many small matrices, two k stages a tile): the workgroups
     of an XCD start a little apart; nothing but their timing changes."""
@@ -132,7 +146,7 @@ def test_direct_path_turns_down_what_it_cannot_read(tc, dev):
     from wmma_extension_amd._lib import WmmaeError
     A = torch.zeros((64, 64), device=dev)
     C = torch.zeros((64, 64), device=dev)
-    for kwargs in (dict(transa="N"), dict(k=48), dict(policy=2), dict(flags=DIRECT | 1)):
+    for kwargs in (dict(transa="N"), dict(k=50), dict(policy=2), dict(flags=DIRECT | 1)):
         a = dict(transa="T", k=64, policy=0, flags=DIRECT)
         a.update(kwargs)
         with pytest.raises(WmmaeError) as e:

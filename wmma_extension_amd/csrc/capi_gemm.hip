@@ -241,6 +241,9 @@ constexpr PathRates kDirect[2] = {{6.0e-6, 0.40e-6, 3.0e-6, 5.0e12, 0.},
                                   {6.0e-6, 0.75e-6, 3.0e-6, 5.0e12, 0.}};
 // with K slices: the GEMM's time against the same kernel on packed operands
 constexpr double kDirectSliceRatio[2] = {1.5, 1.5};
+// k % 32 != 0: the kernel variant that reads a shorter last stage (1024^2 x 1000
+// against x 1024, batch 256: 301 against 336 TFLOPS, of which 2.4 % are the k)
+constexpr double kDirectTailStage = 1.09;
 // the single kernel's 64x64 tile against its 128x128 tile (1024^3: 41 -> 27 us)
 constexpr double kFusedSmallTileTime = 0.65; // whole tile, latency-bound sizes
 constexpr double kFusedSmallStage = 0.33, kFusedSmallTile = 0.5;
@@ -376,7 +379,7 @@ constexpr int ring_depth(const int bm, const int bn, const int terms) {
 }
 
 template <class MT, int TERMS, int BM, int BN, int WGM, int WGN, bool RN,
-          bool DIRECT = false>
+          int DIRECT = 0>
 int launch_gemm(const GemmArgs &g) {
   constexpr int NSTAGE = DIRECT ? 2 : ring_depth(BM, BN, TERMS);
   using Cfg =
@@ -513,8 +516,10 @@ template <class MT, int TERMS, bool RN> int gemm_by_size(const GemmArgs &g) {
   const long long mid =
       ceil_div(g.m, 128) * ceil_div(g.n, 128) * g.batch * z;
   if constexpr (TERMS <= 2 && !RN) {
+    // (k a multiple of 32, or the variant with a shorter last stage)
     if (g.is_direct)
-      return launch_gemm<MT, TERMS, 256, 128, 2, 2, RN, true>(g);
+      return g.k % 32 == 0 ? launch_gemm<MT, TERMS, 256, 128, 2, 2, RN, 1>(g)
+                           : launch_gemm<MT, TERMS, 256, 128, 2, 2, RN, 2>(g);
   }
   // (not with the separate fp32 adds of RN: their temporaries do not fit the
   // register file next to the large tile's accumulators)
@@ -658,7 +663,7 @@ int fused_dispatch(const int policy, const FusedArgs &f) {
 // No packed copy and no split pass, at 1.5 times the time per k stage; it wins
 // where an operand element is used by few tiles (batches of small and medium
 // matrices, K-heavy products).  It needs k contiguous in both operands, k a
-// multiple of 32 and at most two terms; same bits as the packed path.
+// multiple of 4 and at most two terms; same bits as the packed path.
 enum class Path { Fused, Packed, Direct };
 // the direct kernel's time without K slices: rounds of 256x128 tiles over the
 // compute units, and the bytes it moves
@@ -671,9 +676,11 @@ inline DirectTimes direct_times(const int m, const int n, const int k,
   const double kt = static_cast<double>(ceil_div(k, 32));
   const long long tiles256 = ceil_div(m, 256) * ceil_div(n, 128) * batch;
   const double ab = (static_cast<double>(m) + n) * k * batch;
+  // (the variant for k % 32 != 0 spends one more instruction per load)
+  const double stage = d.stage * (k % 32 == 0 ? 1.0 : fit::kDirectTailStage);
   return {fit::kUnits256x128 *
               static_cast<double>(ceil_div(tiles256, device_cus())) *
-              (kt * d.stage + d.tile),
+              (kt * stage + d.tile),
           (4.0 * m * n * batch + 4.0 * ab) / d.bytes_per_s};
 }
 constexpr int kPathFlags =
@@ -764,7 +771,7 @@ inline Path choose_path(const int m, const int n, const int k, const int batch,
 // what the direct kernel needs of a product (the operands' k strides are 1)
 inline bool direct_possible(const int k, const int terms, const int flags,
                             const long long a_rs, const long long b_rs) {
-  return k > 0 && k % 32 == 0 && terms <= 2 &&
+  return k > 0 && k % 4 == 0 && terms <= 2 &&
          (flags & WMMAE_FLAG_RN_MAIN) == 0 && a_rs < (1 << 24) &&
          b_rs < (1 << 24);
 }
@@ -1056,7 +1063,7 @@ int sgemm_impl(const char transa, const char transb, const int m, const int n,
     g.stream = s;
     g.is_direct = true;
     g.direct = wmmae_gemm::DirectSource{A,    B,    a_ptrs,   b_ptrs,
-                                        a_rs, b_rs, stride_a, stride_b, 0};
+                                        a_rs, b_rs, stride_a, stride_b, 0, k};
     plan_k_slices(g, ws, ws_bytes);
     // staggered start for launches bound by their bytes (see the kernel)
     const DirectTimes dt = direct_times(m, n, k, batch, p.terms);

@@ -380,10 +380,13 @@ struct DirectSource {
   // > 0: the workgroups of an XCD start in 32 phases, this many periods of 512
   // cycles apart (see the kernel's prologue)
   int stagger;
+  // floats per row (k); the DIRECT == 2 variant reads a last stage of fewer
+  // than 32
+  int k;
 };
 
 template <class MT, int TERMS, int BM, int BN, int WGM, int WGN, int NSTAGE,
-          bool RN_MAIN, bool DIRECT = false>
+          bool RN_MAIN, int DIRECT = 0>
 struct GemmConfig {
   static constexpr int NW = WGM * WGN;
   static constexpr int NTHREADS = NW * 64;
@@ -412,7 +415,7 @@ struct GemmConfig {
 };
 
 template <class MT, int TERMS, int BM, int BN, int WGM, int WGN, int NSTAGE,
-          bool RN_MAIN, bool DIRECT = false>
+          bool RN_MAIN, int DIRECT = 0>
 __global__ void __launch_bounds__(WGM *WGN * 64)
     tcec_gemm_kernel(const u32x4 *__restrict__ Ap, const u32x4 *__restrict__ Bp,
                      float *__restrict__ C, const int M, const int N,
@@ -565,6 +568,24 @@ __global__ void __launch_bounds__(WGM *WGN * 64)
   unsigned voff[DIRECT ? RPW : 1][2];
   unsigned lane_off = lane * 16u;
   int req_item = 0, req_st = 0, req_stages = 0;
+  // DIRECT == 2 (k a multiple of 4, not of 32): floats from the start of the
+  // cursor's stage to the end of the rows, the same for the stage whose values
+  // wait in registers, and what a lane subtracts from its offset so that it
+  // reads inside the rows.  A lane's four floats are all inside a row or all
+  // outside; in a row's last, shorter stage a lane outside reads the stage's
+  // first four floats instead and its values are replaced by zeros before the
+  // split: the packed operands are padded with zeros, so the results are the
+  // same bits.  (Moving the offsets themselves when the cursor enters and
+  // leaves such a stage, instead of one subtraction per load, was slower:
+  // 1024^2 x 1000 x 256 1.96 against 1.79 ms.)
+  constexpr bool TAIL = DIRECT == 2;
+  int req_left = 0, raw_left = 0;
+  unsigned tail_off = 0;
+  auto set_tail_off = [&]() {
+    if constexpr (TAIL)
+      tail_off =
+          4 * static_cast<int>(lane & 7u) < req_left ? 0u : 16u * (lane & 7u);
+  };
   auto set_sources = [&](const int i) {
     const Item it = decode(i);
     req_stages = stages_of(it);
@@ -572,6 +593,10 @@ __global__ void __launch_bounds__(WGM *WGN * 64)
         partial != nullptr || it.tail >= 0
             ? static_cast<long long>(it.z) * slice_stages(it)
             : 0;
+    if constexpr (TAIL) {
+      req_left = ds.k - static_cast<int>(first_stage) * 32;
+      set_tail_off();
+    }
     if constexpr (DIRECT) {
       // the pointer arrays are read with scalar loads (constant address space)
       typedef const float *const __attribute__((address_space(4))) *ptr_array_t;
@@ -621,12 +646,18 @@ __global__ void __launch_bounds__(WGM *WGN * 64)
   // few redundant requests keep the in-flight count constant, so one
   // s_waitcnt immediate serves the whole loop
   auto advance_request = [&]() {
+    if constexpr (TAIL)
+      raw_left = req_left; // of the stage just loaded
     if (req_st + 1 < req_stages) {
       req_st++;
 #pragma unroll
       for (int g = 0; g < RPW; g++) {
         gsrc[g] += STAGE_BYTES;
         asm volatile("" : "+s"(gsrc[g]));
+      }
+      if constexpr (TAIL) {
+        req_left -= 32;
+        set_tail_off();
       }
     } else if (req_item + 1 < n_my) {
       req_item++;
@@ -702,7 +733,8 @@ __global__ void __launch_bounds__(WGM *WGN * 64)
     // as the instruction's scalar base + 32-bit lane offset, and not hoisted
     // into a vector register pair)
     asm volatile("" : "+v"(voff[g][h]));
-    const f32x4 v = *reinterpret_cast<vec_ptr>(p + voff[g][h]);
+    const f32x4 v = *reinterpret_cast<vec_ptr>(
+        p + (TAIL ? voff[g][h] - tail_off : voff[g][h]));
 #pragma unroll
     for (int x = 0; x < 4; x++)
       raw[g][4 * h + x] = v[x];
@@ -764,6 +796,22 @@ __global__ void __launch_bounds__(WGM *WGN * 64)
   // block and half (the eight rows of one load): the five instructions of each
   // of its two pairs, the writes of the half, the load of the same half of the
   // stage after.
+  // TAIL: when the stage waiting in registers is a row's last, shorter one,
+  // zeros for the lanes past the end, before any of it is split (one branch per
+  // step; the rare side waits for all of the stage's loads at once)
+  auto zero_tail = [&]() {
+    if constexpr (TAIL) {
+      if (__builtin_expect(raw_left < 32, 0)) {
+        if (4 * static_cast<int>(lane & 7u) >= raw_left) {
+#pragma unroll
+          for (int g = 0; g < RPW; g++)
+#pragma unroll
+            for (int x = 0; x < 8; x++)
+              raw[g][x] = 0.f;
+        }
+      }
+    }
+  };
   constexpr int UOPS_PER_HALF = 2 * 5 + 2;
   constexpr int NUOP = RPW * 2 * UOPS_PER_HALF;
   auto direct_uop = [&](const int w_base, auto U) {
@@ -913,6 +961,7 @@ __global__ void __launch_bounds__(WGM *WGN * 64)
                      : "memory");
     }
     asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");
+    zero_tail();
 
     static_for<0, NMFMA>([&](auto N_) {
       constexpr int n = decltype(N_)::value;
@@ -1108,6 +1157,7 @@ __global__ void __launch_bounds__(WGM *WGN * 64)
     advance_request();
 #pragma unroll
     for (int s = 0; s < 2; s++) {
+      zero_tail();
       static_for<0, NUOP>([&](auto U) { direct_uop(wave_base(s), U); });
       advance_request();
     }
