@@ -120,7 +120,8 @@ int wmmae_tcec_sgemm_workspace_bytes(int m, int n, int k, int batch, int policy,
  * 2 packed operands and K slices (when the workspace has room for them),
  * 3 the packed path's GEMM kernel loading and splitting the fp32 operands
  * itself (no packed operands), 4 the same with K slices.  3 and 4 assume
- * k contiguous in both operands ('T','N'); other layouts take 1 and 2.
+ * k contiguous in both operands ('T','N') and need k % 4 == 0; other layouts
+ * take 1 and 2.
  * The answer assumes operands the single kernel can read 16 bytes at a time
  * (k the contiguous direction, k and the leading dimensions multiples of 4,
  * 16-byte aligned bases); other operands with k > 96 take path 1 where this
