@@ -788,14 +788,6 @@ __global__ void __launch_bounds__(WGM *WGN * 64)
                                  g * RB_STEP * CH_PER_RB * 1024 + t * 1024 +
                                  woff[h]) = u32x2{term[t][0], term[t][1]};
   };
-  // A step's producer work, cut into micro-operations of one instruction each
-  // (a half's writes: one per term) so that no matrix instruction is followed
-  // by a burst of vector instructions.  The matrix pipe cannot run ahead of the
-  // wave's issue: five vector instructions after every fourth MFMA cost a bare
-  // stream of these MFMAs 15 %, the same five spread evenly nothing.  Per row
-  // block and half (the eight rows of one load): the five instructions of each
-  // of its two pairs, the writes of the half, the load of the same half of the
-  // stage after.
   // TAIL: when the stage waiting in registers is a row's last, shorter one,
   // zeros for the lanes past the end, before any of it is split (one branch per
   // step; the rare side waits for all of the stage's loads at once)
@@ -812,6 +804,14 @@ __global__ void __launch_bounds__(WGM *WGN * 64)
       }
     }
   };
+  // A step's producer work, cut into micro-operations of one instruction each
+  // (a half's writes: one per term) so that no matrix instruction is followed
+  // by a burst of vector instructions.  The matrix pipe cannot run ahead of the
+  // wave's issue: five vector instructions after every fourth MFMA cost a bare
+  // stream of these MFMAs 15 %, the same five spread evenly nothing.  Per row
+  // block and half (the eight rows of one load): the five instructions of each
+  // of its two pairs, the writes of the half, the load of the same half of the
+  // stage after.
   constexpr int UOPS_PER_HALF = 2 * 5 + 2;
   constexpr int NUOP = RPW * 2 * UOPS_PER_HALF;
   auto direct_uop = [&](const int w_base, auto U) {
@@ -1015,6 +1015,9 @@ __global__ void __launch_bounds__(WGM *WGN * 64)
         constexpr int uhi =
             direct_uops_before(n + 1, RECYCLE, NUOP, NFRAG, NMFMA, SPAN,
                                FIRST_READS, ROW_MFMA, TERMS);
+        static_assert(ulo <= uhi && uhi <= NUOP &&
+                          (n + 1 < NMFMA || uhi == NUOP),
+                      "every micro-operation of a step is issued once");
         static_for<ulo, uhi>([&](auto U) {
           direct_uop(w_base, U);
           __builtin_amdgcn_sched_barrier(0);
