@@ -74,7 +74,7 @@ typedef enum {
 #define WMMAE_FLAG_PATH_FUSED 4  /* the single kernel for small products */
 #define WMMAE_FLAG_PATH_DIRECT 8 /* the packed path's GEMM kernel splitting the
                                     fp32 operands itself: needs op(A) and op(B)
-                                    with k contiguous ('T','N'), k % 4 == 0, a
+                                    with k contiguous ('T','N'), k >= 4, a
                                     policy of one or two terms, no RN_MAIN */
 
 /* Text for a wmmae_status value.  (No counterpart in the reference: its
@@ -120,7 +120,7 @@ int wmmae_tcec_sgemm_workspace_bytes(int m, int n, int k, int batch, int policy,
  * 2 packed operands and K slices (when the workspace has room for them),
  * 3 the packed path's GEMM kernel loading and splitting the fp32 operands
  * itself (no packed operands), 4 the same with K slices.  3 and 4 assume
- * k contiguous in both operands ('T','N') and need k % 4 == 0; other layouts
+ * k contiguous in both operands ('T','N') and need k >= 4; other layouts
  * take 1 and 2.
  * The answer assumes operands the single kernel can read 16 bytes at a time
  * (k the contiguous direction, k and the leading dimensions multiples of 4,

@@ -78,7 +78,7 @@ def test_sgemm_argument_validation(h):
     assert _sgemm(h, policy=7) == -1
     assert _sgemm(h, flags=16) == -1
     assert _sgemm(h, flags=2 | 8) == -1         # at most one path flag
-    assert _sgemm(h, flags=8, k=50, lda=50, ldb=50) == -4    # direct path: k % 4 == 0
+    assert _sgemm(h, flags=8, k=3, lda=3, ldb=3) == -4    # direct path: k >= 4
     assert _sgemm(h, flags=8, ta=b"N") == -4               # ... and k contiguous
     assert _sgemm(h, flags=8 | 1) == -4                      # ... and no RN_MAIN
     assert _sgemm(h, flags=8, policy=2) == -4                # ... and at most two terms

@@ -79,10 +79,14 @@ def test_direct_path_k_slices(tc, orc, dev, policy):
 
 @pytest.mark.parametrize("policy", [0, 1, 3, 4])
 def test_direct_path_k_not_a_multiple_of_32(tc, orc, dev, policy):
-    """k a multiple of 4 only: the last stage of a row is shorter than 32 floats (one stage in
-    all, a few, many; K slices; rows that end at the allocation's last float)."""
+    """Any k from 4 on: the last stage of a row is shorter than 32 floats (one stage in all, a
+    few, many; K slices; rows that end one to three floats into their last stage, or in the
+    middle of a lane's four; rows that end at the allocation's last float)."""
     for (m, n, k, batch) in ((256, 128, 4, 1), (300, 200, 36, 3), (520, 392, 1000, 5),
-                             (512, 384, 16388, 1), (1024, 1024, 100, 9)):
+                             (512, 384, 16388, 1), (1024, 1024, 100, 9), (256, 128, 5, 2),
+                             (300, 200, 33, 3), (300, 200, 34, 1), (300, 200, 35, 2),
+                             (520, 392, 1001, 5), (512, 384, 16387, 1), (384, 256, 31, 4),
+                             (260, 130, 62, 3), (512, 512, 999, 16)):
         (d, p), A, B, _ = _both(tc, dev, m, n, k, batch, policy, seed=k)
         assert torch.equal(d, p), (m, n, k, batch)
     m, n, k = 300, 200, 36
@@ -146,7 +150,7 @@ def test_direct_path_turns_down_what_it_cannot_read(tc, dev):
     from wmma_extension_amd._lib import WmmaeError
     A = torch.zeros((64, 64), device=dev)
     C = torch.zeros((64, 64), device=dev)
-    for kwargs in (dict(transa="N"), dict(k=50), dict(policy=2), dict(flags=DIRECT | 1)):
+    for kwargs in (dict(transa="N"), dict(k=3), dict(policy=2), dict(flags=DIRECT | 1)):
         a = dict(transa="T", k=64, policy=0, flags=DIRECT)
         a.update(kwargs)
         with pytest.raises(WmmaeError) as e:

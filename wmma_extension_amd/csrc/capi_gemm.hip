@@ -663,7 +663,7 @@ int fused_dispatch(const int policy, const FusedArgs &f) {
 // No packed copy and no split pass, at 1.5 times the time per k stage; it wins
 // where an operand element is used by few tiles (batches of small and medium
 // matrices, K-heavy products).  It needs k contiguous in both operands, k a
-// multiple of 4 and at most two terms; same bits as the packed path.
+// least 4 and at most two terms; same bits as the packed path.
 enum class Path { Fused, Packed, Direct };
 // the direct kernel's time without K slices: rounds of 256x128 tiles over the
 // compute units, and the bytes it moves
@@ -771,7 +771,7 @@ inline Path choose_path(const int m, const int n, const int k, const int batch,
 // what the direct kernel needs of a product (the operands' k strides are 1)
 inline bool direct_possible(const int k, const int terms, const int flags,
                             const long long a_rs, const long long b_rs) {
-  return k > 0 && k % 4 == 0 && terms <= 2 &&
+  return k >= 4 && terms <= 2 &&
          (flags & WMMAE_FLAG_RN_MAIN) == 0 && a_rs < (1 << 24) &&
          b_rs < (1 << 24);
 }

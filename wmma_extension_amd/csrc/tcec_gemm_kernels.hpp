@@ -568,23 +568,27 @@ __global__ void __launch_bounds__(WGM *WGN * 64)
   unsigned voff[DIRECT ? RPW : 1][2];
   unsigned lane_off = lane * 16u;
   int req_item = 0, req_st = 0, req_stages = 0;
-  // DIRECT == 2 (k a multiple of 4, not of 32): floats from the start of the
+  // DIRECT == 2 (k not a multiple of 32, k >= 4): floats from the start of the
   // cursor's stage to the end of the rows, the same for the stage whose values
   // wait in registers, and what a lane subtracts from its offset so that it
-  // reads inside the rows.  A lane's four floats are all inside a row or all
-  // outside; in a row's last, shorter stage a lane outside reads the stage's
-  // first four floats instead and its values are replaced by zeros before the
-  // split: the packed operands are padded with zeros, so the results are the
-  // same bits.  (Moving the offsets themselves when the cursor enters and
-  // leaves such a stage, instead of one subtraction per load, was slower:
-  // 1024^2 x 1000 x 256 1.96 against 1.79 ms.)
+  // reads inside the rows.  In a row's last, shorter stage a lane whose four
+  // floats would end past the row reads the row's last four floats instead
+  // (`tail_shift` floats further back); before the split its values are moved
+  // up by that shift and followed by zeros (zero_tail below).  The packed
+  // operands are padded with zeros, so the results are the same bits.  (Moving
+  // the offsets themselves when the cursor enters and leaves such a stage,
+  // instead of one subtraction per load, was slower: 1024^2 x 1000 x 256 1.96
+  // against 1.79 ms.)
   constexpr bool TAIL = DIRECT == 2;
   int req_left = 0, raw_left = 0;
   unsigned tail_off = 0;
+  auto tail_shift = [&](const int left) {
+    const int s = 4 * static_cast<int>(lane & 7u) + 4 - left;
+    return s > 0 ? s : 0;
+  };
   auto set_tail_off = [&]() {
     if constexpr (TAIL)
-      tail_off =
-          4 * static_cast<int>(lane & 7u) < req_left ? 0u : 16u * (lane & 7u);
+      tail_off = 4u * static_cast<unsigned>(tail_shift(req_left));
   };
   auto set_sources = [&](const int i) {
     const Item it = decode(i);
@@ -614,14 +618,18 @@ __global__ void __launch_bounds__(WGM *WGN * 64)
         int row0 = is_a ? it.tm * BM + 16 * r : it.tn * BN + 16 * (r - RBM);
         row0 = row0 < last ? row0 : last;
         const long long ld = is_a ? ds.lda : ds.ldb;
+        // (TAIL: base and offsets biased by four floats, so that a lane that
+        // reads up to three floats before the stage's start - rows that end
+        // one to three floats into their last stage - keeps an offset >= 0)
         gsrc[g] = reinterpret_cast<unsigned long long>(
-            (is_a ? Ab : Bb) + row0 * ld + first_stage * 32);
+            (is_a ? Ab : Bb) + row0 * ld + first_stage * 32 - (TAIL ? 4 : 0));
         asm volatile("" : "+s"(gsrc[g]));
 #pragma unroll
         for (int h = 0; h < 2; h++) {
           int mine = row0 + 8 * h + static_cast<int>(lane >> 3);
           mine = (mine < last ? mine : last) - row0;
-          voff[g][h] = static_cast<unsigned>(mine * ld) * 4u + 16u * (lane & 7u);
+          voff[g][h] = static_cast<unsigned>(mine * ld) * 4u +
+                       16u * (lane & 7u) + (TAIL ? 16u : 0u);
         }
       }
       return;
@@ -788,18 +796,27 @@ __global__ void __launch_bounds__(WGM *WGN * 64)
                                  g * RB_STEP * CH_PER_RB * 1024 + t * 1024 +
                                  woff[h]) = u32x2{term[t][0], term[t][1]};
   };
-  // TAIL: when the stage waiting in registers is a row's last, shorter one,
-  // zeros for the lanes past the end, before any of it is split (one branch per
-  // step; the rare side waits for all of the stage's loads at once)
+  // TAIL: when the stage waiting in registers is a row's last, shorter one, the
+  // lanes that read further back take their own floats from what they read
+  // (value x is the one read at x + shift) and zeros past the row's end, before
+  // any of the stage is split (one branch per step; the rare side waits for all
+  // of the stage's loads at once)
   auto zero_tail = [&]() {
     if constexpr (TAIL) {
       if (__builtin_expect(raw_left < 32, 0)) {
-        if (4 * static_cast<int>(lane & 7u) >= raw_left) {
+        const int shift = tail_shift(raw_left);
+        if (shift > 0) {
 #pragma unroll
           for (int g = 0; g < RPW; g++)
 #pragma unroll
-            for (int x = 0; x < 8; x++)
-              raw[g][x] = 0.f;
+            for (int h = 0; h < 2; h++) {
+              const float v0 = raw[g][4 * h], v1 = raw[g][4 * h + 1],
+                          v2 = raw[g][4 * h + 2], v3 = raw[g][4 * h + 3];
+              raw[g][4 * h] = shift == 1 ? v1 : shift == 2 ? v2 : shift == 3 ? v3 : 0.f;
+              raw[g][4 * h + 1] = shift == 1 ? v2 : shift == 2 ? v3 : 0.f;
+              raw[g][4 * h + 2] = shift == 1 ? v3 : 0.f;
+              raw[g][4 * h + 3] = 0.f;
+            }
         }
       }
     }
