@@ -73,6 +73,10 @@ def test_direct_path_k_slices(tc, orc, dev, policy):
     assert torch.equal(d, p)
     (d2, _), _, _, _ = _both(tc, dev, m, n, k, 1, policy, workspace=False)
     assert torch.equal(d2, d)
+    (d3, p3), _, _, _ = _both(tc, dev, m, n, k + 5, 1, policy)          # a shorter last stage
+    assert torch.equal(d3, p3)
+    (d4, _), _, _, _ = _both(tc, dev, m, n, k + 5, 1, policy, workspace=False)
+    assert torch.equal(d4, d3)
     ref = orc.gemm_f64(A.view(m, k).cpu().numpy(), B.view(n, k).cpu().numpy().T)
     assert orc.max_rel_err(d.view(n, m).cpu().numpy().T, ref) < {0: 4e-6, 3: 2e-4}[policy]
 
@@ -103,10 +107,11 @@ def test_direct_path_staggered_start(tc, dev):
         assert torch.equal(d, p)
 
 
-def test_direct_path_pointer_arrays(tc, dev):
+@pytest.mark.parametrize("k", [128, 100, 37])
+def test_direct_path_pointer_arrays(tc, dev, k):
     """wmmae_tcec_sgemm_batched (device arrays of matrix pointers, test/tcec/batch_gemm.cu:433-443)
-    with entries that are not 16-byte aligned."""
-    m, n, k, batch = 384, 256, 128, 10
+    with entries that are not 16-byte aligned; whole stages and a shorter last one."""
+    m, n, batch = 384, 256, 10
     A = _uniform((batch, m * k + 3), 21, dev)
     B = _uniform((batch, n * k + 3), 22, dev)
     outs = []
