@@ -494,7 +494,9 @@ def main():
                          "when the matrix cores are not power limited; not a valid benchmark value)")
     ap.add_argument("--clock-trace", action="store_true",
                     help="sample the shader clock on a second stream during the timed region and add "
-                         "its statistics to the JSON line (the matrix cores are power limited)")
+                         "its statistics to the JSON line (the matrix cores are power limited); the sampling "
+                         "wave holds one SIMD, which a launch of one persistent workgroup per compute unit "
+                         "(c5a, c5b) pays for with up to twice its time: not a benchmark value there")
     ap.add_argument("--calibrate", action="store_true",
                     help="after the timed region run one 1 GiB read + 1 GiB write elementwise kernel "
                          "(the known-size copy that rocprofv3 FETCH_SIZE / WRITE_SIZE are scaled with)")
