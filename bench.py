@@ -180,9 +180,13 @@ def calibration_copy(torch, dev):
     del src, dst
 
 
-def bench_primitives(args, torch, tcec, dev, w):
-    """Workload c2: the fragment-primitive kernel over a stream of tiles (HBM bound)."""
+def bench_primitives(args, torch, tcec, dev, w, steps=None, warmup=None, cpu=None):
+    """Workload c2: the fragment-primitive kernel over a stream of tiles (HBM bound).
+    Returns the JSON line's fields."""
     import ctypes
+    steps = args.steps if steps is None else steps
+    warmup = args.warmup if warmup is None else warmup
+    cpu = (not args.no_cpu) if cpu is None else cpu
     from wmma_extension_amd import _lib
     T = w["tiles"]
     g = torch.Generator(device=dev)
@@ -196,27 +200,27 @@ def bench_primitives(args, torch, tcec, dev, w):
     def step():
         st = h.wmmae_primitive_tiles(ctypes.c_void_p(tiles.data_ptr()), T, *ptrs, stream)
         assert st == 0
-    for _ in range(args.warmup):
+    for _ in range(warmup):
         step()
     torch.cuda.synchronize()
     e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
     t0 = time.perf_counter()
     e0.record()
-    for _ in range(args.steps):
+    for _ in range(steps):
         step()
     e1.record()
     torch.cuda.synchronize()
     elapsed = time.perf_counter() - t0
     if args.calibrate:
         calibration_copy(torch, dev)
-    kernel_ms = e0.elapsed_time(e1) / args.steps
+    kernel_ms = e0.elapsed_time(e1) / steps
     # per tile: 1024 B fp32 in, 4 x 512 B fp16 fragment dumps, 1024 B accumulator, 2 x 64 B vectors
     nbytes = T * (1024 + 4 * 512 + 1024 + 128)
     gbs = nbytes / (kernel_ms * 1e-3) / 1e9
     res = {
         "metric": "fragment-primitive tile stream, algorithmic GB/s", "value": round(gbs, 1), "unit": "GB/s",
-        "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
-        "ms_per_step": round(elapsed / args.steps * 1e3, 4), "higher_is_better": True, "scaling": "weak",
+        "n_gpus": 1, "steps": steps, "warmup": warmup,
+        "ms_per_step": round(elapsed / steps * 1e3, 4), "higher_is_better": True, "scaling": "weak",
         "vs_baseline": None, "dtype": "f16", "data": "synthetic",
         "config": {"workload": f"c2: {w['desc']}", "tiles": T},
         "roofline": {"bound": "hbm", "achieved": round(gbs, 1), "peak": PEAK_HBM_GBS, "unit": "GB/s",
@@ -227,7 +231,7 @@ def bench_primitives(args, torch, tcec, dev, w):
         "tiles_per_s": round(T / (kernel_ms * 1e-3), 1),
         "cpu_baseline": None,
     }
-    if not args.no_cpu:
+    if cpu:
         # the oracle's layout tables applied with numpy to a sample of the tiles
         import numpy as np
         from oracle import oracle as orc
@@ -244,7 +248,8 @@ def bench_primitives(args, torch, tcec, dev, w):
         res["cpu_baseline"] = {"value": round(sample * (1024 + 4 * 512 + 1024 + 128) / dt / 1e9, 3), "unit": "GB/s",
                                "cores": 1, "kind": "port",
                                "sample": f"oracle layout tables applied with numpy to {sample} tiles, {dt:.2f} s"}
-    print(json.dumps(res))
+    del tiles, out
+    return res
 
 
 def accuracy_block(torch, tcec, orc, A, Bt, Ct, rows):
@@ -475,6 +480,83 @@ def bench_api_gemm(torch, tcec, dev, n=4096, steps=100, warmup=10):
             "mfma_frac": round(3 * tf / PEAK_MFMA_TFLOPS, 4)}
 
 
+# Pinned shapes for the guard of the fitted path / tile / slice choices: (m, n, k, entries,
+# policy).  The reference harness's grid (test/tcec/batch_gemm.cu:655-664: m = n in {512, 1024},
+# k = 128 .. 16384, 256 entries) at its corners, the baseline workloads, ragged and skinny shapes.
+PATHCHECK_SHAPES = [
+    (512, 512, 128, 256, "F16_EC"), (512, 512, 1024, 256, "F16_EC"),
+    (1024, 1024, 128, 256, "F16_EC"), (1024, 1024, 4096, 256, "F16_EC"),
+    (4096, 4096, 4096, 1, "F16_EC"), (256, 256, 256, 1024, "F16_EC"), (1024, 1024, 262144, 1, "F16_EC"),
+    (1000, 900, 50000, 2, "F16_EC"), (777, 1333, 515, 7, "F16_EC"),
+    (48, 832, 1376, 40, "F16_EC"), (4096, 64, 4096, 1, "F16_EC"),
+    (2048, 2048, 2048, 1, "BF16X3_EC"), (1024, 1024, 1024, 1, "BF16X3_EC"), (384, 384, 384, 100, "BF16X3_EC"),
+]
+PATH_NAMES = {0: "chosen", 2: "packed", 4: "fused", 8: "direct"}
+
+
+def bench_pathcheck(torch, tcec, dev, rounds=3):
+    """Every pinned shape as one whole library call (workspace resident) on the path the time
+    estimates choose and on every path forced; the variants of a shape are timed in alternation,
+    the fastest round of each counts.  ratio = chosen / fastest (>= 1 by construction: the chosen
+    call is one of the candidates)."""
+    from wmma_extension_amd._lib import WmmaeError
+    rows, worst = [], 1.0
+    for (m, n, k, batch, pol) in PATHCHECK_SHAPES:
+        policy = tcec.Policy[pol]
+        g = torch.Generator(device=dev)
+        g.manual_seed(0x5EED + 6)
+        A = torch.randn((batch, m, k), generator=g, device=dev, dtype=torch.float32)
+        Bt = torch.randn((batch, n, k), generator=g, device=dev, dtype=torch.float32)
+        Ct = torch.empty((batch, n, m), dtype=torch.float32, device=dev)
+        ws_bytes = tcec.workspace_bytes(m, n, k, batch, policy)
+        ws = torch.empty(ws_bytes, dtype=torch.uint8, device=dev) if ws_bytes else None
+
+        def call(flags):
+            tcec.sgemm_strided_batched("T", "N", m, n, k, 1.0, A, k, m * k, Bt, k, n * k, 0.0,
+                                       Ct, m, n * m, batch, policy, flags, ws)
+        variants, reps = [], {}
+        for flags in (0, 2, 4, 8):
+            try:
+                call(flags)                                  # also the warm-up
+            except WmmaeError as e:
+                if e.status != -4:
+                    raise
+                continue
+            torch.cuda.synchronize()
+            t0 = time.perf_counter()
+            call(flags)
+            torch.cuda.synchronize()
+            est = time.perf_counter() - t0
+            variants.append(flags)
+            reps[flags] = int(max(5, min(200, 4e-3 / max(est, 1e-5))))
+        best = {f: float("inf") for f in variants}
+        for _ in range(rounds):
+            for f in variants:
+                e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+                e0.record()
+                for _ in range(reps[f]):
+                    call(f)
+                e1.record()
+                torch.cuda.synchronize()
+                best[f] = min(best[f], e0.elapsed_time(e1) / reps[f])
+        fastest = min(best.values())
+        ratio = best[0] / fastest
+        worst = max(worst, ratio)
+        path = tcec.sgemm_path(m, n, k, batch, policy)
+        rows.append({"m": m, "n": n, "k": k, "entries": batch, "policy": pol,
+                     "chosen_path": {0: "fused", 1: "packed", 2: "packed + K slices", 3: "direct",
+                                     4: "direct + K slices"}[path],
+                     "ms": {PATH_NAMES[f]: round(best[f], 4) for f in variants},
+                     "chosen_over_best": round(ratio, 3),
+                     "effective_tflops": round(2.0 * m * n * k * batch / (best[0] * 1e-3) / 1e12, 1)})
+        del A, Bt, Ct, ws
+        torch.cuda.empty_cache()
+    return {"worst_ratio": round(worst, 3), "shapes": rows,
+            "what": "whole wmmae_tcec_sgemm_strided_batched calls, N(0,1) operands, workspace resident; "
+                    "each shape on the path the estimates choose and on every path forced, variants "
+                    f"alternating, fastest of {rounds} rounds each"}
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -482,12 +564,15 @@ def main():
                     help="timed steps; default 80 (about 3 s) for the 16384^3 workloads and more for the short "
                          "ones, so that the timed region lasts long enough for the clocks to settle")
     ap.add_argument("--warmup", type=int, default=None, help="untimed steps; default 2 (20 for the short workloads)")
-    ap.add_argument("--workload", default="c4", choices=sorted(WORKLOADS))
+    ap.add_argument("--workload", default="c4", choices=sorted(WORKLOADS) + ["pathcheck"],
+                    help="pathcheck: pinned shapes, each timed on every path the driver has "
+                         "(the guard of the fitted path choices; also part of the default run)")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--no-accuracy", action="store_true")
     ap.add_argument("--no-secondary", action="store_true",
                     help="with the default workload: skip the 4096^3 half of the metric (c3), the "
-                         "API-level GEMM figure and the batched / K-heavy configurations (c5a, c5b)")
+                         "API-level GEMM figure, the batched / K-heavy configurations (c5a, c5b), the "
+                         "primitive tile stream (c2) and the path check")
     ap.add_argument("--flags", type=int, default=0)
     ap.add_argument("--dist", default=None, choices=["uniform", "normal", "exp", "zeros"],
                     help="override the workload's input distribution (zeros: what the kernel reaches "
@@ -511,6 +596,15 @@ def main():
     _lib.lib()
     dev = torch.device("cuda:0")
     torch.cuda.set_device(dev)
+    if args.workload == "pathcheck":
+        r = bench_pathcheck(torch, tcec, dev)
+        print(json.dumps({
+            "metric": "time of the chosen path over the fastest forced path, worst of the pinned shapes",
+            "value": r["worst_ratio"], "unit": "ratio", "n_gpus": 1, "steps": 3, "warmup": 1,
+            "ms_per_step": None, "higher_is_better": False, "scaling": "weak", "vs_baseline": None,
+            "dtype": "f16", "data": "synthetic", "config": {"workload": "pathcheck: " + r["what"]},
+            "pathcheck": r, "roofline": None, "cpu_baseline": None}))
+        return
     w = dict(WORKLOADS[args.workload])
     if args.warmup is None:
         args.warmup = 20 if args.workload in DEFAULT_STEPS else 2
@@ -519,7 +613,8 @@ def main():
     if w.get("kind") == "prim":
         if args.dist is not None:
             w["dist"] = args.dist
-        return bench_primitives(args, torch, tcec, dev, w)
+        print(json.dumps(bench_primitives(args, torch, tcec, dev, w)))
+        return
     if w.get("kind") == "api":
         r = bench_api_gemm(torch, tcec, dev, w["m"], args.steps, args.warmup)
         if args.calibrate:
@@ -570,6 +665,20 @@ def main():
             o, _ = run_gemm_workload(args, torch, tcec, dev, name, DEFAULT_STEPS[name], 20)
             o["unit"] = "TFLOPS"
             out["other_configs"][name] = o
+        # the fragment-primitive tile stream (its own metric: algorithmic GB/s)
+        torch.cuda.empty_cache()
+        c2 = bench_primitives(args, torch, tcec, dev, dict(WORKLOADS["c2"]), DEFAULT_STEPS["c2"], 20,
+                              cpu=not args.no_cpu)
+        for key in ("n_gpus", "higher_is_better", "scaling", "vs_baseline", "data"):
+            c2.pop(key, None)
+        out["other_configs"]["c2"] = c2
+        # the guard of the fitted path choices: chosen path against every forced one
+        torch.cuda.empty_cache()
+        pc = bench_pathcheck(torch, tcec, dev)
+        out["pathcheck"] = {"worst_ratio": pc["worst_ratio"], "what": pc["what"],
+                            "shapes": [{"shape": f"{r['m']}x{r['n']}x{r['k']} x{r['entries']} {r['policy']}",
+                                        "chosen_path": r["chosen_path"], "chosen_over_best": r["chosen_over_best"],
+                                        "ms": r["ms"]} for r in pc["shapes"]]}
     if not args.no_cpu:
         from oracle import oracle as orc
         out["cpu_baseline"] = cpu_baseline(orc, w)

@@ -13,59 +13,14 @@
 // wave64-collective; `sync` arguments are accepted and ignored because a wave
 // runs in lock step.
 #pragma once
+#include "detail/common.hpp"
 #include "detail/functions.hpp"
 #include "detail/policy.hpp"
-#include "detail/split.hpp"
+#include "detail/scale.hpp"
 
 namespace mtk {
 namespace wmma {
 namespace tcec {
-
-namespace detail {
-using mtk::wmma::detail::common::select_value;
-
-template <class Layout, int a, int b> struct layout_switch;
-template <int a, int b> struct layout_switch<col_major, a, b> {
-  static constexpr int value = a;
-};
-template <int a, int b> struct layout_switch<row_major, a, b> {
-  static constexpr int value = b;
-};
-
-// Memory offset of element (i,j) of sub-block at (m_offset, n_offset)
-// (reference: tcec/detail/common.hpp:32-63).
-template <class Layout>
-WMMAE_HD unsigned mem_offset(const unsigned i, const unsigned j,
-                             const unsigned ldm, const unsigned m_offset,
-                             const unsigned n_offset) {
-  if constexpr (std::is_same<Layout, col_major>::value)
-    return (i + m_offset) + (j + n_offset) * ldm;
-  else
-    return (j + n_offset) + (i + m_offset) * ldm;
-}
-
-// The same offsets as function objects under the reference's name
-// (tcec/detail/common.hpp:32-63): from the mem_index a foreach callback
-// receives for a frag_m x frag_n sub-block, or from a position (i, j).
-template <int frag_m, int frag_n, class Layout> struct compute_mem_offset {
-  WMMAE_HD unsigned operator()(const unsigned mem_index, const unsigned ldm,
-                               const unsigned m_offset,
-                               const unsigned n_offset) const {
-    constexpr unsigned lead =
-        std::is_same<Layout, col_major>::value ? frag_m : frag_n;
-    const unsigned major = mem_index / lead, minor = mem_index % lead;
-    if constexpr (std::is_same<Layout, col_major>::value)
-      return mem_offset<Layout>(minor, major, ldm, m_offset, n_offset);
-    else
-      return mem_offset<Layout>(major, minor, ldm, m_offset, n_offset);
-  }
-  WMMAE_HD unsigned operator()(const unsigned i, const unsigned j,
-                               const unsigned ldm, const unsigned m_offset,
-                               const unsigned n_offset) const {
-    return mem_offset<Layout>(i, j, ldm, m_offset, n_offset);
-  }
-};
-} // namespace detail
 
 template <class Use, int m, int n, int k, class T, class Layout = void,
           class Policy_ = typename detail::default_policy<T>::type>
@@ -80,8 +35,8 @@ struct fragment {
   static constexpr bool has_ec =
       std::is_same<typename Policy::error_correction, with_ec>::value;
 
-  using sub_elem_t = typename std::conditional<is_acc, float,
-                                               typename split::mma_tag>::type;
+  using sub_elem_t =
+      typename detail::sub_frag_t<Use, typename split::mma_tag>::type;
   using sub_frag_t =
       typename detail::default_fragment<Use, sub_elem_t, Layout, Policy>::type;
   using storage_t = typename sub_frag_t::storage_element_type;
@@ -205,6 +160,19 @@ template <class F, class MatrixLayout, class MEM_T> struct operand_quads {
       k_runs_of_four<typename F::sub_frag_t::layout_model, is_a>();
 };
 
+// Swizzled staging tiles (additions; the reference pads the rows of its
+// shared-memory tiles instead, test/tcec/batch_gemm.cu:11, a skew found with
+// research/bank-conflict/main.cu:38-71).  On gfx950 no row padding makes the
+// fragment read of a 16x16x32 operand from an fp32 tile conflict free: a
+// 16-byte LDS read is served sixteen lanes at a time, and those sixteen are
+// eight rows of one k group and eight rows of the next.  What does: rows of
+// exactly 32 k (128 bytes, no padding) per k block, with the eight 16-byte
+// pieces of row r stored at piece index p ^ swizzled_piece_mask(r).
+WMMAE_HD constexpr unsigned swizzled_piece_mask(const unsigned row) {
+  return (row >> 1) & 5u;
+}
+template <class MatrixLayout> struct is_swizzled : std::false_type {};
+
 // Value an accumulator element stands for.
 template <class Frag>
 WMMAE_D float combined(const Frag &frag, const unsigned block,
@@ -215,6 +183,28 @@ WMMAE_D float combined(const Frag &frag, const unsigned block,
   else
     return frag.sub_frag[block].x[frag_index];
 }
+} // namespace detail
+
+// Memory layout tags for load_matrix_sync<...>: an fp32 tile with k the
+// contiguous direction (rows of matrix_a / columns of matrix_b, `ldm` floats
+// apart, ldm a multiple of 32) whose 16-byte pieces are permuted inside every
+// aligned block of 32 k: element (r, kk) of the tile is at
+//   r * ldm + (kk & ~31) + 4 * (((kk & 31) / 4) ^ swizzled_piece(r)) + kk % 4
+// with swizzled_piece(r) = (r / 2) & 5.  Fragment loads from such a tile are
+// free of LDS bank conflicts with the policy shape 16x16x32 (other shapes read
+// it correctly, with the conflicts a padded tile would have).  The pointer handed to
+// load_matrix_sync must sit a multiple of 16 rows and of 32 k inside the tile.
+// A writer fills the tile 16 bytes at a time: physical piece q of row r holds
+// the logical piece q ^ swizzled_piece(r) - with utils::cp_async, whose lane l
+// of a wave writes LDS piece base + l, lane l simply fetches that logical piece.
+struct row_major_swizzled; // matrix_a: rows of k
+struct col_major_swizzled; // matrix_b: columns of k
+WMMAE_HD constexpr unsigned swizzled_piece(const unsigned row) {
+  return detail::swizzled_piece_mask(row);
+}
+namespace detail {
+template <> struct is_swizzled<row_major_swizzled> : std::true_type {};
+template <> struct is_swizzled<col_major_swizzled> : std::true_type {};
 } // namespace detail
 
 // ------------------------------------------------------------ fill / neg
@@ -308,6 +298,54 @@ WMMAE_D void load_matrix_sync_with_mul(WMMAE_TCEC_FRAG(Use, Layout) & frag,
       }
       return;
     }
+  }
+  if constexpr (detail::is_swizzled<MatrixLayout>::value) {
+    // swizzled staging tile: 16-byte reads, conflict free in LDS
+    constexpr bool is_a = std::is_same<Use, matrix_a>::value;
+    using L = typename F::sub_frag_t::layout_model;
+    static_assert(!F::is_acc &&
+                      std::is_same<typename std::remove_cv<MEM_T>::type,
+                                   float>::value &&
+                      std::is_same<MatrixLayout,
+                                   typename std::conditional<
+                                       is_a, row_major_swizzled,
+                                       col_major_swizzled>::type>::value &&
+                      detail::k_runs_of_four<L, is_a>(),
+                  "swizzled tiles: fp32 memory, matrix_a with "
+                  "row_major_swizzled or matrix_b with col_major_swizzled, an "
+                  "instruction shape whose lanes own runs of four k");
+    const unsigned lane = mtk::wmma::detail::common::get_lane_id();
+#pragma unroll
+    for (unsigned bn = 0; bn < unsigned(F::num_sub_frag_n); bn++) {
+#pragma unroll
+      for (unsigned bm = 0; bm < unsigned(F::num_sub_frag_m); bm++) {
+        const unsigned block = bm + F::num_sub_frag_m * bn;
+#pragma unroll
+        for (unsigned x = 0; x < L::num_elements; x += 4) {
+          const unsigned i = L::row(lane, x) + bm * bm_size;
+          const unsigned j = L::col(lane, x) + bn * bn_size;
+          const unsigned line = is_a ? i : j, kk = is_a ? j : i;
+          const unsigned off =
+              line * ldm + (kk & ~31u) +
+              4u * (((kk & 31u) >> 2) ^ detail::swizzled_piece_mask(line));
+          const detail::f32x4_t v =
+              *reinterpret_cast<const detail::f32x4_t *>(ptr + off) *
+              static_cast<float>(mul);
+          typename F::storage_t *d1 = nullptr, *d2 = nullptr;
+          if constexpr (F::num_terms >= 2)
+            d1 = &frag.sub_d_frag[block].x[x];
+          if constexpr (F::num_terms >= 3)
+            d2 = &frag.sub_d2_frag[block].x[x];
+          if constexpr (F::num_terms == F::split::num_terms) {
+            detail::split4<T>(v, &frag.sub_frag[block].x[x], d1, d2);
+          } else { // without_ec: the leading term only
+            typename F::storage_t t1[4], t2[4];
+            detail::split4<T>(v, &frag.sub_frag[block].x[x], t1, t2);
+          }
+        }
+      }
+    }
+    return;
   }
   if constexpr (detail::operand_quads<F, MatrixLayout, MEM_T>::value) {
     // k contiguous in memory, base and leading dimension keeping every run

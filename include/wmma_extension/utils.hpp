@@ -29,6 +29,62 @@ cast(const SRC_T v) {
 
 namespace cp_async {
 
+namespace detail {
+// Group bookkeeping of one wave, kept in LDS (wave w of the workgroup owns
+// row w): [0] direct global -> LDS loads issued so far, [1] commits so far,
+// [2 + c % kGroupRing] the value of [0] at commit c.  The hardware counts the
+// wave's outstanding vector-memory instructions, oldest first, so "at most N
+// groups pending" is "at most ([0] now) - ([0] at the N-th last commit)
+// instructions outstanding".  Only differences of these words are ever used,
+// so the LDS need not be initialised: with fewer than N commits behind it,
+// wait_group<N> reads a stale word and waits for more than it has to or for
+// nothing, and both are correct then.
+// The words are read and written with LDS instructions the compiler does not
+// see as such (inline assembly): before an LDS read it knows of, it waits for
+// every direct global -> LDS load in flight, and the bookkeeping of a copy must
+// not wait for the copy.
+constexpr unsigned kGroupRing = 8;
+// LDS byte address of the calling wave's words
+WMMAE_D uint32_t group_state() {
+  __shared__ uint32_t state[16][2 + kGroupRing];
+  const unsigned tid =
+      threadIdx.x + blockDim.x * (threadIdx.y + blockDim.y * threadIdx.z);
+  return static_cast<uint32_t>(reinterpret_cast<uintptr_t>(
+      (__attribute__((address_space(3))) void *)state[(tid >> 6) & 15u]));
+}
+// [0] += 1, by the first active lane
+WMMAE_D void count_issue() {
+  const uint32_t s = group_state();
+  const uint32_t lane = mtk::wmma::detail::common::get_lane_id();
+  if (lane == __builtin_amdgcn_readfirstlane(lane))
+    asm volatile("ds_add_u32 %0, %1" ::"v"(s), "v"(1u) : "memory");
+}
+// words [0] and [1]; every active lane reads the same
+WMMAE_D void read_counts(const uint32_t s, uint32_t &issued,
+                         uint32_t &commits) {
+  typedef uint32_t u32x2 __attribute__((ext_vector_type(2)));
+  u32x2 v;
+  asm volatile("ds_read2_b32 %0, %1 offset1:1\n\ts_waitcnt lgkmcnt(0)"
+               : "=v"(v)
+               : "v"(s)
+               : "memory");
+  issued = v[0];
+  commits = v[1];
+}
+// s_waitcnt vmcnt(t) for a wave-uniform t in [LO, HI]
+template <int LO, int HI> WMMAE_D void wait_vmcnt(const uint32_t t) {
+  if constexpr (LO == HI) {
+    asm volatile("s_waitcnt vmcnt(%0)" ::"n"(LO) : "memory");
+  } else {
+    constexpr int MID = (LO + HI) / 2;
+    if (t <= static_cast<uint32_t>(MID))
+      wait_vmcnt<LO, MID>(t);
+    else
+      wait_vmcnt<MID + 1, HI>(t);
+  }
+}
+} // namespace detail
+
 // Copy Size bytes (4, 8 or 16) per lane from global memory to LDS.  `smem` and
 // `gmem` must be Size-aligned.  The data is visible to the calling wave after
 // wait_all() / wait_group<N>() / wait_pending<N>(), to the workgroup after a
@@ -54,6 +110,7 @@ WMMAE_D void cp_async(void *const smem, const void *const gmem) {
         __builtin_amdgcn_global_load_lds(g, l, 4, 0, 0);
       else
         __builtin_amdgcn_global_load_lds(g, l, 16, 0, 0);
+      detail::count_issue();
       return;
     }
   }
@@ -87,8 +144,19 @@ WMMAE_D void cp_async_lane_linear(void *const smem, const void *const gmem) {
     __builtin_amdgcn_global_load_lds(g, l, 16, 0, 0);
 }
 
-// Group bookkeeping is done by the hardware counter; nothing to do here.
-WMMAE_D void commit() {}
+// Close the group of the copies issued since the last commit()
+// (reference: utils.hpp:46-50, cp.async.commit_group).
+WMMAE_D void commit() {
+  const uint32_t s = detail::group_state();
+  uint32_t issued, commits;
+  detail::read_counts(s, issued, commits);
+  commits += 1u;
+  // (every active lane writes the same two words)
+  asm volatile("ds_write_b32 %0, %1 offset:8\n\tds_write_b32 %2, %3 offset:4" ::"v"(
+                   s + 4u * (commits % detail::kGroupRing)),
+               "v"(issued), "v"(s), "v"(commits)
+               : "memory");
+}
 
 // All copies issued by this wave have landed in LDS.  The compiler may not
 // move instructions across the wait in either direction: arithmetic that
@@ -101,15 +169,39 @@ WMMAE_D void wait_all() {
   __builtin_amdgcn_sched_barrier(0);
 }
 
-// The reference waits until at most N committed groups are pending.  The
-// hardware counts instructions, not groups, and a group may hold any number
-// of copies, so the only bound that is always safe is zero.  Code that knows
-// its group size uses wait_pending instead.
-template <int N> WMMAE_D void wait_group() { wait_all(); }
+// At most the N most recently committed groups of cp_async copies are still
+// pending (reference: utils.hpp:58-62, cp.async.wait_group N; N <= 7 here).
+// Copies issued after the last commit() stay pending as well.  The hardware
+// counter also holds the wave's other vector-memory instructions (ordinary
+// loads and stores issued since), so with those in between the wait can be
+// longer than needed, never shorter.  The copies made by cp_async_lane_linear
+// are not counted: code that uses them knows its group sizes and waits with
+// wait_pending.
+template <int N> WMMAE_D void wait_group() {
+  static_assert(N >= 0 && N < static_cast<int>(detail::kGroupRing),
+                "at most 7 groups can be left pending");
+  if constexpr (N == 0) {
+    wait_all();
+  } else {
+    const uint32_t s = detail::group_state();
+    uint32_t issued, commits, then;
+    detail::read_counts(s, issued, commits);
+    asm volatile("ds_read_b32 %0, %1 offset:8\n\ts_waitcnt lgkmcnt(0)"
+                 : "=v"(then)
+                 : "v"(s + 4u * ((commits - N) % detail::kGroupRing))
+                 : "memory");
+    const uint32_t allowed = __builtin_amdgcn_readfirstlane(issued - then);
+    __builtin_amdgcn_sched_barrier(0);
+    // (more than 63 instructions are never outstanding)
+    if (allowed < 64u)
+      detail::wait_vmcnt<0, 63>(allowed);
+    __builtin_amdgcn_sched_barrier(0);
+  }
+}
 
-// At most N of this wave's cp_async calls (vector-memory instructions, oldest
-// first) are still in flight.  With G calls per group this is the reference's
-// wait_group<N / G>.
+// At most N of this wave's copies (vector-memory instructions, oldest first)
+// are still in flight: wait_group<N / G> for code that knows it issues G copies
+// per group, without the bookkeeping.
 template <int N> WMMAE_D void wait_pending() {
   static_assert(N >= 0 && N <= 63, "the counter has 6 bits");
   __builtin_amdgcn_sched_barrier(0);

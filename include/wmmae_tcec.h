@@ -109,7 +109,16 @@ int wmmae_query(int what, long long *out);
  * kernel on the fp32 operands directly (it splits them on their way into LDS):
  * no packed copy; the workspace then only holds K slices.  All paths give the
  * same bits as long as no K slices are made (those add the partial sums'
- * rounding). */
+ * rounding).
+ *
+ * wmmae_tcec_sgemm_workspace_bytes is an upper bound over the paths: packed
+ * A + packed B + K slices, whichever path the call then takes.  A product the
+ * library runs on the fp32 operands directly (wmmae_tcec_sgemm_path 3 or 4)
+ * touches only the K slices, wmmae_tcec_gemm_packed_workspace_bytes of it, and
+ * path 0 nothing; a caller that knows its products take those paths may pass
+ * that much.  A workspace that is not 16-byte aligned is WMMAE_STATUS_MISALIGNED
+ * on the packed path, which cannot do without it; the other two paths then run
+ * without K slices. */
 int wmmae_tcec_sgemm_workspace_bytes(int m, int n, int k, int batch, int policy,
                                      size_t *bytes);
 
@@ -145,19 +154,27 @@ int wmmae_tcec_sgemm_strided_batched(char transa, char transb, int m, int n,
                                      void *workspace, size_t workspace_bytes,
                                      void *stream);
 
-/* wmmae_tcec_sgemm for callers that cannot allocate device memory (code under
- * HIP graph capture, tight serving loops, harnesses that forbid hipMalloc).
- * No counterpart in the reference.  Same arguments and results as
- * wmmae_tcec_sgemm; the workspace is a fixed device array of
+/* wmmae_tcec_sgemm for callers that cannot allocate device memory (tight
+ * serving loops, harnesses that forbid hipMalloc, code that will be captured
+ * into a HIP graph).  No counterpart in the reference.  Same arguments and
+ * results as wmmae_tcec_sgemm; the workspace is a fixed device array of
  * WMMAE_STATIC_SCRATCH_BYTES inside the library image (every GPU the library
  * runs on holds it until the process ends), so the call makes no hipMalloc /
- * hipFree of any kind.  Products whose split operands need more
- * (wmmae_tcec_sgemm_workspace_bytes; fp16 hi+lo: 4*(m+n)*k bytes rounded up to
- * 16 rows and 32 of k) return WMMAE_STATUS_WORKSPACE_TOO_SMALL; K slices are
- * made only when they fit next to the operands.  All calls on one GPU share
- * the one array: calls that overlap in time on the same GPU (two streams, two
- * threads) race and must be serialised by the caller.  Nothing in the array
- * has to survive between calls and nothing is assumed zero. */
+ * hipFree of any kind.  On the packed path (wmmae_tcec_sgemm_path 1, 2) the
+ * array holds the split operands, and products whose split operands need more
+ * (wmmae_tcec_pack_bytes of A and of B; fp16 hi+lo: 4*(m+n)*k bytes rounded up
+ * to 16 rows and 32 of k) return WMMAE_STATUS_WORKSPACE_TOO_SMALL; K slices
+ * are made only when they fit behind the operands.  On the path that reads the
+ * fp32 operands directly (3, 4) the array holds K slices only, from its start,
+ * and a product of any size succeeds (without K slices when they do not fit);
+ * path 0 does not touch the array.  All calls on one GPU share the one array:
+ * calls that overlap in time on the same GPU (two streams, two threads) race
+ * and must be serialised by the caller.  Nothing in the array has to survive
+ * between calls and nothing is assumed zero.
+ * The first call on a device looks the array's address up
+ * (hipGetSymbolAddress) and the first launch of each kernel sets its LDS
+ * limit (hipFuncSetAttribute): make one call per shape class outside stream
+ * capture before capturing. */
 #define WMMAE_STATIC_SCRATCH_BYTES (64u << 20)
 int wmmae_tcec_sgemm_static(char transa, char transb, int m, int n, int k,
                             const float *alpha, const float *A, int lda,
@@ -263,7 +280,11 @@ int wmmae_tcec_matvec(int type, int ec, float *y, const float *a,
 /* 16-bit split terms held by a 32x32x32 operand fragment (use 0/1) after
  * load_matrix_sync (from_vector == 0) or load_vector (from_vector != 0):
  * terms[(term*E + e)*64 + lane], E = fragment num_elements, e = index of x(e).
- * type 0..2 only (fp32 fragments hold no 16-bit terms).
+ * type 0..2 only (fp32 fragments hold no 16-bit terms).  mem_col 0 / 1: src
+ * is row- / column-major; 2: src (rows of 32 k for use 0, columns of 32 k for
+ * use 1, 16-byte aligned) is first staged into an LDS tile in the swizzled
+ * layout (tcec::row_major_swizzled / col_major_swizzled) with utils::cp_async
+ * and loaded from there - the same terms as mem_col = use.
  * Replaces: test/tcec/vector.cu:15-61 and test/tcec/elementwise.cu:7-26. */
 int wmmae_tcec_frag_dump(int use, int type, int ec, int frag_col,
                          unsigned short *terms, const float *src,
@@ -368,6 +389,21 @@ int wmmae_direct_product(int elem, int terms, int from_float, const float *u,
  * Replaces: cp_async_test_kernel, test/utils/cp_async.cu:15-25. */
 int wmmae_utils_cp_async(int size, int mode, void *dst, const void *src,
                          void *stream);
+
+/* utils::cp_async as a three-stage pipeline written with the reference's
+ * group calls (cp_async<size>, commit, wait_group<2>): one wave moves `groups`
+ * (1..8) groups of `copies` (1..4) copies of 64 x size bytes from src to dst
+ * through a ring of three LDS buffers; dst is written after the pipeline has
+ * drained, so the copies are the wave's only vector-memory instructions while
+ * it runs.  pending (device, groups + 2 ints): the wave's outstanding
+ * vector-memory instructions, read from the hardware, [0] with the first three
+ * groups out, [1 + g] right after the wait_group<2> that releases group g (at
+ * most 2 * copies; above zero while the younger groups are still in flight),
+ * [1 + groups] after wait_all (zero).
+ * Replaces: the commit / wait_group use of utils.hpp:29-64 (the reference has
+ * no test of it). */
+int wmmae_utils_cp_async_pipeline(int size, int copies, int groups, void *dst,
+                                  const void *src, int *pending, void *stream);
 
 /* One wave prints (device printf, the process's stdout) a 16x16x16 half
  * matrix_a fragment loaded from src (16x16 row-major fp32) with

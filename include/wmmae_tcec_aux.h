@@ -29,6 +29,16 @@ int wmmae_mfma_probe(int type, int m, int n, int k, float *d,
                      const unsigned short *a, const unsigned short *b,
                      const float *c, void *stream);
 
+/* Host only, no device access (no counterpart in the reference): where the
+ * GEMM kernel that reads the fp32 operands itself begins a lane's 16-byte read
+ * of k stage `stage` (32 floats a stage) of a row of k contiguous floats, in
+ * floats from the row's start, computed by the address arithmetic the kernel
+ * is compiled from.  tail != 0: the kernel variant for k % 32 != 0.  lane
+ * 0..63, k >= 4, 0 <= stage < ceil(k / 32).  For a test that every read lies
+ * inside its row: 0 <= *first and *first + 4 <= k. */
+int wmmae_direct_read_first(int tail, int k, int stage, int lane,
+                            long long *first);
+
 #ifdef __cplusplus
 }
 #endif

@@ -24,7 +24,7 @@ def test_header_and_library_agree(h):
     declared = set(re.findall(r"\b(wmmae_[a-z0-9_]+)\s*\(", text))
     declared_aux = set(re.findall(r"\b(wmmae_[a-z0-9_]+)\s*\(", aux))
     # the measurement aids live in their own header, outside the product ABI
-    assert declared_aux == {"wmmae_clock_samples", "wmmae_mfma_probe"} and not (declared & declared_aux)
+    assert declared_aux == {"wmmae_clock_samples", "wmmae_mfma_probe", "wmmae_direct_read_first"} and not (declared & declared_aux)
     declared |= declared_aux
     assert declared == set(_lib.EXPORTS)
     for name in declared:
@@ -147,6 +147,8 @@ def test_harness_entries_reject_bad_arguments_on_the_host(h):
     assert h.wmmae_tcec_mma_tile(0, 3, 1, 1, p, p, p, p, 0, 0, 0, 0, 0, None) == -4
     assert h.wmmae_tcec_matvec(3, 1, p, p, p, 0, 0, None) == -4
     assert h.wmmae_tcec_frag_dump(0, 3, 0, 0, p, p, 0, 0, None) == -4
+    assert h.wmmae_tcec_frag_dump(0, 0, 1, 0, p, p, 0, 3, None) == -1
+    assert h.wmmae_tcec_frag_dump(0, 0, 1, 0, p, ctypes.c_void_p(72), 0, 2, None) == -7
     # fragment operators, eye, direct product
     assert h.wmmae_fragment_ops(6, 0, 0, f(1.0), p, p, p, None) == -1
     assert h.wmmae_fragment_ops(0, 3, 0, f(1.0), p, p, p, None) == -1
@@ -161,6 +163,12 @@ def test_harness_entries_reject_bad_arguments_on_the_host(h):
     assert h.wmmae_utils_cp_async(12, 0, p, p, None) == -1
     assert h.wmmae_utils_cp_async(4, 7, p, p, None) == -1
     assert h.wmmae_utils_cp_async(16, 0, p, ctypes.c_void_p(72), None) == -7
+    assert h.wmmae_utils_cp_async_pipeline(4, 2, 3, None, p, p, None) == -2
+    assert h.wmmae_utils_cp_async_pipeline(4, 2, 3, p, p, None, None) == -2
+    assert h.wmmae_utils_cp_async_pipeline(12, 2, 3, p, p, p, None) == -1
+    assert h.wmmae_utils_cp_async_pipeline(4, 5, 3, p, p, p, None) == -1
+    assert h.wmmae_utils_cp_async_pipeline(4, 2, 0, p, p, p, None) == -1
+    assert h.wmmae_utils_cp_async_pipeline(16, 2, 3, p, ctypes.c_void_p(72), p, None) == -7
     assert h.wmmae_utils_cast(0, None, p, 4, None) == -2
     assert h.wmmae_utils_cast(0, p, p, -1, None) == -1
     assert h.wmmae_utils_cast(0, p, p, 0, None) == 0                       # nothing to do
@@ -227,3 +235,28 @@ def test_slice_counts_the_estimates_choose():
     out = ctypes.c_int(-1)
     for shape in ((1792, 1792, 4096), (2048, 2048, 2048)):
         assert h.wmmae_tcec_sgemm_path(*shape, 1, 0, 0, ctypes.byref(out)) == 0 and out.value == 1, shape
+
+
+def test_direct_kernel_reads_stay_inside_their_rows(h):
+    """The GEMM kernel that loads the fp32 operands itself reads 16 bytes per lane and stage.  For
+    every k from 4 on, every stage and every lane, the four floats lie inside the row of k floats
+    (address arithmetic evaluated on the host from the kernel's own functions): rows may end at
+    an allocation's last float."""
+    first = ctypes.c_longlong(0)
+    for k in list(range(4, 200)) + [999, 1000, 1001, 4100, 16387, 100003]:
+        stages = (k + 31) // 32
+        for tail in ((1,) if k % 32 else (0, 1)):
+            for stage in sorted({0, 1, stages // 2, stages - 2, stages - 1} & set(range(stages))):
+                seen = set()
+                for lane in range(64):
+                    assert h.wmmae_direct_read_first(tail, k, stage, lane, ctypes.byref(first)) == 0
+                    f = first.value
+                    assert 0 <= f and f + 4 <= k, (k, tail, stage, lane, f)
+                    seen.update(range(f, f + 4))
+                # together the lanes of a row cover the stage's part of the row
+                assert seen >= set(range(32 * stage, min(k, 32 * stage + 32))), (k, tail, stage)
+    assert h.wmmae_direct_read_first(1, 3, 0, 0, ctypes.byref(first)) == -1
+    assert h.wmmae_direct_read_first(0, 33, 0, 0, ctypes.byref(first)) == -1
+    assert h.wmmae_direct_read_first(1, 33, 2, 0, ctypes.byref(first)) == -1
+    assert h.wmmae_direct_read_first(1, 33, 0, 64, ctypes.byref(first)) == -1
+    assert h.wmmae_direct_read_first(1, 33, 0, 0, None) == -2

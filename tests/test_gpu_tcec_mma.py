@@ -42,23 +42,28 @@ def _run(tc, dev, shape, type_, ec, inst, A, B, C, a_col, b_col, c_col, d_col, r
 @pytest.mark.parametrize("ec", [1, 0])
 @pytest.mark.parametrize("inst", [0, 1, 2])
 @pytest.mark.parametrize("shape", [0, 1])
-def test_mma_tile_all_layouts(tc, orc, dev, type_, ec, inst, shape):
+@pytest.mark.parametrize("rounding", [0, 1, 2])
+def test_mma_tile_all_layouts(tc, orc, dev, type_, ec, inst, shape, rounding):
     """Every memory-layout combination of A, B, C, D, with and without C
-    (the matrix of test/tcec/mma.cu:186-3526), seeded uniform[-1,1]."""
+    (the matrix of test/tcec/mma.cu:186-3526), seeded uniform[-1,1], through mma_sync (the
+    policy's default: mma_rn_sync with error correction, mma_rz_sync without,
+    tcec.hpp:896-927, no_cor.hpp:858-897), mma_rn_sync and mma_rz_sync, each for both policies."""
     m, n, k = _dims(shape, inst)
     rng = np.random.default_rng(1000 * type_ + 100 * ec + 10 * inst + shape)
     kind = KIND_OF_TYPE[type_]
+    # leading product added outside the matrix core (rn) or chained through it (rz)
+    main_outside = bool(ec) if rounding == 0 else rounding == 1
     for a_col, b_col, c_col, d_col, with_c in itertools.product((0, 1), repeat=5):
         A = rng.uniform(-1, 1, (m, k)).astype(np.float32)
         B = rng.uniform(-1, 1, (k, n)).astype(np.float32)
         C = rng.uniform(-1, 1, (m, n)).astype(np.float32) if with_c else None
-        D = _run(tc, dev, shape, type_, ec, inst, A, B, C, a_col, b_col, c_col, d_col, 0)
+        D = _run(tc, dev, shape, type_, ec, inst, A, B, C, a_col, b_col, c_col, d_col, rounding)
         ref = orc.gemm_f64(A, B) + (C if with_c else 0)
         err = orc.max_abs_err(D, ref)
-        # the emulator follows tcec::mma_sync instruction by instruction, each instruction in
-        # the measured accumulate arithmetic of the matrix core: same bits
+        # the emulator follows the device function instruction by instruction, each instruction
+        # in the measured accumulate arithmetic of the matrix core: same bits
         emu = orc.tcec_matmul(A, B, C, kind=kind, ec=bool(ec), fk=INST_K[inst],
-                              main_outside=bool(ec), hw_model=True)
+                              main_outside=main_outside, hw_model=True)
         assert np.array_equal(D.view(np.uint32), emu.view(np.uint32)), \
             (a_col, b_col, c_col, d_col, with_c, np.abs(D - emu).max())
         if ec and type_ != 1:
@@ -88,6 +93,23 @@ def test_mma_tile_exact_cases(tc, orc, dev, type_, ec):
     A = rng.uniform(-1, 1, (32, 32)).astype(np.float32)
     D = _run(tc, dev, 0, type_, ec, 0, A, eye, None, 0, 0, 0, 0, 0)
     assert np.array_equal(D, orc.tcec_matmul(A, eye, kind=KIND_OF_TYPE[type_], ec=bool(ec)))
+
+
+@pytest.mark.parametrize("type_", [0, 1, 2])
+@pytest.mark.parametrize("use", [0, 1])
+def test_fragment_terms_from_a_swizzled_tile(tc, orc, dev, type_, use):
+    """A tile staged in LDS with its 16-byte pieces permuted (tcec::row_major_swizzled for
+    matrix_a, col_major_swizzled for matrix_b; written with utils::cp_async by the recipe of
+    the layout) and loaded with that tag gives the same terms as the plain load of the same
+    matrix, which test_fragment_terms_bit_exact pins against the oracle's split."""
+    rng = np.random.default_rng(22 + type_)
+    N = 32
+    for ec, frag_col in itertools.product((1, 0), (0, 1)):
+        X = rng.uniform(-1, 1, (N, N)).astype(np.float32)
+        src = torch.from_numpy(_mem(X, use)).to(dev)      # A: rows of k; B: columns of k
+        plain = tc.frag_dump(use, type_, ec, frag_col, src, 0, use).cpu().numpy()
+        swz = tc.frag_dump(use, type_, ec, frag_col, src, 0, 2).cpu().numpy()
+        assert plain.any() and np.array_equal(plain, swz), (ec, frag_col)
 
 
 @pytest.mark.parametrize("type_", [0, 2])

@@ -29,6 +29,41 @@ def test_cp_async_copies_every_byte(tc, dev, size, mode):
     assert np.array_equal(got, expect)
 
 
+@pytest.mark.parametrize("size", [4, 16])
+@pytest.mark.parametrize("copies", [1, 3, 4])
+def test_cp_async_three_stage_pipeline_keeps_two_groups_in_flight(tc, dev, size, copies):
+    """cp_async / commit / wait_group<2> as a three-stage pipeline (the use the reference's
+    utils.hpp:29-64 is made for): every byte arrives, and wait_group<2> waits for exactly the
+    oldest group - right after it the wave's own counter of outstanding vector-memory
+    instructions (read from the hardware) is at most the two younger groups' copies, and above
+    zero at least once: later groups are still in flight while the first is consumed."""
+    groups = 8
+    words = groups * copies * 64 * size // 4
+    src = torch.arange(words, dtype=torch.float32, device=dev)
+    # push the source out of the caches (1 GiB written behind it), so that the copies take a
+    # round trip to HBM, much longer than the wave needs to issue three groups
+    junk = torch.empty(1 << 28, dtype=torch.float32, device=dev)
+    junk.fill_(1.0)
+    torch.cuda.synchronize()
+    got, pending = tc.utils_cp_async_pipeline(size, copies, groups, src)
+    torch.cuda.synchronize()
+    assert torch.equal(got, src)
+    p = pending.cpu().numpy()
+    assert 0 <= p[0] <= 3 * copies                     # three groups issued, nothing awaited
+    assert (p[1:1 + groups] >= 0).all() and (p[1:1 + groups] <= 2 * copies).all(), p
+    assert p[1 + groups] == 0                          # wait_all
+    assert p[1:1 + groups].max() > 0, p
+
+
+def test_cp_async_pipeline_register_path_has_nothing_pending(tc, dev):
+    """Size 8 has no direct global -> LDS load: the copies go through registers, are complete when
+    cp_async returns and are not counted as pending."""
+    src = torch.arange(6 * 2 * 64 * 2, dtype=torch.float32, device=dev)
+    got, pending = tc.utils_cp_async_pipeline(8, 2, 6, src)
+    assert torch.equal(got, src)
+    assert (pending.cpu().numpy()[1:] == 0).all()
+
+
 def test_cp_async_argument_checks(tc, dev):
     from wmma_extension_amd._lib import WmmaeError
     src = torch.zeros(1024, dtype=torch.float32, device=dev)

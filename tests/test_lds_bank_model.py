@@ -1,46 +1,92 @@
-"""Host-side LDS bank analysis of the layouts the GEMM kernels use (the reference does
-this on the device for its shared-memory skew, research/bank-conflict/main.cu:38-71).
+"""Host-side LDS bank analysis of the layouts the GEMM kernels use (the reference does this on
+the device for its shared-memory skew, research/bank-conflict/main.cu:38-71, and settles on a
+skew from it, test/tcec/batch_gemm.cu:11).
 
-Model: 64 banks of 4 bytes; a 128-bit read is served sixteen lanes at a time, each lane
-touching four consecutive banks; the conflict degree of a phase is the largest number of
-lanes that hit one bank.  rocprofv3's SQ_LDS_BANK_CONFLICT reads 0 for all three kernels
-on the GPU; this test shows why, and that the obvious alternatives would not."""
+The model is measured, not assumed.  Two-lane probes on gfx950 (two active lanes touching the
+same bank at different addresses; SQ_LDS_BANK_CONFLICT says whether they were served in the same
+cycle) and stride scans under SQ_LDS_BANK_CONFLICT / SQ_LDS_IDX_ACTIVE gave:
+
+  ds_read_b128   4 cycles; the lanes of a cycle are the lane quads 0 3 5 6 | 1 2 4 7 |
+                 8 11 13 14 | 9 10 12 15 (quad q = lanes 4q .. 4q+3); 64 banks of 4 bytes
+  ds_read_b64    2 cycles of 32 consecutive lanes; 64 banks
+  ds_write_b64   4 cycles of 16 consecutive lanes; bank b and bank b + 32 collide (the write
+                 path is 128 bytes wide)
+  ds_write_b128  8 cycles of 8 consecutive lanes; likewise 32 banks
+
+An instruction takes, per cycle group, as many cycles as the most loaded bank has distinct
+addresses.  The literal cycle counts of the stride scans below are the counters' readings (per
+instruction, 1000 repetitions each), which the model has to reproduce; the kernels' own layouts
+are then evaluated with it and compared with what rocprofv3 reads for them."""
 import numpy as np
 
+QUADS_OF_CYCLE = ((0, 3, 5, 6), (1, 2, 4, 7), (8, 11, 13, 14), (9, 10, 12, 15))
 
-def _degree_b128(byte_addr):
-    """Worst conflict degree over the four 16-lane phases of a 64-lane ds_read_b128."""
-    worst = 0
-    for phase in range(4):
-        hits = np.zeros(64, dtype=int)
-        for lane in range(16 * phase, 16 * phase + 16):
-            first = (byte_addr[lane] // 4) % 64
-            for b in range(4):
-                hits[(first + b) % 64] += 1
-        worst = max(worst, hits.max())
-    return worst
+
+def _groups(op):
+    if op == "read_b128":
+        return [[4 * q + i for q in quads for i in range(4)] for quads in QUADS_OF_CYCLE], 64
+    if op == "read_b64":
+        return [list(range(32 * p, 32 * p + 32)) for p in range(2)], 64
+    if op == "write_b64":
+        return [list(range(16 * p, 16 * p + 16)) for p in range(4)], 32
+    if op == "write_b128":
+        return [list(range(8 * p, 8 * p + 8)) for p in range(8)], 32
+    raise ValueError(op)
+
+
+def cycles(op, byte_addr):
+    """LDS cycles of one 64-lane instruction with the given per-lane byte addresses."""
+    width = {"read_b128": 16, "write_b128": 16, "read_b64": 8, "write_b64": 8}[op]
+    groups, banks = _groups(op)
+    total = 0
+    for lanes in groups:
+        per_bank = {}
+        for lane in lanes:
+            for w in range(width // 4):
+                dword = int(byte_addr[lane]) // 4 + w
+                per_bank.setdefault(dword % banks, set()).add(dword)
+        total += max(len(v) for v in per_bank.values())
+    return total
+
+
+def free(op):
+    return len(_groups(op)[0])
+
+
+LANE = np.arange(64)
+
+
+def test_model_reproduces_the_measured_stride_scans():
+    """Lane l reads 16 bytes of row l % R at float 8 * (l / R) of a tile with a row stride of ld
+    floats (R = 16: an operand fragment of the 16x16x32 instruction read from a row-major fp32
+    tile; R = 32: the 32-row pattern).  Counter readings per instruction, ld = 32 .. 72."""
+    measured_16 = {32: 16, 36: 8, 40: 8, 44: 8, 48: 8, 52: 8, 56: 8, 60: 8, 64: 32, 68: 8, 72: 8}
+    measured_32 = {32: 32, 36: 4, 40: 8, 44: 4, 48: 16, 52: 4, 56: 8, 60: 4, 64: 64, 68: 4, 72: 8}
+    for ld, want in measured_16.items():
+        addr = ((LANE % 16) * ld + 8 * (LANE // 16)) * 4
+        assert cycles("read_b128", addr) == want, ld
+    for ld, want in measured_32.items():
+        addr = ((LANE % 32) * ld + 8 * (LANE // 32)) * 4
+        assert cycles("read_b128", addr) == want, ld
 
 
 def test_fragment_major_chunks_are_conflict_free():
-    """Packed operands and the fused kernel's term buffers: lane l reads base + 16*l."""
-    lane = np.arange(64)
-    assert _degree_b128(16 * lane) == 1
+    """Packed operands and the term buffers of the single-kernel path: lane l reads base + 16*l."""
+    assert cycles("read_b128", 16 * LANE) == free("read_b128")
 
 
 def test_fused_kernel_raw_layout():
-    """Raw fp32 row block of the fused kernel: 16 rows x 128 bytes.  Lane l converts row
-    r = l%16, floats 8*(l/16) .. +7.  Stored row-major, all sixteen rows of a phase start
-    in the same banks; with the pieces of a row permuted as the kernel does
-    (32-byte pair index XOR (r/2)%4, halves swapped for r >= 8) every phase covers all
-    banks exactly once."""
-    lane = np.arange(64)
-    r, g = lane % 16, lane // 16
+    """Raw fp32 row block of the single-kernel path: 16 rows x 128 bytes.  Lane l converts row
+    r = l % 16, floats 8 * (l / 16) .. +7.  Stored row-major, every read is a four-way conflict;
+    with the pieces of a row permuted as the kernel does (32-byte pair index XOR (r / 2) % 4,
+    halves swapped for r >= 8) both reads are conflict free (the counter reads 0 for it)."""
+    r, g = LANE % 16, LANE // 16
     plain = r * 128 + g * 32
-    assert _degree_b128(plain) == 8 and _degree_b128(plain + 16) == 8
+    assert cycles("read_b128", plain) == 16 and cycles("read_b128", plain + 16) == 16
     base = r * 128 + 32 * (g ^ ((r >> 1) & 3))
     lo = base + 16 * (r >> 3)
     hi = base + 16 * (1 - (r >> 3))
-    assert _degree_b128(lo) == 1 and _degree_b128(hi) == 1
+    assert cycles("read_b128", lo) == 4 and cycles("read_b128", hi) == 4
     # the permutation is the one the requests write: lane l of request h fetches row
     # 8h + l/8, piece (l%8) ^ (2*((l/16)%4) + h) into slot h*1024 + 16*l
     where = {}
@@ -55,17 +101,57 @@ def test_fused_kernel_raw_layout():
         assert where[(r[l], 2 * g[l] + 1)] == hi[l]              # floats 8g+4 .. 8g+7
 
 
-def test_api_level_kernel_skew():
-    """The API-level GEMM stages fp32 tiles with a leading dimension of 32 + 4 floats
-    (the reference settles on a skew of 8 floats for its 32-lane warps, batch_gemm.cu:11).
-    A fragment load takes lane l's eight floats of row l%16 from k = 8*(l/16) on, as two
-    128-bit reads: with the skew of 4 the sixteen rows of a phase start 36 banks apart and
-    cover all banks once; unpadded they all start in the same or the opposite half."""
-    lane = np.arange(64)
+def _direct_swizzle(q):
+    return (12 * (q & 1)) ^ (4 * (q >> 1))
 
-    def degree(ld):
-        addr = ((lane % 16) * ld + 8 * (lane // 16)) * 4
-        return max(_degree_b128(addr), _degree_b128(addr + 16))
-    assert degree(36) == 1
-    assert degree(32) == 8
-    assert degree(40) > 1          # the reference's skew of 8 does not suit 64 banks
+
+def test_direct_kernel_image_writes_and_reads():
+    """The GEMM kernel that splits the fp32 operands itself writes each term of a row block as
+    8-byte halves of the fragment positions (two writes per term, position (row r, k group q) at
+    16-byte slot 16q + (r ^ swz(q))).  The fragment reads are conflict free; an 8-byte write of
+    sixteen consecutive lanes touches 32 different banks, but on the 128-byte write path banks b
+    and b + 32 collide: two-way, 8 cycles instead of 4.  Per stage and wave: 24 such writes and 24
+    fragment reads, so SQ_LDS_BANK_CONFLICT / SQ_LDS_IDX_ACTIVE = 96 / 288 = 33.3 % - what the
+    counters read for this kernel (33.3 % and 33.5 % on the K-heavy and the batched workload)."""
+    swz = np.array([_direct_swizzle(q) for q in range(4)])
+    write_cycles = []
+    for h in range(2):
+        r, q = 8 * h + (LANE >> 3), (LANE & 7) >> 1
+        woff = 256 * q + 16 * (r ^ swz[q]) + 8 * (LANE & 1)
+        write_cycles.append(cycles("write_b64", woff))
+    assert write_cycles == [8, 8]
+    slot = (LANE & 48) + ((LANE & 15) ^ swz[LANE >> 4])
+    assert cycles("read_b128", 16 * slot) == 4
+    assert sorted(slot) == list(range(64))                       # a permutation of the chunk
+    writes = reads = 24
+    conflict = writes * (8 - free("write_b64"))
+    active = writes * 8 + reads * 4
+    assert abs(conflict / active - 1 / 3) < 1e-12
+    # 16-byte writes (a lane owning a whole fragment position, eight lanes = two rows x four k
+    # groups) with slot 16q + (r ^ 2q) would be conflict free on both sides; the kernel built that
+    # way ran at the same speed (the matrix pipe does not wait for the LDS here) and is not kept
+    r, q = LANE >> 2, LANE & 3
+    assert cycles("write_b128", 16 * (16 * q + (r ^ (2 * q)))) == free("write_b128")
+    assert cycles("read_b128", 16 * ((LANE & 48) + ((LANE & 15) ^ (2 * (LANE >> 4))))) == 4
+
+
+def test_api_level_kernel_tiles():
+    """The GEMM written on the public API stages fp32 tiles of 32 k per row.  A fragment load
+    takes lane l's eight floats of row l % 16 from k = 8 * (l / 16) on, as two 128-bit reads.
+    No row padding makes that pattern conflict free (the scan above: every stride that is a
+    multiple of four floats costs at least two-way; the reference's skew of 8 floats, chosen for
+    32 banks and 32 lanes, too).  Unpadded rows with the 16-byte pieces of row r stored at piece
+    index p ^ ((r / 2) & 5) are: that is the tile tcec::load_matrix_sync reads with the
+    swizzled memory layout tags, and the counter reads 0 conflicts for it."""
+    r, g = LANE % 16, LANE // 16
+    for ld in (32, 36, 40):
+        addr = (r * ld + 8 * g) * 4
+        assert cycles("read_b128", addr) > 4 and cycles("read_b128", addr + 16) > 4
+    f = (r >> 1) & 5
+    for e in range(2):
+        assert cycles("read_b128", r * 128 + 16 * ((2 * g + e) ^ f)) == 4
+    # the writer's side: a direct global -> LDS copy fills 64 consecutive 16-byte pieces, eight
+    # rows; lane l's piece is physical piece l % 8 of row l / 8, i.e. logical piece
+    # (l % 8) ^ f(row): every logical piece of every row exactly once
+    seen = {(row, (l % 8) ^ ((row >> 1) & 5)) for row in range(16) for l in range(8)}
+    assert len(seen) == 128

@@ -12,7 +12,9 @@ ROOT = os.path.dirname(_PKG)
 INCLUDE_DIR = os.path.join(ROOT, "include")
 CSRC_DIR = os.path.join(_PKG, "csrc")
 LIB_DIR = os.path.join(_PKG, "lib")
-LIB_PATH = os.path.join(LIB_DIR, "libwmmae_tcec.so")
+# WMMAE_TCEC_LIB names another build of the same library (for comparing two
+# builds on one GPU); the default is the in-tree one
+LIB_PATH = os.environ.get("WMMAE_TCEC_LIB") or os.path.join(LIB_DIR, "libwmmae_tcec.so")
 
 HIPCC_FLAGS = [
     "--offload-arch=gfx950",
@@ -56,9 +58,11 @@ EXPORTS = [
     "wmmae_direct_product",
     "wmmae_clock_samples",
     "wmmae_utils_cp_async",
+    "wmmae_utils_cp_async_pipeline",
     "wmmae_print_fragment",
     "wmmae_utils_cast",
     "wmmae_mfma_probe",
+    "wmmae_direct_read_first",
 ]
 
 
@@ -138,9 +142,11 @@ _SIGNATURES = {
     "wmmae_direct_product": (_i, [_i, _i, _i, _vp, _vp, _vp, _vp]),
     "wmmae_clock_samples": (_i, [_vp, _i, _ll, _vp]),
     "wmmae_utils_cp_async": (_i, [_i, _i, _vp, _vp, _vp]),
+    "wmmae_utils_cp_async_pipeline": (_i, [_i, _i, _i, _vp, _vp, _vp, _vp]),
     "wmmae_print_fragment": (_i, [_i, _i, _vp, _c.c_float, _vp]),
     "wmmae_utils_cast": (_i, [_i, _vp, _vp, _ll, _vp]),
     "wmmae_mfma_probe": (_i, [_i, _i, _i, _i, _vp, _vp, _vp, _vp, _vp]),
+    "wmmae_direct_read_first": (_i, [_i, _i, _i, _i, _c.POINTER(_ll)]),
 }
 
 
@@ -154,6 +160,8 @@ def lib():
                 "(hipcc --offload-arch=gfx950); there is no CPU fallback")
         handle = ctypes.CDLL(LIB_PATH)
         for name, (restype, argtypes) in _SIGNATURES.items():
+            if not hasattr(handle, name) and os.environ.get("WMMAE_TCEC_LIB"):
+                continue          # an older build named for a comparison: fewer entry points
             fn = getattr(handle, name)
             fn.restype = restype
             fn.argtypes = argtypes

@@ -378,6 +378,49 @@ constexpr int ring_depth(const int bm, const int bn, const int terms) {
   return fit > 4 ? 4 : fit;
 }
 
+// Workgroups of one GEMM kernel that a compute unit holds at a time: what the
+// runtime's occupancy query says (registers, LDS and wave slots together),
+// looked up once per kernel and device; the LDS bound alone where the query
+// gives nothing (no device visible).  The persistent work-item modes give
+// every resident workgroup a fixed share of the items, so a count the
+// registers do not allow would leave the extra workgroups' shares to run after
+// everything else (the one-term direct kernel: 48 KiB of LDS, three by that
+// bound, but 512 registers a lane).
+template <class MT, int TERMS, int BM, int BN, int WGM, int WGN, bool RN,
+          int DIRECT = 0>
+int workgroups_per_cu() {
+  constexpr int NSTAGE = DIRECT ? 2 : ring_depth(BM, BN, TERMS);
+  using Cfg =
+      wmmae_gemm::GemmConfig<MT, TERMS, BM, BN, WGM, WGN, NSTAGE, RN, DIRECT>;
+  constexpr int by_lds =
+      (160 * 1024) / Cfg::LDS_BYTES > 4 ? 4 : (160 * 1024) / Cfg::LDS_BYTES;
+  static std::atomic<int> cached[64];
+  static std::atomic<unsigned long long> lds_allowed{0};
+  int dev = 0;
+  if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 64) {
+    (void)hipGetLastError();
+    return by_lds;
+  }
+  const int c = cached[dev].load(std::memory_order_relaxed);
+  if (c > 0)
+    return c;
+  auto kernel = wmmae_gemm::tcec_gemm_kernel<MT, TERMS, BM, BN, WGM, WGN,
+                                             NSTAGE, RN, DIRECT>;
+  int n = 0;
+  if (allow_dynamic_lds(reinterpret_cast<const void *>(kernel), Cfg::LDS_BYTES,
+                        lds_allowed) != hipSuccess ||
+      hipOccupancyMaxActiveBlocksPerMultiprocessor(
+          &n, reinterpret_cast<const void *>(kernel), Cfg::NTHREADS,
+          Cfg::LDS_BYTES) != hipSuccess ||
+      n <= 0) {
+    (void)hipGetLastError();
+    return by_lds;
+  }
+  n = n < by_lds ? n : by_lds;
+  cached[dev].store(n, std::memory_order_relaxed);
+  return n;
+}
+
 template <class MT, int TERMS, int BM, int BN, int WGM, int WGN, bool RN,
           int DIRECT = 0>
 int launch_gemm(const GemmArgs &g) {
@@ -420,8 +463,8 @@ int launch_gemm(const GemmArgs &g) {
   //    one workgroup per item, handed out by the hardware as compute units
   //    become free, which evens out compute units of unequal speed over many
   //    rounds (a fixed share per workgroup measured 7 % slower at 16384^3).
-  constexpr int per_cu =
-      (160 * 1024) / Cfg::LDS_BYTES > 4 ? 4 : (160 * 1024) / Cfg::LDS_BYTES;
+  const int per_cu =
+      workgroups_per_cu<MT, TERMS, BM, BN, WGM, WGN, RN, DIRECT>();
   const long long resident = static_cast<long long>(device_cus()) * per_cu;
   int grid = static_cast<int>(std::min(items, resident));
   int entry_per_xcd = 0;
@@ -563,6 +606,34 @@ int gemm_dispatch(const int policy, const int flags, const GemmArgs &g) {
     return rn ? WMMAE_STATUS_NOT_SUPPORTED : gemm_by_size<__bf16, 1, false>(g);
   default:
     return WMMAE_STATUS_INVALID_VALUE;
+  }
+}
+
+// Resident workgroups per compute unit of the packed kernel a policy runs with
+// tile shape 0 (256x128), 1 (128x128) or 2 (64x64): the number launch_gemm
+// plans its rounds with, for the workspace query.
+template <class MT, int TERMS> int per_cu_by_shape(const int shape) {
+  switch (shape) {
+  case 0:
+    return workgroups_per_cu<MT, TERMS, 256, 128, 2, 2, false>();
+  case 1:
+    return workgroups_per_cu<MT, TERMS, 128, 128, 2, 2, false>();
+  default:
+    return workgroups_per_cu<MT, TERMS, 64, 64, 2, 2, false>();
+  }
+}
+int per_cu_of(const int policy, const int shape) {
+  switch (policy) {
+  case WMMAE_POLICY_F16_EC:
+    return per_cu_by_shape<_Float16, 2>(shape);
+  case WMMAE_POLICY_F16_NOEC:
+    return per_cu_by_shape<_Float16, 1>(shape);
+  case WMMAE_POLICY_BF16X3_EC:
+    return per_cu_by_shape<__bf16, 3>(shape);
+  case WMMAE_POLICY_BF16X2_EC:
+    return per_cu_by_shape<__bf16, 2>(shape);
+  default:
+    return per_cu_by_shape<__bf16, 1>(shape);
   }
 }
 
@@ -1036,14 +1107,12 @@ int sgemm_impl(const char transa, const char transb, const int m, const int n,
     void *ws = workspace;
     size_t ws_bytes = workspace_bytes;
     bool own = false;
-    if (ws == nullptr) {
-      if (bytes_c > 0) {
-        WMMAE_HIP_TRY(hipMallocAsync(&ws, bytes_c, s));
-        ws_bytes = bytes_c;
-        own = true;
-      }
-    } else if (reinterpret_cast<uintptr_t>(ws) % 16 != 0) {
-      return WMMAE_STATUS_MISALIGNED;
+    // (a caller's workspace that is not 16-byte aligned is left alone by
+    // plan_k_slices: this path can do without, as the single kernel does)
+    if (ws == nullptr && bytes_c > 0) {
+      WMMAE_HIP_TRY(hipMallocAsync(&ws, bytes_c, s));
+      ws_bytes = bytes_c;
+      own = true;
     }
     GemmArgs g;
     g.a = nullptr;
@@ -1209,10 +1278,9 @@ int wmmae_tcec_gemm_packed_workspace_bytes(const int policy, const int m,
     const int KT = packed_k_tiles(k);
     size_t need = 0;
     const int shapes[3][2] = {{256, 128}, {128, 128}, {64, 64}};
-    for (const auto &sh : shapes) {
-      const int lds = ring_depth(sh[0], sh[1], p.terms) *
-                      (sh[0] / 16 + sh[1] / 16) * p.terms * 1024;
-      const int per_cu = std::min(4, (160 * 1024) / lds);
+    for (int i = 0; i < 3; i++) {
+      const int *const sh = shapes[i];
+      const int per_cu = per_cu_of(policy, i);
       const TailPlan t =
           plan_tail(ceil_div(m, sh[0]) * ceil_div(n, sh[1]),
                     static_cast<long long>(device_cus()) * per_cu, KT);
@@ -1300,6 +1368,18 @@ int wmmae_tcec_sgemm_batched(const char transa, const char transb, const int m,
   return sgemm_impl(transa, transb, m, n, k, alpha, nullptr, A_array, lda, 0,
                     nullptr, B_array, ldb, 0, beta, nullptr, C_array, ldc, 0,
                     batch, policy, flags, workspace, workspace_bytes, stream);
+}
+
+int wmmae_direct_read_first(const int tail, const int k, const int stage,
+                            const int lane, long long *const first) {
+  if (first == nullptr)
+    return WMMAE_STATUS_NULL_POINTER;
+  if (k < 4 || stage < 0 || stage >= ceil_div(k, 32) || lane < 0 || lane > 63 ||
+      (tail == 0 && k % 32 != 0))
+    return WMMAE_STATUS_INVALID_VALUE;
+  *first = wmmae_gemm::direct_read_first(tail != 0, k, stage,
+                                         static_cast<unsigned>(lane));
+  return WMMAE_STATUS_SUCCESS;
 }
 
 // ---------------------------------------------- entry point that allocates

@@ -205,8 +205,11 @@ int wmmae_tcec_frag_dump(const int use, const int type, const int ec,
                          const int mem_col, void *const stream) {
   if (!terms || !src)
     return WMMAE_STATUS_NULL_POINTER;
-  if (use < 0 || use > 1)
+  if (use < 0 || use > 1 || mem_col < 0 || mem_col > 2)
     return WMMAE_STATUS_INVALID_VALUE;
+  // (the swizzled tile is staged with 16-byte copies)
+  if (mem_col == 2 && reinterpret_cast<uintptr_t>(src) % 16 != 0)
+    return WMMAE_STATUS_MISALIGNED;
   if (type == 3) // fp32 fragments hold no 16-bit terms
     return WMMAE_STATUS_NOT_SUPPORTED;
   hipStream_t s = static_cast<hipStream_t>(stream);
@@ -471,6 +474,34 @@ int wmmae_utils_cp_async(const int size, const int mode, void *const dst,
   else
     hipLaunchKernelGGL(wmmae_harness::cp_async_kernel<16>, dim3(1), dim3(128),
                        0, s, d, g, mode);
+  return launch_status();
+}
+
+int wmmae_utils_cp_async_pipeline(const int size, const int copies,
+                                  const int groups, void *const dst,
+                                  const void *const src, int *const pending,
+                                  void *const stream) {
+  if (!dst || !src || !pending)
+    return WMMAE_STATUS_NULL_POINTER;
+  if ((size != 4 && size != 8 && size != 16) || copies < 1 || copies > 4 ||
+      groups < 1 || groups > 8)
+    return WMMAE_STATUS_INVALID_VALUE;
+  if (reinterpret_cast<uintptr_t>(src) % size != 0 ||
+      reinterpret_cast<uintptr_t>(dst) % 4 != 0 ||
+      reinterpret_cast<uintptr_t>(pending) % 4 != 0)
+    return WMMAE_STATUS_MISALIGNED;
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  uint32_t *const d = static_cast<uint32_t *>(dst);
+  const uint32_t *const g = static_cast<const uint32_t *>(src);
+  if (size == 4)
+    hipLaunchKernelGGL(wmmae_harness::cp_async_pipeline_kernel<4>, dim3(1),
+                       dim3(64), 0, s, d, g, groups, copies, pending);
+  else if (size == 8)
+    hipLaunchKernelGGL(wmmae_harness::cp_async_pipeline_kernel<8>, dim3(1),
+                       dim3(64), 0, s, d, g, groups, copies, pending);
+  else
+    hipLaunchKernelGGL(wmmae_harness::cp_async_pipeline_kernel<16>, dim3(1),
+                       dim3(64), 0, s, d, g, groups, copies, pending);
   return launch_status();
 }
 

@@ -40,6 +40,8 @@
 //   clock_samples_kernel    : (constant-rate clock, shader clock) pairs over time
 //   cp_async_kernel         : utils::cp_async global -> LDS copies
 //                             (reference: test/utils/cp_async.cu:15-25)
+//   cp_async_pipeline_kernel: the same calls as a three-stage pipeline
+//                             (commit / wait_group<2>, reference utils.hpp:29-64)
 //   cast_kernel             : utils::cast (reference: test/utils/cast.cu)
 //   print_fragment_kernel   : print_fragment of a primitive and a TCEC fragment
 //                             (reference: test/primitive/print_fragment.cu)
@@ -331,6 +333,26 @@ __global__ void __launch_bounds__(64)
   tcec::fill_zero(f);
   if (from_vector) {
     tcec::load_vector(f, src);
+  } else if (mem_col == 2) {
+    // the swizzled staging tile: src (rows of matrix_a / columns of matrix_b,
+    // N = 32 k each) is copied into LDS the way a GEMM stages it - lane l of a
+    // pass writes physical piece l % 8 of line l / 8 and fetches the logical
+    // piece that belongs there - and loaded with the swizzled layout tag
+    static_assert(N == 32, "lines of 32 k");
+    __shared__ __attribute__((aligned(16))) float tile[N * N];
+    const unsigned t = threadIdx.x;
+    namespace cpa = w::utils::cp_async;
+    for (unsigned l0 = 0; l0 < unsigned(N); l0 += 8) {
+      const unsigned line = l0 + t / 8;
+      const unsigned piece = (t % 8) ^ tcec::swizzled_piece(line);
+      cpa::cp_async<16>(tile + 4 * (8 * l0 + t), src + line * N + 4 * piece);
+    }
+    cpa::commit();
+    cpa::wait_all();
+    if constexpr (std::is_same<Use, w::matrix_a>::value)
+      tcec::load_matrix_sync<tcec::row_major_swizzled>(f, tile, N);
+    else
+      tcec::load_matrix_sync<tcec::col_major_swizzled>(f, tile, N);
   } else {
     if (mem_col)
       tcec::load_matrix_sync<w::col_major>(f, src, N);
@@ -821,6 +843,73 @@ __global__ void __launch_bounds__(128)
     cpa::wait_all();
     out(128 + t, &smem[1][t * W]);
   }
+}
+
+// utils::cp_async as a three-stage pipeline written with the reference's group
+// calls only (cp_async, commit, wait_group<2>; the use its utils.hpp:29-64 is
+// made for): one wave moves `groups` (<= 8) groups of `copies` (<= 4) copies
+// (64 lanes x Size bytes each) through a ring of three LDS buffers; while group
+// g is consumed, groups g+1 and g+2 are in flight.  The consumer moves a group
+// on inside LDS, and dst is written after the pipeline has drained, so that the
+// copies are the wave's only vector-memory instructions while it runs and
+// pending[] shows them alone: pending[0] is the wave's count of outstanding
+// vector-memory instructions (the hardware's own counter) once the first three
+// groups are out, pending[1 + g] the same right after the wait_group<2> that
+// releases group g, pending[1 + groups] after wait_all.
+template <unsigned Size>
+__global__ void __launch_bounds__(64)
+    cp_async_pipeline_kernel(uint32_t *const dst, const uint32_t *const src,
+                             const int groups, const int copies,
+                             int *const pending) {
+  namespace cpa = w::utils::cp_async;
+  constexpr unsigned W = Size / 4, STAGES = 3, MAX_COPIES = 4, MAX_GROUPS = 8;
+  constexpr unsigned GROUP_WORDS = MAX_COPIES * 64 * W;
+  __shared__ __attribute__((aligned(16))) uint32_t ring[STAGES][GROUP_WORDS];
+  __shared__ __attribute__((aligned(16))) uint32_t landed[MAX_GROUPS][GROUP_WORDS];
+  __shared__ int seen[MAX_GROUPS + 2];
+  const unsigned lane = threadIdx.x;
+  // vm_cnt of the wave: bits 3:0 and 23:22 of the instruction-buffer status
+  auto outstanding = [&]() {
+    const unsigned v = __builtin_amdgcn_s_getreg((31 << 11) | 7);
+    return static_cast<int>((v & 15u) | (((v >> 22) & 3u) << 4));
+  };
+  auto issue = [&](const int g) {
+    if (g < groups)
+      for (int c = 0; c < copies; c++)
+        cpa::cp_async<Size>(&ring[g % STAGES][(c * 64 + lane) * W],
+                            src + (static_cast<size_t>(g * copies + c) * 64 + lane) * W);
+    cpa::commit(); // (an empty group past the end keeps the group count in step)
+  };
+  for (int g = 0; g < static_cast<int>(STAGES); g++)
+    issue(g);
+  int now = outstanding();
+  if (lane == 0)
+    seen[0] = now;
+  for (int g = 0; g < groups; g++) {
+    cpa::wait_group<STAGES - 1>();
+    now = outstanding();
+    if (lane == 0)
+      seen[1 + g] = now;
+    for (int c = 0; c < copies; c++)
+      for (unsigned i = 0; i < W; i++)
+        landed[g][(c * 64 + lane) * W + i] =
+            ring[g % STAGES][(c * 64 + lane) * W + i];
+    // the buffer is refilled only after its contents have been read out
+    asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+    issue(g + STAGES);
+  }
+  cpa::wait_all();
+  now = outstanding();
+  if (lane == 0)
+    seen[1 + groups] = now;
+  __syncthreads();
+  for (int g = 0; g < groups; g++)
+    for (int c = 0; c < copies; c++)
+      for (unsigned i = 0; i < W; i++)
+        dst[(static_cast<size_t>(g * copies + c) * 64 + lane) * W + i] =
+            landed[g][(c * 64 + lane) * W + i];
+  for (int i = static_cast<int>(lane); i < groups + 2; i += 64)
+    pending[i] = seen[i];
 }
 
 // print_fragment of both layers, one wave: a 16x16x16 half matrix_a fragment

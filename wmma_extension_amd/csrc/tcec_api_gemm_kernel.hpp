@@ -12,14 +12,19 @@
 //     are 16 bytes wide) and multiplies with tcec::mma_sync;
 //   * the operand fragments are double buffered over the k steps of a stage.
 //
-// Rows of a staged tile are SK + 4 floats apart: sixteen lanes reading 16
-// bytes of sixteen consecutive rows then cover all 64 LDS banks once.  The
-// direct global->LDS copy of gfx950 writes lane-linear destinations only, so
-// the copy walks the padded tile image linearly, 16 bytes per lane
-// (cp_async_lane_linear), and lets the lanes that land on a row's padding
-// fetch that row's last piece again.
+// Rows of a staged tile are exactly SK = 32 floats (128 bytes), unpadded, with
+// the eight 16-byte pieces of row r stored at piece index p ^ ((r / 2) & 5)
+// (tcec::row_major_swizzled / col_major_swizzled): a 16-byte LDS read is served
+// sixteen lanes at a time - eight rows of one k group and eight rows of the
+// next - and with this permutation they hit all 64 banks once.  No row padding
+// does that (every padded stride costs a two-way conflict; the reference's
+// skew of 8 floats, batch_gemm.cu:11, is made for 32 banks and 32 lanes).  The
+// direct global->LDS copy of gfx950 writes lane-linear destinations, so the
+// copy walks the tile image linearly, 16 bytes per lane
+// (cp_async_lane_linear), and each lane fetches the logical piece that belongs
+// at its place.
 //
-// Two workgroups of four waves share a compute unit (72 KiB of LDS and at
+// Two workgroups of four waves share a compute unit (64 KiB of LDS and at
 // most 256 registers each, WAVES_PER_SIMD = 2): while one waits at its
 // barrier or for its copies, the other computes.  (One workgroup per compute
 // unit with up to 512 registers measured slower for every policy, the
@@ -45,36 +50,32 @@ struct ApiGemmShape {
   static constexpr int SK = 32;            // k per stage
   static constexpr int WM = 64, WN = 64;   // wave tile (2 x 2 waves)
   static constexpr int WK = 32;            // k per fragment
-  static constexpr int SKEW = 4;
-  static constexpr int LD = SK + SKEW;
+  static constexpr int LD = SK;            // unpadded rows, pieces swizzled
   static constexpr int STAGES = 2;
   static constexpr int THREADS = 256;
   static constexpr int STAGE_FLOATS = (BM + BN) * LD;
   static constexpr int LDS_BYTES = STAGES * STAGE_FLOATS * 4;
 };
 
-// Copy ROWS x SK floats (row r at src + r*ld) into a tile with rows LD apart.
-// A pass moves as many whole padded rows as the workgroup has lanes for (28
-// rows of nine 16-byte pieces with 256 threads; the last four threads idle),
-// so that a thread keeps its place inside a row and its source address moves
-// by the same amount from pass to pass.
-template <int ROWS, int SK, int LD, int THREADS>
+// Copy ROWS x SK floats (row r at src + r*ld) into a swizzled tile (see above).
+// A pass of the workgroup moves THREADS / 8 whole rows: thread t writes
+// physical piece t % 8 of row t / 8 and fetches the logical piece
+// (t % 8) ^ swizzled_piece(row) for it; the rows of a pass are a multiple of
+// 16, so a thread's logical piece and source offset are the same in every pass.
+template <int ROWS, int SK, int THREADS>
 __device__ __forceinline__ void stage_tile(float *const dst,
                                            const float *const src,
                                            const long long ld) {
-  constexpr int PR = LD / 4;             // 16-byte pieces per padded row
-  constexpr int RP = THREADS / PR;       // rows per pass
+  static_assert(SK == 32, "rows of 128 bytes");
+  constexpr int RP = THREADS / 8; // rows per pass
+  static_assert(RP % 16 == 0 && ROWS % RP == 0, "whole passes of whole rows");
   const int tid = static_cast<int>(threadIdx.x);
-  const int r_in = tid / PR;
-  int c = tid - r_in * PR;
-  c = c < SK / 4 ? c : SK / 4 - 1;       // padding: the last piece once more
+  const int r_in = tid / 8;
+  const int c = (tid % 8) ^ static_cast<int>(tcec::swizzled_piece(r_in));
   const float *const from = src + r_in * ld + 4 * c;
-  if (tid < RP * PR) {
 #pragma unroll
-    for (int r0 = 0; r0 < ROWS; r0 += RP)
-      if (r0 + RP <= ROWS || r0 + r_in < ROWS)
-        cpa::cp_async_lane_linear<16>(dst + 4 * (r0 * PR + tid), from + r0 * ld);
-  }
+  for (int r0 = 0; r0 < ROWS; r0 += RP)
+    cpa::cp_async_lane_linear<16>(dst + 4 * (r0 * 8 + tid), from + r0 * ld);
 }
 
 // C tile = alpha * A tile * B tile + beta * C tile for one 128 x 128 tile of
@@ -131,8 +132,8 @@ __global__ void __launch_bounds__(ApiGemmShape::THREADS, WAVES_PER_SIMD)
   auto stage_in = [&](const int stage, const int k0) {
     float *const sa = smem + stage * S::STAGE_FLOATS;
     float *const sb = sa + S::BM * S::LD;
-    stage_tile<S::BM, S::SK, S::LD, S::THREADS>(sa, a_base + k0, lda);
-    stage_tile<S::BN, S::SK, S::LD, S::THREADS>(sb, b_base + k0, ldb);
+    stage_tile<S::BM, S::SK, S::THREADS>(sa, a_base + k0, lda);
+    stage_tile<S::BN, S::SK, S::THREADS>(sb, b_base + k0, ldb);
     cpa::commit();
   };
 
@@ -154,13 +155,15 @@ __global__ void __launch_bounds__(ApiGemmShape::THREADS, WAVES_PER_SIMD)
     // fragments double buffered over the k steps of the stage
     FragA fa[2];
     FragB fb[2];
-    tcec::load_matrix_sync(fa[0], sa, S::LD, false);
-    tcec::load_matrix_sync(fb[0], sb, S::LD, false);
+    tcec::load_matrix_sync<tcec::row_major_swizzled>(fa[0], sa, S::LD, false);
+    tcec::load_matrix_sync<tcec::col_major_swizzled>(fb[0], sb, S::LD, false);
 #pragma unroll
     for (int kk = S::WK; kk < S::SK; kk += S::WK) {
       const int cur = (kk / S::WK) & 1;
-      tcec::load_matrix_sync(fa[cur], sa + kk, S::LD, false);
-      tcec::load_matrix_sync(fb[cur], sb + kk, S::LD, false);
+      tcec::load_matrix_sync<tcec::row_major_swizzled>(fa[cur], sa + kk, S::LD,
+                                                       false);
+      tcec::load_matrix_sync<tcec::col_major_swizzled>(fb[cur], sb + kk, S::LD,
+                                                       false);
       tcec::mma_sync(fc, fa[1 - cur], fb[1 - cur], fc);
     }
     constexpr int last = ((S::SK / S::WK) - 1) & 1;

@@ -48,6 +48,31 @@ __device__ __forceinline__ void static_for(F &&f) {
 __host__ __device__ constexpr unsigned direct_swizzle(const unsigned q) {
   return 12u * (q & 1u) ^ 4u * (q >> 1);
 }
+// DIRECT == 2 (rows of k floats, k not a multiple of 32): the pieces of a
+// lane's read address in a row's last, shorter stage, shared by the kernel and
+// by a host-side check that no read leaves its row.  A lane reads four floats;
+// the one whose four would end past the row reads the row's last four instead.
+//   kDirectBias       : floats by which the row block's base is moved back and
+//                       every lane offset forward, so that a lane reading up
+//                       to three floats before the stage's start keeps an
+//                       offset >= 0
+//   direct_tail_shift : floats a lane moves back, `left` = floats from the
+//                       stage's start to the row's end
+//   direct_read_first : first float, counted from the row's start, that lane
+//                       `lane` reads in stage `stage` (`tail`: that variant)
+constexpr int kDirectBias = 4;
+__host__ __device__ constexpr int direct_tail_shift(const unsigned lane,
+                                                    const int left) {
+  const int s = 4 * static_cast<int>(lane & 7u) + 4 - left;
+  return s > 0 ? s : 0;
+}
+__host__ __device__ constexpr long long
+direct_read_first(const bool tail, const int k, const int stage,
+                  const unsigned lane) {
+  const long long base = 32ll * stage - (tail ? kDirectBias : 0);
+  const long long lane_off = 4ll * (lane & 7u) + (tail ? kDirectBias : 0);
+  return base + lane_off - (tail ? direct_tail_shift(lane, k - 32 * stage) : 0);
+}
 // Number of LDS reads that have been issued once `count` MFMAs of a step are
 // out: read r is due after MFMA number (r+1)*span/nfrag.
 __host__ __device__ constexpr int reads_due(const int count, const int span,
@@ -583,8 +608,7 @@ __global__ void __launch_bounds__(WGM *WGN * 64)
   int req_left = 0, raw_left = 0;
   unsigned tail_off = 0;
   auto tail_shift = [&](const int left) {
-    const int s = 4 * static_cast<int>(lane & 7u) + 4 - left;
-    return s > 0 ? s : 0;
+    return direct_tail_shift(lane, left);
   };
   auto set_tail_off = [&]() {
     if constexpr (TAIL)
@@ -622,14 +646,15 @@ __global__ void __launch_bounds__(WGM *WGN * 64)
         // reads up to three floats before the stage's start - rows that end
         // one to three floats into their last stage - keeps an offset >= 0)
         gsrc[g] = reinterpret_cast<unsigned long long>(
-            (is_a ? Ab : Bb) + row0 * ld + first_stage * 32 - (TAIL ? 4 : 0));
+            (is_a ? Ab : Bb) + row0 * ld + first_stage * 32 -
+            (TAIL ? kDirectBias : 0));
         asm volatile("" : "+s"(gsrc[g]));
 #pragma unroll
         for (int h = 0; h < 2; h++) {
           int mine = row0 + 8 * h + static_cast<int>(lane >> 3);
           mine = (mine < last ? mine : last) - row0;
           voff[g][h] = static_cast<unsigned>(mine * ld) * 4u +
-                       16u * (lane & 7u) + (TAIL ? 16u : 0u);
+                       16u * (lane & 7u) + (TAIL ? 4u * kDirectBias : 0u);
         }
       }
       return;

@@ -350,6 +350,19 @@ def utils_cp_async(size, mode, src):
     return dst
 
 
+def utils_cp_async_pipeline(size, copies, groups, src):
+    """src: groups * copies * 64 elements of `size` bytes (CUDA).  Returns (the copy made by a
+    three-stage cp_async / commit / wait_group<2> pipeline of one wave, the wave's outstanding
+    vector-memory instructions at start, after every wait_group and at the end)."""
+    _need_cuda(src)
+    dst = torch.full_like(src, -1)
+    pending = torch.full((groups + 2,), -1, dtype=torch.int32, device=src.device)
+    st = _lib.lib().wmmae_utils_cp_async_pipeline(size, copies, groups, _ptr(dst), _ptr(src),
+                                                  _ptr(pending), _stream())
+    _lib.check(st, "wmmae_utils_cp_async_pipeline")
+    return dst, pending
+
+
 def print_fragment(type_, ec, src, base):
     """Device printf of a primitive and a TCEC fragment (one wave) to the process's stdout."""
     _need_cuda(src)
