@@ -134,7 +134,8 @@ __global__ void __launch_bounds__(ApiGemmShape::THREADS, WAVES_PER_SIMD)
     float *const sb = sa + S::BM * S::LD;
     stage_tile<S::BM, S::SK, S::THREADS>(sa, a_base + k0, lda);
     stage_tile<S::BN, S::SK, S::THREADS>(sb, b_base + k0, ldb);
-    cpa::commit();
+    // (no cp_async::commit(): the loop waits with wait_all(), which needs no
+    // groups, and commit() costs a round trip to its bookkeeping in LDS)
   };
 
   stage_in(0, 0);

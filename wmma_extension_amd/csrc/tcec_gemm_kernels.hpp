@@ -1255,6 +1255,8 @@ __global__ void __launch_bounds__(WGM *WGN * 64)
       asm volatile("s_nop 15\n\ts_nop 15" ::: "memory");
     else
       asm volatile("s_waitcnt vmcnt(0)\n\ts_nop 15\n\ts_nop 15" ::: "memory");
+    // (the reads of the accumulators must not be scheduled above the no-ops)
+    __builtin_amdgcn_sched_barrier(0);
     skip_waits = NSTAGE - 1;
     store_item(it);
   }
