@@ -39,6 +39,24 @@ int wmmae_mfma_probe(int type, int m, int n, int k, float *d,
 int wmmae_direct_read_first(int tail, int k, int stage, int lane,
                             long long *first);
 
+/* Host only (no counterpart in the reference): the number of K slices
+ * wmmae_tcec_sgemm* cuts a product into on the path it takes for these
+ * arguments (flags as there, path flags included; a workspace of
+ * wmmae_tcec_sgemm_workspace_bytes assumed).  1: K is not cut, or the single
+ * kernel runs.  The two GEMM kernels plan their slices for their own tiles, so
+ * the counts of the forced packed and the forced direct path may differ - and
+ * with them the last bits of C, since the slices' partial sums are rounded. */
+int wmmae_tcec_sgemm_k_slices(int m, int n, int k, int batch, int policy,
+                              int flags, int *slices);
+
+/* Test hook (no counterpart in the reference): the calling thread's next
+ * wmmae_tcec_sgemm* / wmmae_tcec_gemm_packed calls and workspace queries cut K
+ * into `slices` slices (at most 32, at least six k stages of 32 each: smaller
+ * products get fewer) instead of what the time estimates choose; 0 restores
+ * the estimates.  For running two paths on the same cut of K, where they give
+ * the same bits. */
+int wmmae_tcec_force_k_slices(int slices);
+
 #ifdef __cplusplus
 }
 #endif

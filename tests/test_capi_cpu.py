@@ -24,7 +24,8 @@ def test_header_and_library_agree(h):
     declared = set(re.findall(r"\b(wmmae_[a-z0-9_]+)\s*\(", text))
     declared_aux = set(re.findall(r"\b(wmmae_[a-z0-9_]+)\s*\(", aux))
     # the measurement aids live in their own header, outside the product ABI
-    assert declared_aux == {"wmmae_clock_samples", "wmmae_mfma_probe", "wmmae_direct_read_first"} and not (declared & declared_aux)
+    assert declared_aux == {"wmmae_clock_samples", "wmmae_mfma_probe", "wmmae_direct_read_first",
+                            "wmmae_tcec_sgemm_k_slices", "wmmae_tcec_force_k_slices"} and not (declared & declared_aux)
     declared |= declared_aux
     assert declared == set(_lib.EXPORTS)
     for name in declared:
@@ -228,13 +229,64 @@ def test_slice_counts_the_estimates_choose():
         return out.value // (m * n * batch * 4)
     assert planes(0, 1024, 1024, 262144) == 8
     assert planes(2, 1024, 1024, 262144) == 8    # three terms: 256x128 tiles too, one slice per XCD
-    assert planes(0, 1024, 1024, 4096) == 4
+    # room for the larger of the two kernels' plans: four slices of 128x128 tiles on packed
+    # operands, eight for the kernel that splits the fp32 operands itself (32 tiles of 256x128)
+    assert planes(0, 1024, 1024, 4096) == 8
+    assert planes(2, 1024, 1024, 4096) == 4      # three terms: packed operands only
     assert planes(0, 1280, 1280, 4096) == 5      # 250 tiles of 256x128: one round
     assert planes(0, 512, 512, 1024) == 5
     assert planes(0, 1000, 900, 50000, 2) == 4
     out = ctypes.c_int(-1)
     for shape in ((1792, 1792, 4096), (2048, 2048, 2048)):
         assert h.wmmae_tcec_sgemm_path(*shape, 1, 0, 0, ctypes.byref(out)) == 0 and out.value == 1, shape
+
+
+def test_k_slice_query_and_hook(h):
+    """The slice count per path, and the hook that fixes it for the calling thread: the forced
+    count is canonical (no empty slices), at most 32, at least six stages a slice, shows in the
+    workspace query, and 0 hands the choice back to the estimates."""
+    out = ctypes.c_int(-1)
+    ws = ctypes.c_size_t(0)
+    def slices(m, n, k, batch, policy, flags):
+        assert h.wmmae_tcec_sgemm_k_slices(m, n, k, batch, policy, flags, ctypes.byref(out)) == 0
+        return out.value
+    PACKED, FUSED, DIRECT = 2, 4, 8
+    assert slices(1024, 1024, 4096, 1, 0, PACKED) == 4 and slices(1024, 1024, 4096, 1, 0, DIRECT) == 8
+    assert slices(1024, 1024, 4096, 1, 0, FUSED) == 1
+    assert slices(1024, 1024, 262144, 1, 0, 0) == 8 and slices(4096, 4096, 4096, 1, 0, 0) == 1
+    assert slices(0, 16, 16, 1, 0, 0) == 1
+    assert h.wmmae_tcec_sgemm_k_slices(64, 64, 64, 1, 2, DIRECT, ctypes.byref(out)) == -4   # three terms
+    assert h.wmmae_tcec_sgemm_k_slices(64, 64, 64, 1, 0, 16, ctypes.byref(out)) == -1
+    assert h.wmmae_tcec_sgemm_k_slices(64, 64, 64, 1, 0, 0, None) == -2
+    try:
+        assert h.wmmae_tcec_force_k_slices(5) == 0
+        assert slices(4096, 4096, 4096, 1, 0, PACKED) == 5 and slices(4096, 4096, 4096, 1, 0, DIRECT) == 5
+        h.wmmae_tcec_gemm_packed_workspace_bytes.argtypes = [ctypes.c_int] * 5 + [ctypes.POINTER(ctypes.c_size_t)]
+        assert h.wmmae_tcec_gemm_packed_workspace_bytes(0, 512, 512, 4096, 1, ctypes.byref(ws)) == 0
+        assert ws.value == 5 * 512 * 512 * 4
+        assert slices(512, 512, 32 * 33, 1, 0, PACKED) == 5       # 33 stages: 7 7 7 7 5
+        assert slices(512, 512, 32 * 35, 1, 0, PACKED) == 5
+        assert slices(512, 512, 32 * 29, 1, 0, PACKED) == 4       # at least six stages a slice
+        assert slices(512, 512, 64, 1, 0, PACKED) == 1
+        assert h.wmmae_tcec_force_k_slices(7) == 0
+        assert slices(512, 512, 32 * 48, 1, 0, PACKED) == 7       # 7 7 7 7 7 7 6
+        assert slices(512, 512, 32 * 45, 1, 0, PACKED) == 7
+        assert h.wmmae_tcec_force_k_slices(24) == 0
+        assert slices(512, 512, 32 * 150, 1, 0, PACKED) == 22     # 7 stages a slice: 22 slices, no empty one
+        assert h.wmmae_tcec_force_k_slices(100) == 0
+        assert slices(512, 512, 1 << 20, 1, 0, DIRECT) == 32
+        assert h.wmmae_tcec_force_k_slices(-1) == -1
+    finally:
+        assert h.wmmae_tcec_force_k_slices(0) == 0
+    assert slices(4096, 4096, 4096, 1, 0, PACKED) == 1
+    # the hook belongs to the thread that set it
+    import threading
+    seen = []
+    assert h.wmmae_tcec_force_k_slices(3) == 0
+    t = threading.Thread(target=lambda: seen.append(slices(4096, 4096, 4096, 1, 0, PACKED)))
+    t.start(); t.join()
+    assert seen == [1] and slices(4096, 4096, 4096, 1, 0, PACKED) == 3
+    assert h.wmmae_tcec_force_k_slices(0) == 0
 
 
 def test_direct_kernel_reads_stay_inside_their_rows(h):

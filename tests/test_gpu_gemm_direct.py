@@ -2,7 +2,12 @@
 splitting them on their way into LDS (WMMAE_FLAG_PATH_DIRECT forces it, the time estimates
 choose it for batches of medium-sized matrices and K-heavy products).  It issues the same
 products in the same order as the packed path, so every case compares bits with the packed
-path forced on the same arguments; one case per group is also held against FP64."""
+path forced on the same arguments; one case per group is also held against FP64.
+
+Where K is cut into slices the two kernels plan the cut for their own tiles (256x128 only for
+this kernel, 128x128 and 64x64 too for the packed path), and the slices' partial sums are
+rounded: the direct path runs on its own plan, as a caller gets it, and the packed path is
+given the same number of slices for the comparison."""
 import numpy as np
 import pytest
 import torch
@@ -27,10 +32,12 @@ def _both(tc, dev, m, n, k, batch, policy, lda=None, ldb=None, ldc=None, alpha=1
     ws = (torch.empty(tc.workspace_bytes(m, n, k, batch, policy), dtype=torch.uint8, device=dev)
           if workspace else None)
     out = []
+    slices = tc.sgemm_k_slices(m, n, k, batch, policy, DIRECT)
     for flag in (DIRECT, PACKED):
         C = C0.clone()
-        tc.sgemm_strided_batched("T", "N", m, n, k, alpha, A[a_off:], lda, m * lda, B[b_off:], ldb,
-                                 n * ldb, beta, C, ldc, n * ldc, batch, policy, flag, ws)
+        with tc.forced_k_slices(slices if flag == PACKED else 0):
+            tc.sgemm_strided_batched("T", "N", m, n, k, alpha, A[a_off:], lda, m * lda, B[b_off:],
+                                     ldb, n * ldb, beta, C, ldc, n * ldc, batch, policy, flag, ws)
         out.append(C)
     torch.cuda.synchronize()
     return out, A[a_off:], B[b_off:], C0
@@ -65,10 +72,11 @@ def test_direct_path_any_leading_dimension_and_base(tc, dev, policy):
 
 @pytest.mark.parametrize("policy", [0, 3])
 def test_direct_path_k_slices(tc, orc, dev, policy):
-    """A K-heavy product: with room for the slices both paths cut K the same way and fold the
-    slices in the same order; without a workspace the direct path allocates the planes
-    itself."""
+    """A K-heavy product: on the same cut of K both paths fold the slices in the same order;
+    without a workspace the direct path allocates the planes itself.  Then every slice count
+    from one to nine forced on both paths."""
     m, n, k = 512, 384, 16384
+    assert tc.sgemm_k_slices(m, n, k, 1, policy, DIRECT) > 1
     (d, p), A, B, _ = _both(tc, dev, m, n, k, 1, policy)
     assert torch.equal(d, p)
     (d2, _), _, _, _ = _both(tc, dev, m, n, k, 1, policy, workspace=False)
@@ -79,6 +87,22 @@ def test_direct_path_k_slices(tc, orc, dev, policy):
     assert torch.equal(d4, d3)
     ref = orc.gemm_f64(A.view(m, k).cpu().numpy(), B.view(n, k).cpu().numpy().T)
     assert orc.max_rel_err(d.view(n, m).cpu().numpy().T, ref) < {0: 4e-6, 3: 2e-4}[policy]
+    seen = set()
+    for s in range(1, 10):
+        res = []
+        with tc.forced_k_slices(s):
+            assert tc.sgemm_k_slices(m, n, k, 1, policy, DIRECT) == s
+            ws = torch.empty(tc.workspace_bytes(m, n, k, 1, policy), dtype=torch.uint8, device=dev)
+            for flag in (DIRECT, PACKED):
+                C = torch.zeros((n, m), dtype=torch.float32, device=dev)
+                tc.sgemm("T", "N", m, n, k, 1.0, A[:m * k], k, B[:n * k], k, 0.0, C, m, policy, flag, ws)
+                res.append(C)
+        torch.cuda.synchronize()
+        assert torch.equal(res[0], res[1]), s
+        assert orc.max_rel_err(res[0].cpu().numpy().T, ref) < {0: 4e-6, 3: 2e-4}[policy]
+        seen.add(res[0].cpu().numpy().tobytes())
+    assert len(seen) > 1                     # the cut does show in the last bits
+    assert tc.sgemm_k_slices(m, n, k, 1, policy, DIRECT) > 1      # the hook is off again
 
 
 @pytest.mark.parametrize("policy", [0, 1, 3, 4])

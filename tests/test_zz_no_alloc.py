@@ -2,6 +2,8 @@
 wmmae_tcec_sgemm on a caller-provided workspace: same bits, on two calls in a row,
 the second with a smaller input so that the first call's leftovers in the shared
 array would show."""
+import gc
+
 import pytest
 import torch
 
@@ -111,6 +113,7 @@ def test_static_calls_allocate_nothing(dev):
             tcec.sgemm_static("T", "N", m, n, k, 1.0, A, k, Bt, k, 0.0, C0, m, pol, flags)
         torch.cuda.synchronize()
     run_all()
+    gc.collect()          # tensors that earlier tests left to the collector go now, not below
     free0, _ = torch.cuda.mem_get_info(dev)
     alloc0, reserved0 = torch.cuda.memory_allocated(dev), torch.cuda.memory_reserved(dev)
     for _ in range(3):

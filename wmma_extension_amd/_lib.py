@@ -63,6 +63,8 @@ EXPORTS = [
     "wmmae_utils_cast",
     "wmmae_mfma_probe",
     "wmmae_direct_read_first",
+    "wmmae_tcec_sgemm_k_slices",
+    "wmmae_tcec_force_k_slices",
 ]
 
 
@@ -147,6 +149,8 @@ _SIGNATURES = {
     "wmmae_utils_cast": (_i, [_i, _vp, _vp, _ll, _vp]),
     "wmmae_mfma_probe": (_i, [_i, _i, _i, _i, _vp, _vp, _vp, _vp, _vp]),
     "wmmae_direct_read_first": (_i, [_i, _i, _i, _i, _c.POINTER(_ll)]),
+    "wmmae_tcec_sgemm_k_slices": (_i, [_i, _i, _i, _i, _i, _i, _c.POINTER(_i)]),
+    "wmmae_tcec_force_k_slices": (_i, [_i]),
 }
 
 

@@ -239,8 +239,11 @@ constexpr PathRates kPacked[3] = {{8.9e-6, 0.31e-6, 2.0e-6, 5.0e12, 6.6e12},
 //    1.0 us), a tile 6 us on top.
 constexpr PathRates kDirect[2] = {{6.0e-6, 0.40e-6, 3.0e-6, 5.0e12, 0.},
                                   {6.0e-6, 0.75e-6, 3.0e-6, 5.0e12, 0.}};
-// with K slices: the GEMM's time against the same kernel on packed operands
-constexpr double kDirectSliceRatio[2] = {1.5, 1.5};
+// with K slices: the GEMM's time against the packed kernel's estimate for the
+// same slices of 256x128 tiles (two terms: twelve K-sliced products, m, n =
+// 64 .. 4096, k = 2048 .. 262144, each run on either path: with 1.4 the faster
+// path is chosen for all of them, with 1.5 for eleven)
+constexpr double kDirectSliceRatio[2] = {1.5, 1.4};
 // k % 32 != 0: the kernel variant that reads a shorter last stage (1024^2 x 1000
 // against x 1024, batch 256: 301 against 336 TFLOPS, of which 2.4 % are the k)
 constexpr double kDirectTailStage = 1.09;
@@ -288,8 +291,14 @@ inline bool big_tile_candidate(const int terms, const long long mid,
                                const int kt) {
   return mid > device_cus() && !(terms == 1 && kt <= 32);
 }
+// `direct`: the kernel that splits the fp32 operands itself, which has the
+// 256x128 tile only and takes kDirectSliceRatio times the packed kernel's time
+// (its slice count must be planned with its own tiles: 4096 x 64 x 4096 cut
+// for the 128x128 tiles of the packed path left half the compute units
+// without a 256x128 item, 48 against 39 us).
 inline double split_time(const int terms, const int m, const int n,
-                         const int batch, const int kt, const int slices) {
+                         const int batch, const int kt, const int slices,
+                         const bool direct = false) {
   const long long cus = device_cus();
   const int stages = static_cast<int>(ceil_div(kt, slices));
   const long long z = ceil_div(kt, stages);
@@ -298,8 +307,9 @@ inline double split_time(const int terms, const int m, const int n,
   double stage_time, rounds;
   const double r_big = static_cast<double>(ceil_div(big, cus));
   const double r_mid = static_cast<double>(ceil_div(mid, cus));
-  if (big_tile_candidate(terms, mid, stages) &&
-      r_big * fit::units256x128(terms) <= r_mid * fit::units128x128(terms)) {
+  if (direct ||
+      (big_tile_candidate(terms, mid, stages) &&
+       r_big * fit::units256x128(terms) <= r_mid * fit::units128x128(terms))) {
     stage_time = fit::kStage256x128[terms - 1];
     rounds = r_big;
   } else if (mid >= cus || (m > 64 && n > 64)) {
@@ -314,20 +324,31 @@ inline double split_time(const int terms, const int m, const int n,
   if (z > 1)
     t += fit::kFoldLaunch + static_cast<double>(z + 1) * m * n * batch * 4.0 /
                                 fit::kFoldBytesPerS;
-  return t;
+  return direct ? t * fit::kDirectSliceRatio[terms - 1] : t;
 }
+// Test hook (wmmae_tcec_force_k_slices): a slice count for the calling thread's
+// next calls instead of the estimates' choice, so that two kernels can be run on
+// the same cut of K and compared bit by bit.  0: the estimates choose.
+thread_local int t_forced_k_slices = 0;
+constexpr int kMaxSplits = 32, kMinStagesPerSplit = 6;
 inline int choose_splits(const int terms, const int m, const int n, const int k,
-                         const int batch) {
+                         const int batch, const bool direct = false) {
   const long long tiles = ceil_div(m, 256) * ceil_div(n, 128) * batch;
   const int kt = static_cast<int>(ceil_div(k, 32));
+  if (t_forced_k_slices > 0) {
+    const int s = std::max(
+        1, std::min({t_forced_k_slices, kMaxSplits, kt / kMinStagesPerSplit}));
+    return static_cast<int>(ceil_div(kt, ceil_div(kt, s)));
+  }
   if (tiles * 2 > device_cus())
     return 1;
   int best = 1;
-  double t_best = fit::kSplitMustBeat * split_time(terms, m, n, batch, kt, 1);
-  for (int s = 2; s <= 32 && s * 6 <= kt; s++) {
+  double t_best =
+      fit::kSplitMustBeat * split_time(terms, m, n, batch, kt, 1, direct);
+  for (int s = 2; s <= kMaxSplits && s * kMinStagesPerSplit <= kt; s++) {
     if (ceil_div(kt, ceil_div(kt, s)) != s)
       continue; // the same slices as a smaller count
-    const double t = split_time(terms, m, n, batch, kt, s);
+    const double t = split_time(terms, m, n, batch, kt, s, direct);
     if (t < t_best) {
       t_best = t;
       best = s;
@@ -774,16 +795,19 @@ inline Path choose_path(const int m, const int n, const int k, const int batch,
   const int splits = choose_splits(terms, m, n, k, batch);
   if (splits != 1) {
     // K slices: the split pass against the slower stages of the direct kernel
+    // (cut into the slices that suit its own tile)
     if (!direct_ok)
       return Path::Packed;
     const fit::PathRates &pk = fit::kPacked[terms - 1];
     const double ab = (static_cast<double>(m) + n) * k * batch;
-    const double gemm = split_time(terms, m, n, batch,
-                                   static_cast<int>(ceil_div(k, 32)), splits);
+    const int kt = static_cast<int>(ceil_div(k, 32));
     const double t_packed =
-        pk.launch + (4.0 + 2.0 * terms) * ab / pk.split_bytes_per_s + gemm;
+        pk.launch + (4.0 + 2.0 * terms) * ab / pk.split_bytes_per_s +
+        split_time(terms, m, n, batch, kt, splits);
     const double t_direct =
-        fit::kDirect[terms - 1].launch + gemm * fit::kDirectSliceRatio[terms - 1];
+        fit::kDirect[terms - 1].launch +
+        split_time(terms, m, n, batch, kt,
+                   choose_splits(terms, m, n, k, batch, true), true);
     return t_direct < t_packed ? Path::Direct : Path::Packed;
   }
   const bool fused_allowed = fused_vec || k <= 96;
@@ -967,7 +991,7 @@ int pack_impl(const int policy, const int rows, const int k,
 // supplied room for the slices
 void plan_k_slices(GemmArgs &g, void *const workspace,
                    const size_t workspace_bytes) {
-  g.splits = choose_splits(g.terms, g.m, g.n, g.k, g.batch);
+  g.splits = choose_splits(g.terms, g.m, g.n, g.k, g.batch, g.is_direct);
   g.partial = nullptr;
   g.tail_ws = nullptr;
   g.tail_ws_bytes = 0;
@@ -1267,9 +1291,15 @@ int wmmae_tcec_gemm_packed_workspace_bytes(const int policy, const int m,
     return WMMAE_STATUS_NULL_POINTER;
   if (!policy_info(policy, p) || m < 0 || n < 0 || k < 0 || batch < 0)
     return WMMAE_STATUS_INVALID_VALUE;
-  const int splits = (m == 0 || n == 0 || k == 0 || batch == 0)
-                         ? 1
-                         : choose_splits(p.terms, m, n, k, batch);
+  // (room for the slices of either kernel: the one that splits the fp32
+  // operands itself plans them for its own tile)
+  const int splits =
+      (m == 0 || n == 0 || k == 0 || batch == 0)
+          ? 1
+          : std::max(choose_splits(p.terms, m, n, k, batch),
+                     direct_possible(k, p.terms, 0, 1, 1)
+                         ? choose_splits(p.terms, m, n, k, batch, true)
+                         : 1);
   if (splits > 1) {
     *bytes = static_cast<size_t>(splits) * batch * m * n * 4u;
   } else if (batch == 1 && m > 0 && n > 0) {
@@ -1305,19 +1335,57 @@ int wmmae_tcec_sgemm_path(const int m, const int n, const int k,
   if (m < 0 || n < 0 || k < 0 || batch < 0 || !policy_info(policy, p) ||
       (flags & ~WMMAE_FLAG_RN_MAIN) != 0)
     return WMMAE_STATUS_INVALID_VALUE;
-  const bool slices = m > 0 && n > 0 && k > 0 && batch > 0 &&
-                      choose_splits(p.terms, m, n, k, batch) > 1;
+  const bool any = m > 0 && n > 0 && k > 0 && batch > 0;
+  const bool slices = any && choose_splits(p.terms, m, n, k, batch) > 1;
   switch (choose_path(m, n, k, batch, flags, p.terms, policy, true,
                       direct_possible(k, p.terms, flags, 1, 1))) {
   case Path::Fused:
     *path = 0;
     break;
   case Path::Direct:
-    *path = slices ? 4 : 3;
+    *path = any && choose_splits(p.terms, m, n, k, batch, true) > 1 ? 4 : 3;
     break;
   default:
     *path = slices ? 2 : 1;
   }
+  return WMMAE_STATUS_SUCCESS;
+}
+
+int wmmae_tcec_force_k_slices(const int slices) {
+  if (slices < 0)
+    return WMMAE_STATUS_INVALID_VALUE;
+  t_forced_k_slices = slices;
+  return WMMAE_STATUS_SUCCESS;
+}
+
+int wmmae_tcec_sgemm_k_slices(const int m, const int n, const int k,
+                              const int batch, const int policy,
+                              const int flags, int *const slices) {
+  PolicyInfo p;
+  if (slices == nullptr)
+    return WMMAE_STATUS_NULL_POINTER;
+  constexpr int kPathFlags = WMMAE_FLAG_PATH_PACKED | WMMAE_FLAG_PATH_FUSED |
+                             WMMAE_FLAG_PATH_DIRECT;
+  if (m < 0 || n < 0 || k < 0 || batch < 0 || !policy_info(policy, p) ||
+      (flags & ~(WMMAE_FLAG_RN_MAIN | kPathFlags)) != 0)
+    return WMMAE_STATUS_INVALID_VALUE;
+  *slices = 1;
+  if (m == 0 || n == 0 || k == 0 || batch == 0)
+    return WMMAE_STATUS_SUCCESS;
+  const bool direct_ok = direct_possible(k, p.terms, flags, 1, 1);
+  Path path = choose_path(m, n, k, batch, flags & WMMAE_FLAG_RN_MAIN, p.terms,
+                          policy, true, direct_ok);
+  if ((flags & WMMAE_FLAG_PATH_DIRECT) != 0) {
+    if (!direct_ok)
+      return WMMAE_STATUS_NOT_SUPPORTED;
+    path = Path::Direct;
+  } else if ((flags & WMMAE_FLAG_PATH_FUSED) != 0) {
+    path = Path::Fused;
+  } else if ((flags & WMMAE_FLAG_PATH_PACKED) != 0) {
+    path = Path::Packed;
+  }
+  if (path != Path::Fused)
+    *slices = choose_splits(p.terms, m, n, k, batch, path == Path::Direct);
   return WMMAE_STATUS_SUCCESS;
 }
 

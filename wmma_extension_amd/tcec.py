@@ -117,6 +117,30 @@ def sgemm_path(m, n, k, batch=1, policy=Policy.F16_EC, flags=0):
     return out.value
 
 
+def sgemm_k_slices(m, n, k, batch=1, policy=Policy.F16_EC, flags=0):
+    """How many K slices the GEMM entry points cut this product into on the path `flags`
+    select (1: none)."""
+    out = ctypes.c_int(-1)
+    _lib.check(_lib.lib().wmmae_tcec_sgemm_k_slices(m, n, k, batch, int(policy), flags,
+                                                    ctypes.byref(out)), "wmmae_tcec_sgemm_k_slices")
+    return out.value
+
+
+class forced_k_slices:
+    """Test aid: within the block, this thread's GEMM calls cut K into `slices` slices."""
+
+    def __init__(self, slices):
+        self.slices = slices
+
+    def __enter__(self):
+        _lib.check(_lib.lib().wmmae_tcec_force_k_slices(self.slices), "wmmae_tcec_force_k_slices")
+        return self
+
+    def __exit__(self, *exc):
+        _lib.lib().wmmae_tcec_force_k_slices(0)
+        return False
+
+
 def pack_bytes(rows, k, batch=1, policy=Policy.F16_EC):
     out = ctypes.c_size_t(0)
     _lib.check(_lib.lib().wmmae_tcec_pack_bytes(rows, k, batch, int(policy), ctypes.byref(out)),
