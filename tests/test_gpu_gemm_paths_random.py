@@ -1,0 +1,83 @@
+"""Random products through every path of the driver (the library's choice, and the packed, the
+single-kernel and the direct path forced), all four transpose combinations, padded leading
+dimensions, alpha / beta, one to forty entries, dimensions that are no multiples of anything:
+
+  * every result within the policy's tolerance of FP64 (reference metric, test/primitive/common.hpp:54-103);
+  * the padding of C untouched;
+  * the default call gives the bits of the forced path it reports (wmmae_tcec_sgemm_path);
+  * the paths give each other's bits wherever they cut K alike (they issue the same products in the
+    same order on the same accumulators).
+"""
+import random
+
+import pytest
+import torch
+
+pytestmark = pytest.mark.gpu
+
+PACKED, FUSED, DIRECT = 2, 4, 8
+TOL = {0: 4e-6, 1: 3e-3, 2: 4e-6, 3: 3e-4, 4: 3e-2}
+
+
+def _cases(seed, count):
+    rnd = random.Random(seed)
+
+    def dim(lo, hi):
+        return max(1, int(2 ** rnd.uniform(lo, hi)) + rnd.choice([0, 0, 0, 1, -1, 3, 5, 17]))
+    out = []
+    while len(out) < count:
+        batch = rnd.choice([1, 1, 1, 2, 3, 5, 9, 17, 40])
+        m, n = dim(3, 11.5), dim(3, 11.5)
+        k = dim(2, 14.5) if batch == 1 else dim(2, 11)
+        if (m * k + n * k + m * n) * batch * 4 > 3e8 or 2.0 * m * n * k * batch > 1e11:
+            continue
+        out.append(dict(m=m, n=n, k=k, batch=batch, policy=rnd.choice([0, 0, 1, 2, 3, 4]),
+                        trans=rnd.choice([("T", "N")] * 3 + [("N", "N"), ("N", "T"), ("T", "T")]),
+                        ab=rnd.choice([(1.0, 0.0), (1.0, 0.0), (1.5, -0.25), (-0.5, 1.0)]),
+                        pad=rnd.choice([0, 0, 1, 4, 7])))
+    return out
+
+
+@pytest.mark.parametrize("seed", [11, 12, 13])
+def test_random_products_on_every_path(tc, dev, seed):
+    from wmma_extension_amd._lib import WmmaeError
+    for it, c in enumerate(_cases(seed, 60)):
+        m, n, k, batch, policy, pad = c["m"], c["n"], c["k"], c["batch"], c["policy"], c["pad"]
+        (ta, tb), (alpha, beta) = c["trans"], c["ab"]
+        lda = (k if ta == "T" else m) + pad
+        ldb = (k if tb == "N" else n) + pad
+        ldc = m + pad
+        g = torch.Generator(device="cpu").manual_seed(seed * 100003 + it)
+        A = (torch.rand((batch, (m if ta == "T" else k), lda), generator=g) * 2 - 1).to(dev)
+        B = (torch.rand((batch, (n if tb == "N" else k), ldb), generator=g) * 2 - 1).to(dev)
+        C0 = (torch.rand((batch, n, ldc), generator=g) * 2 - 1).to(dev)
+        a_op = A[:, :, :k].double() if ta == "T" else A[:, :, :m].double().transpose(1, 2)
+        b_op = B[:, :, :k].double() if tb == "N" else B[:, :, :n].double().transpose(1, 2)
+        ref = alpha * torch.bmm(b_op, a_op.transpose(1, 2)) + beta * C0[:, :, :m].double()
+        scale = ref.abs().max().item() + 1e-30
+        res, slices = {}, {}
+        for flag in (0, PACKED, FUSED, DIRECT):
+            C = C0.clone()
+            ws = torch.empty(max(16, tc.workspace_bytes(m, n, k, batch, policy)), dtype=torch.uint8, device=dev)
+            try:
+                slices[flag] = tc.sgemm_k_slices(m, n, k, batch, policy, flag)
+                tc.sgemm_strided_batched(ta, tb, m, n, k, alpha, A, lda, A.stride(0), B, ldb, B.stride(0),
+                                         beta, C, ldc, n * ldc, batch, policy, flag, ws)
+            except WmmaeError as e:
+                # the direct kernel wants k contiguous in both operands, k >= 4, at most two terms
+                assert flag == DIRECT and e.status == -4, (c, flag, e)
+                assert (ta, tb) != ("T", "N") or k < 4 or policy == 2, c
+                continue
+            torch.cuda.synchronize()
+            assert torch.equal(C[:, :, m:], C0[:, :, m:]), (c, flag)
+            err = (C[:, :, :m].double() - ref).abs().max().item() / scale
+            assert err <= TOL[policy] * (3 if beta != 0 else 1), (c, flag, err)
+            res[flag] = C
+        chosen = {0: FUSED, 1: PACKED, 2: PACKED, 3: DIRECT, 4: DIRECT}[tc.sgemm_path(m, n, k, batch, policy, 0)]
+        if (ta, tb) == ("T", "N") or chosen != DIRECT:
+            # (the path query assumes the layout the direct kernel can read)
+            assert torch.equal(res[0], res[chosen]), (c, chosen)
+        if slices[PACKED] == 1:
+            assert torch.equal(res[FUSED], res[PACKED]), c
+        if DIRECT in res and slices[DIRECT] == slices[PACKED]:
+            assert torch.equal(res[DIRECT], res[PACKED]), c
