@@ -4,6 +4,7 @@ The library is built in-tree with hipcc for gfx950 and loaded with ctypes.
 There is no fallback: if the shared object is missing, `lib()` raises.
 """
 import ctypes
+import glob
 import os
 import subprocess
 
@@ -70,6 +71,12 @@ EXPORTS = [
 
 # one object per translation unit; compiled side by side, then linked
 SOURCES = ["capi_gemm.hip", "capi_harness.hip", "capi_api_gemm.hip"]
+ASM_MFMA_SOURCES = ["capi_gemm.hip"]
+
+
+def device_asm_path(name):
+    """Where build() leaves the gfx950 assembly of a translation unit with inline-asm MFMAs."""
+    return os.path.join(LIB_DIR, name.replace(".hip", "") + "-hip-amdgcn-amd-amdhsa-gfx950.s")
 
 
 def _run(cmd, verbose):
@@ -93,10 +100,22 @@ def build(verbose=False, only=None):
         obj = os.path.join(LIB_DIR, name.replace(".hip", ".o"))
         objs.append(obj)
         if only is None or name in only or not os.path.exists(obj):
-            jobs.append([hipcc, *flags, "-I" + INCLUDE_DIR, "-c",
+            # (the translation units whose kernels issue MFMAs from inline asm keep their
+            # device assembly, for the check below)
+            keep = ["-save-temps=obj"] if name in ASM_MFMA_SOURCES else []
+            jobs.append([hipcc, *flags, *keep, "-I" + INCLUDE_DIR, "-c",
                          os.path.join(CSRC_DIR, name), "-o", obj])
     with ThreadPoolExecutor(max_workers=len(SOURCES)) as pool:
         list(pool.map(lambda c: _run(c, verbose), jobs))
+    from . import isa_check
+    for name in ASM_MFMA_SOURCES:
+        stem = os.path.join(LIB_DIR, name.replace(".hip", ""))
+        for f in glob.glob(stem + "-*") + glob.glob(stem + ".hip-*"):
+            if not f.endswith("-gfx950.s"):
+                os.remove(f)
+        # pipeline hazards around the hand-placed MFMAs, which the compiler does not see:
+        # no library is linked from code that has one
+        isa_check.check_file(device_asm_path(name))
     _run([hipcc, "--offload-arch=gfx950", "-shared", "-fPIC", *objs, "-o", LIB_PATH], verbose)
     return LIB_PATH
 

@@ -360,12 +360,12 @@ __global__ void __launch_bounds__(64 * NW)
           continue;
         f32x4 o = acc_main[i][j];
         if constexpr (TERMS >= 2)
-          o += acc_err[i][j] * p.inv_scale;
+          o = epilogue_fold(o, acc_err[i][j], p.inv_scale);
         o *= alpha;
         float *const dst = Cb + row + static_cast<long long>(col) * p.ldc;
         if (vec_out && row + 3 < M) {
           if (beta != 0.f)
-            o += beta * *reinterpret_cast<const f32x4 *>(dst);
+            o = epilogue_beta(o, beta, *reinterpret_cast<const f32x4 *>(dst));
           *reinterpret_cast<f32x4 *>(dst) = o;
         } else {
 #pragma unroll
@@ -373,7 +373,7 @@ __global__ void __launch_bounds__(64 * NW)
             if (row + x < M) {
               float e = o[x];
               if (beta != 0.f)
-                e += beta * dst[x];
+                e = epilogue_beta(e, beta, dst[x]);
               dst[x] = e;
             }
           }

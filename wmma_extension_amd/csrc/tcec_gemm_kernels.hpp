@@ -34,6 +34,9 @@ typedef float f32x4 __attribute__((ext_vector_type(4)));
 constexpr int kChunkRows = 16; // rows per packed chunk (MFMA M / N)
 constexpr int kChunkK = 32;    // k per packed chunk (MFMA K) = one pipeline stage
 
+#ifndef WMMAE_MFMA_GUARD
+#define WMMAE_MFMA_GUARD ""
+#endif
 template <int I> using ic = std::integral_constant<int, I>;
 // Compile-time loop: f(std::integral_constant<int, I>) for I in [B, E).
 template <int B, int E, class F>
@@ -42,6 +45,35 @@ __device__ __forceinline__ void static_for(F &&f) {
     f(std::integral_constant<int, B>{});
     static_for<B + 1, E>(f);
   }
+}
+
+// The value the lane with the lowest lane-number bit flipped holds (DPP
+// quad_perm [1, 0, 3, 2]); every lane of the wave must be active.
+__device__ __forceinline__ float neighbour_lane(const float v) {
+  return __builtin_bit_cast(
+      float, __builtin_amdgcn_mov_dpp(__builtin_bit_cast(int, v), 0xB1, 0xF, 0xF,
+                                      true));
+}
+// The epilogue's arithmetic, spelled out so that every kernel and every store
+// path rounds alike whatever the compiler would contract: the error sum is
+// folded in with one fma, alpha is a multiplication of its own, and beta * C
+// enters with one fma.
+__device__ __forceinline__ f32x4 epilogue_fold(const f32x4 main_sum,
+                                                   const f32x4 err_sum,
+                                                   const float inv_scale) {
+  return __builtin_elementwise_fma(
+      err_sum, f32x4{inv_scale, inv_scale, inv_scale, inv_scale}, main_sum);
+}
+__device__ __forceinline__ f32x4 epilogue_beta(const f32x4 scaled,
+                                                   const float beta,
+                                                   const f32x4 c_old) {
+  return __builtin_elementwise_fma(f32x4{beta, beta, beta, beta}, c_old,
+                                   scaled);
+}
+__device__ __forceinline__ float epilogue_beta(const float scaled,
+                                               const float beta,
+                                               const float c_old) {
+  return __builtin_fmaf(beta, c_old, scaled);
 }
 // Row permutation of k group q (0..3) of a chunk written by the DIRECT
 // variant of tcec_gemm_kernel.
@@ -879,11 +911,11 @@ __global__ void __launch_bounds__(WGM *WGN * 64)
   constexpr bool USE_ASM = MT_ * NT_ >= 8;
   auto mfma_acc = [](f32x4 &z, const ab_vec x, const ab_vec y) {
     if constexpr (std::is_same<MT, _Float16>::value)
-      asm volatile("v_mfma_f32_16x16x32_f16 %0, %1, %2, %0"
+      asm volatile(WMMAE_MFMA_GUARD "v_mfma_f32_16x16x32_f16 %0, %1, %2, %0"
                    : "+a"(z)
                    : "v"(x), "v"(y));
     else
-      asm volatile("v_mfma_f32_16x16x32_bf16 %0, %1, %2, %0"
+      asm volatile(WMMAE_MFMA_GUARD "v_mfma_f32_16x16x32_bf16 %0, %1, %2, %0"
                    : "+a"(z)
                    : "v"(x), "v"(y));
   };
@@ -1132,40 +1164,130 @@ __global__ void __launch_bounds__(WGM *WGN * 64)
                          4 * static_cast<int>(lane >> 4);
     const int col_base = (to_tail ? 0 : it.tn * BN) + wn * Cfg::WN +
                          static_cast<int>(lane & 15u);
+    // the value of tile (i, j) as it goes to memory, before beta
+    const auto out_value = [&](const int i, const int j) {
+      f32x4 v = acc_main[i][j];
+      if constexpr (TERMS >= 2)
+        v = epilogue_fold(v, acc_err[i][j], inv_scale);
+      return v * a_out;
+    };
+    // (every destination is device memory: global-memory instructions, not
+    // generic ones, which would also count as LDS operations and make the
+    // compiler drain both memory counters before the next step's first
+    // dependent instruction)
+    typedef __attribute__((address_space(1))) float gfloat;
+    typedef __attribute__((address_space(1))) f32x4 gf32x4;
+    // one 16x16 tile: a lane stores rows 4q .. 4q+3 of its column, 16 bytes
+    const auto store_tile = [&](const int i, const int j) {
+      const int col = col_base + 16 * j;
+      const int row = row_base + 16 * i;
+      if (col >= N || row >= M)
+        return;
+      f32x4 v = out_value(i, j);
+      gfloat *const dst =
+          (gfloat *)(Cb + row + static_cast<long long>(col) * ld_out);
+      if (vec_out && row + 3 < M) {
+        if (b_out != 0.f)
+          v = epilogue_beta(v, b_out, *reinterpret_cast<const gf32x4 *>(dst));
+        *reinterpret_cast<gf32x4 *>(dst) = v;
+      } else {
+#pragma unroll
+        for (int x = 0; x < 4; x++) {
+          if (row + x < M) {
+            float o = v[x];
+            if (b_out != 0.f)
+              o = epilogue_beta(o, b_out, dst[x]);
+            dst[x] = o;
+          }
+        }
+      }
+    };
+    // Two tiles of one tile column (32 rows x 16 columns, all inside C): as
+    // above a store instruction would write 64 bytes of every column.  The
+    // lanes of neighbouring columns swap one tile's values instead, so that
+    // eight lanes cover 32 consecutive rows of one column: an instruction
+    // writes whole 128-byte lines, first of the even columns, then of the odd.
+    // Forced packed path, same box: 1024^2 x 128 x 256 entries 0.458 -> 0.434
+    // ms, 2048^2 x 256 x 16 0.152 -> 0.145, one term 0.336 -> 0.314, 4096^3
+    // 0.322 -> 0.318.  Not in the kernel that splits the fp32 operands itself:
+    // the values the swap keeps live cost its K loop two more registers in
+    // scratch (c5b 1.45 -> 1.60 ms), nor in the round-to-nearest variants (their
+    // fragments then come back from AGPR copies right in front of the MFMAs
+    // that read them, see wmma_extension_amd/isa_check.py).
+    constexpr bool WHOLE_LINES = !DIRECT && !RN_MAIN && MT_ % 2 == 0;
+    const int odd = static_cast<int>(lane & 1u);
+    const int blk_row0 = (to_tail ? 0 : it.tm * BM) + wm * Cfg::WM;
+    const int blk_col0 = (to_tail ? 0 : it.tn * BN) + wn * Cfg::WN;
+    const auto store_tile_pair = [&](const int i, const int j) {
+      const f32x4 v0 = out_value(i, j), v1 = out_value(i + 1, j);
+      f32x4 d1, d2;
+#pragma unroll
+      for (int x = 0; x < 4; x++) {
+        // (through a function taking the element by value: __builtin_bit_cast
+        // applied to `v0[x]` directly read element 0 for every x)
+        const float n0 = neighbour_lane(v0[x]), n1 = neighbour_lane(v1[x]);
+        d1[x] = odd ? n1 : v0[x]; // even column: own rows | neighbour's next 16
+        d2[x] = odd ? v1[x] : n0; // odd column
+      }
+      const int row = row_base + 16 * (i + odd);
+      const int col = col_base + 16 * j;
+      gfloat *const dst1 =
+          (gfloat *)(Cb + row + static_cast<long long>(col & ~1) * ld_out);
+      gfloat *const dst2 =
+          (gfloat *)(Cb + row + static_cast<long long>(col | 1) * ld_out);
+      if (b_out != 0.f) {
+        d1 = epilogue_beta(d1, b_out, *reinterpret_cast<const gf32x4 *>(dst1));
+        d2 = epilogue_beta(d2, b_out, *reinterpret_cast<const gf32x4 *>(dst2));
+      }
+      *reinterpret_cast<gf32x4 *>(dst1) = d1;
+      *reinterpret_cast<gf32x4 *>(dst2) = d2;
+    };
 #pragma unroll
     for (int j = 0; j < NT_; j++) {
-      const int col = col_base + 16 * j;
-      if (col >= N)
-        continue;
+      const bool cols_inside = blk_col0 + 16 * j + 16 <= N;
+      if constexpr (WHOLE_LINES) {
 #pragma unroll
-      for (int i = 0; i < MT_; i++) {
-        const int row = row_base + 16 * i;
-        if (row >= M)
+        for (int i = 0; i < MT_; i += 2) {
+          // (wave-uniform: both lanes of a swap take the same branch)
+          if (vec_out && cols_inside && blk_row0 + 16 * i + 32 <= M) {
+            store_tile_pair(i, j);
+          } else {
+            store_tile(i, j);
+            store_tile(i + 1, j);
+          }
+        }
+      } else {
+        // (the loop as one piece, with the compiler's own contraction of
+        // a * x + b * y, which comes out in the helpers' form: the kernel that
+        // splits its own operands has no register to spare, and through
+        // store_tile one more of its K loop's values went to scratch)
+        const int col = col_base + 16 * j;
+        if (col >= N)
           continue;
-        f32x4 v = acc_main[i][j];
-        if constexpr (TERMS >= 2)
-          v += acc_err[i][j] * inv_scale;
-        v *= a_out;
-        // (every destination is device memory: global-memory instructions, not
-        // generic ones, which would also count as LDS operations and make the
-        // compiler drain both memory counters before the next step's first
-        // dependent instruction)
-        typedef __attribute__((address_space(1))) float gfloat;
-        typedef __attribute__((address_space(1))) f32x4 gf32x4;
-        gfloat *const dst =
-            (gfloat *)(Cb + row + static_cast<long long>(col) * ld_out);
-        if (vec_out && row + 3 < M) {
-          if (b_out != 0.f)
-            v += b_out * *reinterpret_cast<const gf32x4 *>(dst);
-          *reinterpret_cast<gf32x4 *>(dst) = v;
-        } else {
 #pragma unroll
-          for (int x = 0; x < 4; x++) {
-            if (row + x < M) {
-              float o = v[x];
-              if (b_out != 0.f)
-                o += b_out * dst[x];
-              dst[x] = o;
+        for (int i = 0; i < MT_; i++) {
+          const int row = row_base + 16 * i;
+          if (row >= M)
+            continue;
+          f32x4 v = acc_main[i][j];
+          if constexpr (TERMS >= 2)
+            v += acc_err[i][j] * inv_scale;
+          v *= a_out;
+          gfloat *const dst =
+              (gfloat *)(Cb + row + static_cast<long long>(col) * ld_out);
+          if (vec_out && row + 3 < M) {
+            if (b_out != 0.f)
+              v += b_out * *reinterpret_cast<const gf32x4 *>(dst);
+            *reinterpret_cast<gf32x4 *>(dst) = v;
+          } else {
+#pragma unroll
+            for (int x = 0; x < 4; x++) {
+              if (row + x < M) {
+                float o = v[x];
+                if (b_out != 0.f)
+                  o += b_out * dst[x];
+                dst[x] = o;
+              }
             }
           }
         }
