@@ -348,36 +348,79 @@ __global__ void __launch_bounds__(64 * NW)
     const float alpha = p.alpha, beta = p.beta;
     const int row_base = tm * BM + wm * WM + 4 * static_cast<int>(lane >> 4);
     const int col_base = tn * BN + wn * WN + r16;
-#pragma unroll
-    for (int j = 0; j < NT_; j++) {
+    const auto out_value = [&](const int i, const int j) {
+      f32x4 o = acc_main[i][j];
+      if constexpr (TERMS >= 2)
+        o = epilogue_fold(o, acc_err[i][j], p.inv_scale);
+      return o * alpha;
+    };
+    // one 16x16 tile: a lane stores rows 4q .. 4q+3 of its column, 16 bytes
+    const auto store_one = [&](const int i, const int j) {
       const int col = col_base + 16 * j;
-      if (col >= N)
-        continue;
+      const int row = row_base + 16 * i;
+      if (col >= N || row >= M)
+        return;
+      f32x4 o = out_value(i, j);
+      float *const dst = Cb + row + static_cast<long long>(col) * p.ldc;
+      if (vec_out && row + 3 < M) {
+        if (beta != 0.f)
+          o = epilogue_beta(o, beta, *reinterpret_cast<const f32x4 *>(dst));
+        *reinterpret_cast<f32x4 *>(dst) = o;
+      } else {
 #pragma unroll
-      for (int i = 0; i < MT_; i++) {
-        const int row = row_base + 16 * i;
-        if (row >= M)
-          continue;
-        f32x4 o = acc_main[i][j];
-        if constexpr (TERMS >= 2)
-          o = epilogue_fold(o, acc_err[i][j], p.inv_scale);
-        o *= alpha;
-        float *const dst = Cb + row + static_cast<long long>(col) * p.ldc;
-        if (vec_out && row + 3 < M) {
-          if (beta != 0.f)
-            o = epilogue_beta(o, beta, *reinterpret_cast<const f32x4 *>(dst));
-          *reinterpret_cast<f32x4 *>(dst) = o;
-        } else {
-#pragma unroll
-          for (int x = 0; x < 4; x++) {
-            if (row + x < M) {
-              float e = o[x];
-              if (beta != 0.f)
-                e = epilogue_beta(e, beta, dst[x]);
-              dst[x] = e;
-            }
+        for (int x = 0; x < 4; x++) {
+          if (row + x < M) {
+            float e = o[x];
+            if (beta != 0.f)
+              e = epilogue_beta(e, beta, dst[x]);
+            dst[x] = e;
           }
         }
+      }
+    };
+    // two tiles of one tile column, all inside C: whole 128-byte lines per
+    // store instruction after a swap between the lanes of neighbouring columns
+    // (tcec_gemm_kernel's store_tile_pair)
+    const int odd = static_cast<int>(lane & 1u);
+    const auto store_pair = [&](const int i, const int j) {
+      const f32x4 v0 = out_value(i, j), v1 = out_value(i + 1, j);
+      f32x4 d1, d2;
+#pragma unroll
+      for (int x = 0; x < 4; x++) {
+        const float n0 = neighbour_lane(v0[x]), n1 = neighbour_lane(v1[x]);
+        d1[x] = odd ? n1 : v0[x];
+        d2[x] = odd ? v1[x] : n0;
+      }
+      const int row = row_base + 16 * (i + odd);
+      const int col = col_base + 16 * j;
+      float *const dst1 = Cb + row + static_cast<long long>(col & ~1) * p.ldc;
+      float *const dst2 = Cb + row + static_cast<long long>(col | 1) * p.ldc;
+      if (beta != 0.f) {
+        d1 = epilogue_beta(d1, beta, *reinterpret_cast<const f32x4 *>(dst1));
+        d2 = epilogue_beta(d2, beta, *reinterpret_cast<const f32x4 *>(dst2));
+      }
+      *reinterpret_cast<f32x4 *>(dst1) = d1;
+      *reinterpret_cast<f32x4 *>(dst2) = d2;
+    };
+    const int blk_row0 = tm * BM + wm * WM, blk_col0 = tn * BN + wn * WN;
+#pragma unroll
+    for (int j = 0; j < NT_; j++) {
+      const bool cols_inside = blk_col0 + 16 * j + 16 <= N;
+      if constexpr (MT_ % 2 == 0) {
+#pragma unroll
+        for (int i = 0; i < MT_; i += 2) {
+          // (wave-uniform: both lanes of a swap take the same branch)
+          if (vec_out && cols_inside && blk_row0 + 16 * i + 32 <= M) {
+            store_pair(i, j);
+          } else {
+            store_one(i, j);
+            store_one(i + 1, j);
+          }
+        }
+      } else {
+#pragma unroll
+        for (int i = 0; i < MT_; i++)
+          store_one(i, j);
       }
     }
   };
