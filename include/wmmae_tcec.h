@@ -131,10 +131,11 @@ int wmmae_tcec_sgemm_workspace_bytes(int m, int n, int k, int batch, int policy,
  * itself (no packed operands), 4 the same with K slices.  3 and 4 assume
  * k contiguous in both operands ('T','N') and need k >= 4; other layouts
  * take 1 and 2.
- * The answer assumes operands the single kernel can read 16 bytes at a time
- * (k the contiguous direction, k and the leading dimensions multiples of 4,
- * 16-byte aligned bases); other operands with k > 96 take path 1 where this
- * says 0. */
+ * The answer is for op(A) = 'T', op(B) = 'N' with tight leading dimensions
+ * (lda = ldb = k) and 16-byte aligned bases: with k a multiple of 4 the
+ * single kernel reads such operands 16 bytes at a time, which is what the
+ * time estimates behind the choice assume; other leading dimensions or bases
+ * can move a product from path 0 to another one. */
 int wmmae_tcec_sgemm_path(int m, int n, int k, int batch, int policy, int flags,
                           int *path);
 

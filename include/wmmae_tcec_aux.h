@@ -49,6 +49,16 @@ int wmmae_direct_read_first(int tail, int k, int stage, int lane,
 int wmmae_tcec_sgemm_k_slices(int m, int n, int k, int batch, int policy,
                               int flags, int *slices);
 
+/* Host only (no counterpart in the reference): the time estimates the driver
+ * chooses its path with, in seconds, for op(A) = 'T', op(B) = 'N' with tight
+ * leading dimensions and aligned bases: seconds[0] the single kernel,
+ * seconds[1] split passes + GEMM on packed operands, seconds[2] the GEMM kernel
+ * that splits the fp32 operands itself; infinity for a path the product cannot
+ * take.  The smallest is the path wmmae_tcec_sgemm* takes.  For checking the
+ * estimates against measured times. */
+int wmmae_tcec_path_estimates(int m, int n, int k, int batch, int policy,
+                              double *seconds);
+
 /* Test hook (no counterpart in the reference): the calling thread's next
  * wmmae_tcec_sgemm* / wmmae_tcec_gemm_packed calls and workspace queries cut K
  * into `slices` slices (at most 32, at least six k stages of 32 each: smaller

@@ -74,8 +74,9 @@ def test_random_products_on_every_path(tc, dev, seed):
             assert err <= TOL[policy] * (3 if beta != 0 else 1), (c, flag, err)
             res[flag] = C
         chosen = {0: FUSED, 1: PACKED, 2: PACKED, 3: DIRECT, 4: DIRECT}[tc.sgemm_path(m, n, k, batch, policy, 0)]
-        if (ta, tb) == ("T", "N") or chosen != DIRECT:
-            # (the path query assumes the layout the direct kernel can read)
+        if (ta, tb) == ("T", "N") and pad % 4 == 0:
+            # (the path query assumes op(A) = 'T', op(B) = 'N', tight leading dimensions and
+            # aligned bases: what the kernels can read 16 bytes at a time depends on those)
             assert torch.equal(res[0], res[chosen]), (c, chosen)
         if slices[PACKED] == 1:
             assert torch.equal(res[FUSED], res[PACKED]), c

@@ -43,7 +43,7 @@ def _both(dev, m, n, k, policy, alpha, beta, seed):
 def test_static_workspace_matches_caller_workspace(dev, policy):
     # first a product on packed operands with K slices, then a smaller one on packed operands,
     # then one the single kernel takes (no workspace at all)
-    shapes = [(520, 392, 8192, tcec.PATH_PACKED_SPLIT_K), (1160, 1544, 1056, tcec.PATH_PACKED),
+    shapes = [(904, 1000, 1544, tcec.PATH_PACKED_SPLIT_K), (1160, 1544, 1056, tcec.PATH_PACKED),
               (200, 136, 328, tcec.PATH_FUSED)]
     for i, (m, n, k, path) in enumerate(shapes):
         assert tcec.sgemm_path(m, n, k, 1, policy) == path, (m, n, k)
@@ -81,7 +81,7 @@ def test_static_calls_back_to_back_share_the_array_in_stream_order(dev):
     them: packed operands in the array, then K-slice planes at its start, then packed operands
     again.  Stream order is all the calls need."""
     pol = tcec.Policy.F16_EC
-    shapes = [(1160, 1544, 1056, 0), (512, 384, 16384, 0), (520, 392, 8192, 0), (200, 136, 328, 0),
+    shapes = [(1160, 1544, 1056, 0), (512, 384, 16384, 0), (904, 1000, 1544, 0), (200, 136, 328, 0),
               (1024, 520, 512, DIRECT), (1160, 1544, 1056, 0)]
     ops = [_operands(dev, m, n, k, 400 + i) for i, (m, n, k, _) in enumerate(shapes)]
     want = []

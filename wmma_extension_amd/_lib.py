@@ -66,6 +66,7 @@ EXPORTS = [
     "wmmae_direct_read_first",
     "wmmae_tcec_sgemm_k_slices",
     "wmmae_tcec_force_k_slices",
+    "wmmae_tcec_path_estimates",
 ]
 
 
@@ -170,6 +171,7 @@ _SIGNATURES = {
     "wmmae_direct_read_first": (_i, [_i, _i, _i, _i, _c.POINTER(_ll)]),
     "wmmae_tcec_sgemm_k_slices": (_i, [_i, _i, _i, _i, _i, _i, _c.POINTER(_i)]),
     "wmmae_tcec_force_k_slices": (_i, [_i]),
+    "wmmae_tcec_path_estimates": (_i, [_i, _i, _i, _i, _i, _c.POINTER(_c.c_double)]),
 }
 
 

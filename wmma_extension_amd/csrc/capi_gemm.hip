@@ -3,6 +3,7 @@
 // GEMM and the single-kernel GEMM.  Declarations and per-entry documentation
 // live in include/wmmae_tcec.h.
 #include "capi_common.hpp"
+#include <limits>
 #include "tcec_gemm_fused_kernel.hpp"
 #include "tcec_gemm_kernels.hpp"
 
@@ -215,44 +216,78 @@ constexpr double units128x128(const int terms) {
 // -- K slices for a partly empty last round: slices, pipeline refills, fold.
 //    Sweep: 126 products, 2304^2 .. 8192^2, k = 2048 .. 8192, two policies.
 constexpr double kTailOverhead = 0.2;
-// -- single-kernel (fused) or packed path.  Sweep: 573 products measured with
-//    either path forced, m = n = 384 .. 4096, k = 64 .. 8192, 1 .. 256 entries,
-//    three policies (median error of either estimate 5 %; the choice costs
-//    0.8 % against always taking the faster path; refitted once after the tile
-//    rule changed: 0.7 % over 577 products).  Rows: one, two, three terms.
+// -- which path: the single kernel, split passes + GEMM on packed operands, or
+//    the GEMM kernel that splits the fp32 operands itself.  Fit: 1860 random
+//    products (m, n = 45 .. 5000, k = 32 .. 32768, 1 .. 1024 entries, half of
+//    them with dimensions that are multiples of nothing, all five policies),
+//    each run with every path forced; the constants below minimise the
+//    squared log error of each path's estimate on 1060 of them and on 137
+//    structured products (the reference harness's grid with 256 entries,
+//    squares 1024 .. 8192, the baseline workloads; weighted four times).  On
+//    the 800 held out the path chosen with them is 1.4 % slower than always
+//    taking the fastest forced path on average (37 of 800 above 1.10 x, six
+//    above 1.25 x), on the structured ones 0.5 % (two above 1.10 x); the
+//    constants before (fits to the harness's grid and to square products)
+//    were 3 to 6 % slower on the same 800, 3.1 x at worst.  Whole default
+//    calls on 400 further random products: 1.1 % (worst 1.48 x).
+//    Rows: one, two, three terms.
 struct PathRates {
   double launch, stage, tile, bytes_per_s; // seconds, seconds, seconds, B/s
   double split_bytes_per_s;                // packed path only
+  // A k stage takes longer the fuller the chip is (power limit, contention in
+  // L2 and HBM): stage * (1 + busy * (compute units with a tile / all compute
+  // units, averaged over the rounds))
+  double busy;
 };
-constexpr PathRates kFused[3] = {{5.0e-6, 0.76e-6, 3.0e-6, 5.0e12, 0.},
-                                 {5.0e-6, 1.11e-6, 3.0e-6, 5.0e12, 0.},
-                                 {5.0e-6, 1.41e-6, 3.1e-6, 5.0e12, 0.}};
-constexpr PathRates kPacked[3] = {{8.9e-6, 0.31e-6, 2.0e-6, 5.0e12, 6.6e12},
-                                  {6.5e-6, 0.50e-6, 3.8e-6, 3.6e12, 5.6e12},
-                                  {8.8e-6, 0.99e-6, 3.4e-6, 3.4e12, 5.9e12}};
+constexpr PathRates kFused[3] = {
+    {6.01e-6, 0.643e-6, 2.88e-6, 5.32e12, 0., 0.101},
+    {6.50e-6, 0.992e-6, 1.85e-6, 5.27e12, 0., 0.170},
+    {5.37e-6, 1.39e-6, 2.22e-6, 5.14e12, 0., 0.141}};
+constexpr PathRates kPacked[3] = {
+    {8.35e-6, 0.131e-6, 3.07e-6, 3.65e12, 5.61e12, 0.359},
+    {8.17e-6, 0.287e-6, 3.69e-6, 6.50e12, 5.57e12, 0.649},
+    {7.10e-6, 0.652e-6, 4.65e-6, 6.50e12, 4.92e12, 0.361}};
 // -- the packed path's GEMM kernel reading and splitting the fp32 operands
-//    itself (256x128 tiles only; rows: one, two terms).  Sweep: 45 products
-//    run on this path and on the estimated one of the other two (the
-//    reference harness's grid m = n = 512, 1024, k = 128 .. 16384, 256
-//    entries; single and batched products of other shapes, four policies): a
-//    k stage of a 256x128 tile takes 0.8 / 1.5 us (packed operands: 0.5 /
-//    1.0 us), a tile 6 us on top.
-constexpr PathRates kDirect[2] = {{6.0e-6, 0.40e-6, 3.0e-6, 5.0e12, 0.},
-                                  {6.0e-6, 0.75e-6, 3.0e-6, 5.0e12, 0.}};
+//    itself (256x128 tiles only; rows: one, two terms)
+constexpr PathRates kDirect[2] = {
+    {3.41e-6, 0.173e-6, 3.76e-6, 4.62e12, 0., 1.18},
+    {5.00e-6, 0.355e-6, 3.65e-6, 4.92e12, 0., 0.750}};
+// ... as the host sees it when it decides whether a launch of that kernel is
+// bound by its bytes and should start its workgroups staggered (a fit of its
+// own, to the reference harness's grid: 0.8 / 1.5 us per k stage of a 256x128
+// tile and 6 us per tile, in units of half a tile)
+constexpr PathRates kDirectStagger[2] = {
+    {6.0e-6, 0.40e-6, 3.0e-6, 5.0e12, 0., 0.},
+    {6.0e-6, 0.75e-6, 3.0e-6, 5.0e12, 0., 0.}};
 // with K slices: the GEMM's time against the packed kernel's estimate for the
 // same slices of 256x128 tiles (two terms: twelve K-sliced products, m, n =
 // 64 .. 4096, k = 2048 .. 262144, each run on either path: with 1.4 the faster
 // path is chosen for all of them, with 1.5 for eleven)
 constexpr double kDirectSliceRatio[2] = {1.5, 1.4};
+// Products that are cut into K slices (few output tiles): what the slice
+// planner's time (split_time, whose constants are fitted for choosing the slice
+// count) has to be scaled and shifted by to be the time of the whole call on
+// each path; same fit as above.  Rows: scale, shift in seconds; by terms.
+constexpr double kSlicedFused[2][3] = {{1.16, 1.08, 1.03},
+                                       {-3.73e-6, -2.84e-6, -2.89e-6}};
+constexpr double kSlicedPacked[2][3] = {{0.724, 0.954, 0.955},
+                                        {-0.65e-6, -6.0e-6, -6.0e-6}};
+constexpr double kSlicedDirect[2][2] = {{0.759, 0.890}, {-6.0e-6, -6.0e-6}};
+// Calls issued back to back cannot complete faster than the host issues their
+// launches (250 products below 1.5e8 flop, called in a loop: 11, 14.5 and 12 us
+// per call in the median): what decides among the paths for tiny products -
+// one launch for the single kernel and the direct kernel, two or three for
+// the packed path.  Order: single kernel, packed, direct.
+constexpr double kCallFloor[3] = {11.0e-6, 14.3e-6, 11.5e-6};
 // k % 32 != 0: the kernel variant that reads a shorter last stage (1024^2 x 1000
 // against x 1024, batch 256: 301 against 336 TFLOPS, of which 2.4 % are the k)
-constexpr double kDirectTailStage = 1.09;
+constexpr double kDirectTailStage = 1.47;
 // the single kernel's 64x64 tile against its 128x128 tile (1024^3: 41 -> 27 us)
 constexpr double kFusedSmallTileTime = 0.65; // whole tile, latency-bound sizes
-constexpr double kFusedSmallStage = 0.33, kFusedSmallTile = 0.5;
+constexpr double kFusedSmallStage = 0.599, kFusedSmallTile = 0.467;
 // 4-byte instead of 16-byte requests: 114 random products with k % 4 != 0 ran
 // at 0.55 of the packed path's speed in the median
-constexpr double kFusedNarrowRequests = 2.5;
+constexpr double kFusedNarrowRequests = 3.50;
 } // namespace fit
 
 // XCDs (chiplets with an L2 of their own) behind the current device.  HIP does
@@ -733,43 +768,45 @@ int fused_dispatch(const int policy, const FusedArgs &f) {
   }
 }
 
-// Fused (split inside the GEMM kernel) or packed (split pass + MFMA kernel)?
-// The fused kernel moves only the fp32 operands and C but needs about twice as
-// long per 128x128x32 tile step; the packed path first writes and re-reads the
-// split operands, which pays off when every operand element is used by many
-// tiles.  Both times are estimated with the same shape, a launch cost plus
-// rounds of tiles over the compute units times (k stages * time per stage +
-// time per tile), bounded below by the bytes moved, with parameters fitted to
-// 573 measured products on MI355X (m = n = 384 .. 4096, k = 64 .. 8192, 1 to
-// 256 entries, one to three terms; median error of either estimate 5 %, the
-// choice costs 0.8 % over always taking the faster path).  K-heavy products
-// that want K slices stay on the packed path.
+// Which of the three paths?  The single ("fused") kernel moves only the fp32
+// operands and C but needs about twice as long per 128x128x32 tile step and
+// converts every element once per wave that uses it; the packed path first
+// writes and re-reads the split operands, which pays off when every operand
+// element is used by many tiles; the "direct" path is the packed path's GEMM
+// kernel (256x128 tiles) loading the fp32 operands itself and splitting them
+// on their way into LDS - no packed copy and no split pass, at 1.2 to 1.9
+// times the time per k stage; it wins where an operand element is used by
+// few tiles (batches of small and medium matrices, K-heavy products) and
+// needs k contiguous in both operands, k at least 4 and at most two terms;
+// same bits as the packed path.  All three times are estimated with the same
+// shape, a launch cost plus rounds of tiles over the compute units times (k
+// stages * time per stage + time per tile), bounded below by the bytes moved;
+// products that are cut into K slices take the slice planner's time, rescaled.
+// The constants and what they were fitted to: namespace fit.
 // fused_vec: the fused kernel can request 16 bytes per lane from both
 // operands (k contiguous, k and the strides multiples of 4, aligned bases).
-// Without that it issues four times as many requests and ran at 0.55 of the
-// packed path's speed in the median over 114 random products with k % 4 != 0
-// (faster than the packed path in one of them, by 10 %, at k = 77), so such
-// products take the packed path unless k is very short.
-// The third path, "direct": the packed path's GEMM kernel (256x128 tiles)
-// loading the fp32 operands itself and splitting them on their way into LDS.
-// No packed copy and no split pass, at 1.5 times the time per k stage; it wins
-// where an operand element is used by few tiles (batches of small and medium
-// matrices, K-heavy products).  It needs k contiguous in both operands, k a
-// least 4 and at most two terms; same bits as the packed path.
+// Without that it issues four times as many requests (3.5 times the time per
+// stage), so such products take another path unless k is very short.
 enum class Path { Fused, Packed, Direct };
+// (see PathRates::busy)
+inline double busy_factor(const fit::PathRates &r, const long long tiles) {
+  const long long cus = device_cus();
+  return 1.0 + r.busy * static_cast<double>(tiles) /
+                   static_cast<double>(ceil_div(tiles, cus) * cus);
+}
 // the direct kernel's time without K slices: rounds of 256x128 tiles over the
 // compute units, and the bytes it moves
 struct DirectTimes {
   double tiles, bytes;
 };
 inline DirectTimes direct_times(const int m, const int n, const int k,
-                                const int batch, const int terms) {
-  const fit::PathRates &d = fit::kDirect[terms - 1];
+                                const int batch, const fit::PathRates &d) {
   const double kt = static_cast<double>(ceil_div(k, 32));
   const long long tiles256 = ceil_div(m, 256) * ceil_div(n, 128) * batch;
   const double ab = (static_cast<double>(m) + n) * k * batch;
   // (the variant for k % 32 != 0 spends one more instruction per load)
-  const double stage = d.stage * (k % 32 == 0 ? 1.0 : fit::kDirectTailStage);
+  const double stage = d.stage * busy_factor(d, tiles256) *
+                       (k % 32 == 0 ? 1.0 : fit::kDirectTailStage);
   return {fit::kUnits256x128 *
               static_cast<double>(ceil_div(tiles256, device_cus())) *
               (kt * stage + d.tile),
@@ -782,6 +819,97 @@ inline bool one_path_at_most(const int flags) {
   const int f = flags & kPathFlags;
   return (f & (f - 1)) == 0;
 }
+// Estimated time of a call on each path, in seconds; a path that cannot run
+// the product (or is not considered for it) has infinity.
+struct PathEstimates {
+  double fused, packed, direct;
+};
+inline PathEstimates estimate_paths(const int m, const int n, const int k,
+                                    const int batch, const int terms,
+                                    const bool fused_vec, const bool direct_ok) {
+  constexpr double kNever = std::numeric_limits<double>::infinity();
+  PathEstimates e{kNever, kNever, kNever};
+  const fit::PathRates &f = fit::kFused[terms - 1], &p = fit::kPacked[terms - 1];
+  const long long cus = device_cus();
+  const int kti = static_cast<int>(ceil_div(k, 32));
+  const double kt = static_cast<double>(kti);
+  const double c_bytes = 4.0 * m * n * batch;
+  const double ab = (static_cast<double>(m) + n) * k * batch; // operand elements
+  const long long tiles64 = ceil_div(m, 64) * ceil_div(n, 64) * batch;
+  const long long tiles128 = ceil_div(m, 128) * ceil_div(n, 128) * batch;
+  const long long tiles256 = ceil_div(m, 256) * ceil_div(n, 128) * batch;
+
+  // fused kernel: 128x128 tiles, or 64x64 ones (a third of the stage time,
+  // half of the per-tile time) under fused_by_size's rule
+  if (fused_vec || k <= 96) {
+    const bool small = fused_small_tiles(m, n, batch);
+    const long long f_tiles = small ? tiles64 : tiles128;
+    const double f_rounds = static_cast<double>(ceil_div(f_tiles, cus));
+    e.fused =
+        f.launch +
+        std::max(f_rounds * (kt * f.stage * busy_factor(f, f_tiles) *
+                                 (fused_vec ? 1.0 : fit::kFusedNarrowRequests) *
+                                 (small ? fit::kFusedSmallStage : 1.0) +
+                             f.tile * (small ? fit::kFusedSmallTile : 1.0)),
+                 (c_bytes + 4.0 * ab) / f.bytes_per_s);
+  }
+  const double split_pass = (4.0 + 2.0 * terms) * ab / p.split_bytes_per_s;
+  const int splits = choose_splits(terms, m, n, k, batch);
+  if (splits != 1) {
+    // K slices: the split pass and the packed kernel's slices against the
+    // slower stages of the direct kernel (cut into the slices that suit its own
+    // tile)
+    e.fused = e.fused * fit::kSlicedFused[0][terms - 1] +
+              fit::kSlicedFused[1][terms - 1];
+    e.packed = (p.launch + split_pass +
+                split_time(terms, m, n, batch, kti, splits)) *
+                   fit::kSlicedPacked[0][terms - 1] +
+               fit::kSlicedPacked[1][terms - 1];
+    if (direct_ok)
+      e.direct =
+          (fit::kDirect[terms - 1].launch +
+           split_time(terms, m, n, batch, kti,
+                      choose_splits(terms, m, n, k, batch, true), true)) *
+              fit::kSlicedDirect[0][terms - 1] +
+          fit::kSlicedDirect[1][terms - 1];
+    return e;
+  }
+  // packed path: rounds in units of one 128x128 tile as gemm_by_size counts
+  // them (a 256x128 tile 2.0 and a 128x128 tile 1.2 for one and two terms,
+  // 1.8 and 1.0 for three, a 64x64 tile 0.4)
+  double units;
+  long long p_tiles;
+  const double r128 = static_cast<double>(ceil_div(tiles128, cus));
+  if (big_tile_candidate(terms, tiles128, kti) &&
+      fit::units256x128(terms) * static_cast<double>(ceil_div(tiles256, cus)) <=
+          fit::units128x128(terms) * r128) {
+    units = fit::units256x128(terms) *
+            static_cast<double>(ceil_div(tiles256, cus));
+    p_tiles = tiles256;
+  } else if (tiles128 >= cus || (m > 64 && n > 64)) {
+    units = r128 * fit::units128x128(terms);
+    p_tiles = tiles128;
+  } else {
+    units = fit::kUnits64x64 * static_cast<double>(ceil_div(tiles64, cus));
+    p_tiles = tiles64;
+  }
+  e.packed = p.launch + split_pass +
+             std::max(units * (kt * p.stage * busy_factor(p, p_tiles) + p.tile),
+                      c_bytes / p.bytes_per_s);
+  if (direct_ok) {
+    const DirectTimes d =
+        direct_times(m, n, k, batch, fit::kDirect[terms - 1]);
+    // (it cuts K for its own tile even where the packed path would not)
+    const int own = choose_splits(terms, m, n, k, batch, true);
+    e.direct =
+        own > 1 ? (fit::kDirect[terms - 1].launch +
+                   split_time(terms, m, n, batch, kti, own, true)) *
+                          fit::kSlicedDirect[0][terms - 1] +
+                      fit::kSlicedDirect[1][terms - 1]
+                : fit::kDirect[terms - 1].launch + std::max(d.tiles, d.bytes);
+  }
+  return e;
+}
 inline Path choose_path(const int m, const int n, const int k, const int batch,
                         const int flags, const int terms, const int policy,
                         const bool fused_vec, const bool direct_ok) {
@@ -792,75 +920,18 @@ inline Path choose_path(const int m, const int n, const int k, const int batch,
       policy != WMMAE_POLICY_BF16X3_EC;
   if (k <= 0 || rn_unsupported)
     return Path::Packed;
-  const int splits = choose_splits(terms, m, n, k, batch);
-  if (splits != 1) {
-    // K slices: the split pass against the slower stages of the direct kernel
-    // (cut into the slices that suit its own tile)
-    if (!direct_ok)
-      return Path::Packed;
-    const fit::PathRates &pk = fit::kPacked[terms - 1];
-    const double ab = (static_cast<double>(m) + n) * k * batch;
-    const int kt = static_cast<int>(ceil_div(k, 32));
-    const double t_packed =
-        pk.launch + (4.0 + 2.0 * terms) * ab / pk.split_bytes_per_s +
-        split_time(terms, m, n, batch, kt, splits);
-    const double t_direct =
-        fit::kDirect[terms - 1].launch +
-        split_time(terms, m, n, batch, kt,
-                   choose_splits(terms, m, n, k, batch, true), true);
-    return t_direct < t_packed ? Path::Direct : Path::Packed;
-  }
-  const bool fused_allowed = fused_vec || k <= 96;
-  const fit::PathRates &f = fit::kFused[terms - 1], &p = fit::kPacked[terms - 1];
-  const long long cus = device_cus();
-  const double kt = static_cast<double>(ceil_div(k, 32));
-  const double c_bytes = 4.0 * m * n * batch;
-  const double ab = (static_cast<double>(m) + n) * k * batch; // operand elements
-  const long long tiles64 = ceil_div(m, 64) * ceil_div(n, 64) * batch;
-  const long long tiles128 = ceil_div(m, 128) * ceil_div(n, 128) * batch;
-  const long long tiles256 = ceil_div(m, 256) * ceil_div(n, 128) * batch;
-
-  // fused kernel: 128x128 tiles, or 64x64 ones (a third of the stage time,
-  // half of the per-tile time) under fused_by_size's rule
-  const bool small = fused_small_tiles(m, n, batch);
-  const double f_rounds =
-      static_cast<double>(ceil_div(small ? tiles64 : tiles128, cus));
-  const double t_fused =
-      f.launch +
-      std::max(f_rounds * (kt * f.stage *
-                               (fused_vec ? 1.0 : fit::kFusedNarrowRequests) *
-                               (small ? fit::kFusedSmallStage : 1.0) +
-                           f.tile * (small ? fit::kFusedSmallTile : 1.0)),
-                          (c_bytes + 4.0 * ab) / f.bytes_per_s);
-
-  // packed path: rounds in units of one 128x128 tile as gemm_by_size counts
-  // them (a 256x128 tile 2.0 and a 128x128 tile 1.2 for one and two terms,
-  // 1.8 and 1.0 for three, a 64x64 tile 0.4)
-  double units;
-  const double r128 = static_cast<double>(ceil_div(tiles128, cus));
-  if (big_tile_candidate(terms, tiles128, static_cast<int>(kt)) &&
-      fit::units256x128(terms) * static_cast<double>(ceil_div(tiles256, cus)) <=
-          fit::units128x128(terms) * r128)
-    units = fit::units256x128(terms) *
-            static_cast<double>(ceil_div(tiles256, cus));
-  else if (tiles128 >= cus || (m > 64 && n > 64))
-    units = r128 * fit::units128x128(terms);
-  else
-    units = fit::kUnits64x64 * static_cast<double>(ceil_div(tiles64, cus));
-  const double t_packed =
-      p.launch + (4.0 + 2.0 * terms) * ab / p.split_bytes_per_s +
-      std::max(units * (kt * p.stage + p.tile), c_bytes / p.bytes_per_s);
-  double t_best = t_packed;
+  PathEstimates e = estimate_paths(m, n, k, batch, terms, fused_vec, direct_ok);
+  e.fused = std::max(e.fused, fit::kCallFloor[0]);
+  e.packed = std::max(e.packed, fit::kCallFloor[1]);
+  e.direct = std::max(e.direct, fit::kCallFloor[2]);
   Path best = Path::Packed;
-  if (fused_allowed && t_fused < t_best) {
-    t_best = t_fused;
+  double t_best = e.packed;
+  if (e.fused < t_best) {
+    t_best = e.fused;
     best = Path::Fused;
   }
-  if (direct_ok) {
-    const DirectTimes d = direct_times(m, n, k, batch, terms);
-    if (fit::kDirect[terms - 1].launch + std::max(d.tiles, d.bytes) < t_best)
-      best = Path::Direct;
-  }
+  if (e.direct < t_best)
+    best = Path::Direct;
   return best;
 }
 // what the direct kernel needs of a product (the operands' k strides are 1)
@@ -1159,7 +1230,8 @@ int sgemm_impl(const char transa, const char transb, const int m, const int n,
                                         a_rs, b_rs, stride_a, stride_b, 0, k};
     plan_k_slices(g, ws, ws_bytes);
     // staggered start for launches bound by their bytes (see the kernel)
-    const DirectTimes dt = direct_times(m, n, k, batch, p.terms);
+    const DirectTimes dt =
+        direct_times(m, n, k, batch, fit::kDirectStagger[p.terms - 1]);
     if (g.splits <= 1 && batch >= 8 && dt.bytes > dt.tiles)
       g.direct.stagger = 1;
     int st = gemm_dispatch(policy, 0, g);
@@ -1337,7 +1409,7 @@ int wmmae_tcec_sgemm_path(const int m, const int n, const int k,
     return WMMAE_STATUS_INVALID_VALUE;
   const bool any = m > 0 && n > 0 && k > 0 && batch > 0;
   const bool slices = any && choose_splits(p.terms, m, n, k, batch) > 1;
-  switch (choose_path(m, n, k, batch, flags, p.terms, policy, true,
+  switch (choose_path(m, n, k, batch, flags, p.terms, policy, k % 4 == 0,
                       direct_possible(k, p.terms, flags, 1, 1))) {
   case Path::Fused:
     *path = 0;
@@ -1348,6 +1420,22 @@ int wmmae_tcec_sgemm_path(const int m, const int n, const int k,
   default:
     *path = slices ? 2 : 1;
   }
+  return WMMAE_STATUS_SUCCESS;
+}
+
+int wmmae_tcec_path_estimates(const int m, const int n, const int k,
+                              const int batch, const int policy,
+                              double *const seconds) {
+  PolicyInfo p;
+  if (seconds == nullptr)
+    return WMMAE_STATUS_NULL_POINTER;
+  if (m <= 0 || n <= 0 || k <= 0 || batch <= 0 || !policy_info(policy, p))
+    return WMMAE_STATUS_INVALID_VALUE;
+  const PathEstimates e = estimate_paths(m, n, k, batch, p.terms, k % 4 == 0,
+                                         direct_possible(k, p.terms, 0, 1, 1));
+  seconds[0] = e.fused;
+  seconds[1] = e.packed;
+  seconds[2] = e.direct;
   return WMMAE_STATUS_SUCCESS;
 }
 
@@ -1374,7 +1462,7 @@ int wmmae_tcec_sgemm_k_slices(const int m, const int n, const int k,
     return WMMAE_STATUS_SUCCESS;
   const bool direct_ok = direct_possible(k, p.terms, flags, 1, 1);
   Path path = choose_path(m, n, k, batch, flags & WMMAE_FLAG_RN_MAIN, p.terms,
-                          policy, true, direct_ok);
+                          policy, k % 4 == 0, direct_ok);
   if ((flags & WMMAE_FLAG_PATH_DIRECT) != 0) {
     if (!direct_ok)
       return WMMAE_STATUS_NOT_SUPPORTED;

@@ -126,6 +126,15 @@ def sgemm_k_slices(m, n, k, batch=1, policy=Policy.F16_EC, flags=0):
     return out.value
 
 
+def path_estimates(m, n, k, batch=1, policy=Policy.F16_EC):
+    """(fused, packed, direct) time estimates in seconds the driver chooses its path with
+    (inf: the path cannot take the product)."""
+    out = (ctypes.c_double * 3)()
+    _lib.check(_lib.lib().wmmae_tcec_path_estimates(m, n, k, batch, int(policy), out),
+               "wmmae_tcec_path_estimates")
+    return tuple(out)
+
+
 class forced_k_slices:
     """Test aid: within the block, this thread's GEMM calls cut K into `slices` slices."""
 
