@@ -494,14 +494,37 @@ PATHCHECK_SHAPES = [
 PATH_NAMES = {0: "chosen", 2: "packed", 4: "fused", 8: "direct"}
 
 
-def bench_pathcheck(torch, tcec, dev, rounds=3):
+def random_path_shapes(count, seed):
+    """Seeded random products for the path check: m, n = 45 .. 5000, k = 32 .. 32768, 1 .. 1024
+    entries, 1e8 .. 4e11 flop, half of them with dimensions that are multiples of nothing, all
+    five policies (the distribution the estimates' constants were fitted on, another seed)."""
+    import random
+    rnd = random.Random(seed)
+    names = ["F16_EC", "F16_EC", "F16_EC", "F16_NOEC", "BF16X3_EC", "BF16X3_EC", "BF16X2_EC", "BF16_NOEC", "BF16_NOEC"]
+    shapes = []
+    while len(shapes) < count:
+        batch = rnd.choice([1, 1, 1, 2, 4, 8, 16, 32, 64, 128, 256, 1024])
+        m, n, k = int(2 ** rnd.uniform(5.5, 12.3)), int(2 ** rnd.uniform(5.5, 12.3)), int(2 ** rnd.uniform(5, 15))
+        r = rnd.random()
+        if r < 0.5:
+            m, n, k = (m + 15) // 16 * 16, (n + 15) // 16 * 16, (k + 31) // 32 * 32
+        elif r < 0.75:
+            k = (k + 3) // 4 * 4
+        flop = 2.0 * m * n * k * batch
+        if flop > 4e11 or flop < 1e8 or (m * k + n * k + m * n) * batch * 4 > 2e9:
+            continue
+        shapes.append((m, n, k, batch, rnd.choice(names)))
+    return shapes
+
+
+def bench_pathcheck(torch, tcec, dev, rounds=3, shapes=None):
     """Every pinned shape as one whole library call (workspace resident) on the path the time
     estimates choose and on every path forced; the variants of a shape are timed in alternation,
     the fastest round of each counts.  ratio = chosen / fastest (>= 1 by construction: the chosen
     call is one of the candidates)."""
     from wmma_extension_amd._lib import WmmaeError
     rows, worst = [], 1.0
-    for (m, n, k, batch, pol) in PATHCHECK_SHAPES:
+    for (m, n, k, batch, pol) in (PATHCHECK_SHAPES if shapes is None else shapes):
         policy = tcec.Policy[pol]
         g = torch.Generator(device=dev)
         g.manual_seed(0x5EED + 6)
@@ -551,7 +574,9 @@ def bench_pathcheck(torch, tcec, dev, rounds=3):
                      "effective_tflops": round(2.0 * m * n * k * batch / (best[0] * 1e-3) / 1e12, 1)})
         del A, Bt, Ct, ws
         torch.cuda.empty_cache()
-    return {"worst_ratio": round(worst, 3), "shapes": rows,
+    ratios = sorted(r["chosen_over_best"] for r in rows)
+    return {"worst_ratio": round(worst, 3), "mean_ratio": round(sum(ratios) / len(ratios), 4),
+            "above_1.10": sum(1 for x in ratios if x > 1.10), "count": len(ratios), "shapes": rows,
             "what": "whole wmmae_tcec_sgemm_strided_batched calls, N(0,1) operands, workspace resident; "
                     "each shape on the path the estimates choose and on every path forced, variants "
                     f"alternating, fastest of {rounds} rounds each"}
@@ -567,6 +592,10 @@ def main():
     ap.add_argument("--workload", default="c4", choices=sorted(WORKLOADS) + ["pathcheck"],
                     help="pathcheck: pinned shapes, each timed on every path the driver has "
                          "(the guard of the fitted path choices; also part of the default run)")
+    ap.add_argument("--random-shapes", type=int, default=0, metavar="N",
+                    help="with --workload pathcheck: N seeded random products instead of the pinned shapes "
+                         "(value = mean ratio; the worst and the number above 1.10 are in the line too)")
+    ap.add_argument("--seed", type=int, default=2024, help="seed of --random-shapes")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--no-accuracy", action="store_true")
     ap.add_argument("--no-secondary", action="store_true",
@@ -597,10 +626,16 @@ def main():
     dev = torch.device("cuda:0")
     torch.cuda.set_device(dev)
     if args.workload == "pathcheck":
-        r = bench_pathcheck(torch, tcec, dev)
+        shapes = random_path_shapes(args.random_shapes, args.seed) if args.random_shapes > 0 else None
+        r = bench_pathcheck(torch, tcec, dev, shapes=shapes)
+        if shapes is not None:
+            r["what"] = f"{len(shapes)} random products (seed {args.seed}); " + r["what"]
+            r["shapes"] = sorted(r["shapes"], key=lambda x: -x["chosen_over_best"])[:12]   # the worst ones
         print(json.dumps({
-            "metric": "time of the chosen path over the fastest forced path, worst of the pinned shapes",
-            "value": r["worst_ratio"], "unit": "ratio", "n_gpus": 1, "steps": 3, "warmup": 1,
+            "metric": ("time of the chosen path over the fastest forced path, "
+                       + ("mean over random products" if shapes is not None else "worst of the pinned shapes")),
+            "value": r["mean_ratio"] if shapes is not None else r["worst_ratio"],
+            "unit": "ratio", "n_gpus": 1, "steps": 3, "warmup": 1,
             "ms_per_step": None, "higher_is_better": False, "scaling": "weak", "vs_baseline": None,
             "dtype": "f16", "data": "synthetic", "config": {"workload": "pathcheck: " + r["what"]},
             "pathcheck": r, "roofline": None, "cpu_baseline": None}))
