@@ -6,7 +6,8 @@ dimensions, alpha / beta, one to forty entries, dimensions that are no multiples
   * the padding of C untouched;
   * the default call gives the bits of the forced path it reports (wmmae_tcec_sgemm_path);
   * the paths give each other's bits wherever they cut K alike (they issue the same products in the
-    same order on the same accumulators).
+    same order on the same accumulators); a case with much larger shapes, where the packed path
+    also cuts K for the tiles of its last round, is compared with that cut switched off.
 """
 import random
 
@@ -78,7 +79,39 @@ def test_random_products_on_every_path(tc, dev, seed):
             # (the path query assumes op(A) = 'T', op(B) = 'N', tight leading dimensions and
             # aligned bases: what the kernels can read 16 bytes at a time depends on those)
             assert torch.equal(res[0], res[chosen]), (c, chosen)
-        if slices[PACKED] == 1:
+        # (a single large product may also cut K for the tiles of a partly empty last round, with
+        # planes in the workspace: those tiles then sum in another order)
+        tail_planes = slices[PACKED] == 1 and tc.gemm_packed_workspace_bytes(policy, m, n, k, batch) > 0
+        if slices[PACKED] == 1 and not tail_planes:
             assert torch.equal(res[FUSED], res[PACKED]), c
-        if DIRECT in res and slices[DIRECT] == slices[PACKED]:
+        if DIRECT in res and slices[DIRECT] == slices[PACKED] and not tail_planes:
             assert torch.equal(res[DIRECT], res[PACKED]), c
+
+
+def test_tail_slices_are_the_only_difference_on_a_large_single_product(tc, dev):
+    """2293 x 1802 x 5518: the packed path, given room for them, cuts K for the tiles of its partly
+    empty last round, and those tiles come out with other last bits; with a workspace that only
+    holds the packed operands it gives the bits of the direct and of the single kernel, with
+    alpha and beta too."""
+    m, n, k, policy = 2293, 1802, 5518, 0
+    g = torch.Generator(device="cpu").manual_seed(5)
+    A = (torch.rand((m, k), generator=g) * 2 - 1).to(dev)
+    B = (torch.rand((n, k), generator=g) * 2 - 1).to(dev)
+    C0 = (torch.rand((n, m), generator=g) * 2 - 1).to(dev)
+    full = tc.workspace_bytes(m, n, k, 1, policy)
+    operands = tc.pack_bytes(m, k, 1, policy) + tc.pack_bytes(n, k, 1, policy)
+    assert full > operands and tc.sgemm_k_slices(m, n, k, 1, policy, PACKED) == 1
+    for alpha, beta in ((1.0, 0.0), (-0.5, 1.0)):
+        out = {}
+        for name, flag, size in (("packed", PACKED, operands), ("tail", PACKED, full), ("direct", DIRECT, full),
+                                 ("fused", FUSED, 0)):
+            C = C0.clone()
+            ws = torch.empty(size, dtype=torch.uint8, device=dev) if size else None
+            tc.sgemm("T", "N", m, n, k, alpha, A, k, B, k, beta, C, m, policy, flag, ws)
+            out[name] = C
+        torch.cuda.synchronize()
+        assert torch.equal(out["direct"], out["packed"]) and torch.equal(out["fused"], out["packed"])
+        differing = int((out["tail"] != out["packed"]).sum())
+        assert 0 < differing < m * n // 4
+        scale = out["packed"].abs().max().item()
+        assert (out["tail"] - out["packed"]).abs().max().item() < 1e-5 * scale
