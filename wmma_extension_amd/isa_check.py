@@ -149,5 +149,8 @@ def check_file(path):
         findings = scan(f.read())
     if findings:
         raise RuntimeError(f"{path}: {len(findings)} pipeline hazard(s) around inline-asm MFMAs that the "
-                           f"compiler does not handle:\n" + format_findings(findings))
+                           f"compiler does not handle:\n" + format_findings(findings) +
+                           "\n(change the kernel so that the allocation comes out differently, or, at a cost of up "
+                           "to 13 % in the kernel that splits its own operands, put a wait state in front of "
+                           "every such MFMA: -DWMMAE_MFMA_GUARD='\"s_nop 0\\n\\t\"')")
     return 0
