@@ -29,6 +29,18 @@ int wmmae_mfma_probe(int type, int m, int n, int k, float *d,
                      const unsigned short *a, const unsigned short *b,
                      const float *c, void *stream);
 
+/* Probe of the pipeline hazard that wmma_extension_amd/isa_check.py looks for
+ * in the generated code (no counterpart in the reference): one wave multiplies
+ * a 16x32 tile of ones by a 32x16 tile of ones (bf16, 16x16x32 MFMA placed by
+ * inline asm) right after a vector-ALU instruction has overwritten two of each
+ * lane's eight k of the A operand with twos.  d: 256 floats (the wave's
+ * accumulator registers), each 40 if the matrix core read the new register
+ * contents and 32 if it read the old ones.  producer 0: v_mov_b32, 1:
+ * v_accvgpr_read_b32; gap 0: the write directly in front of the MFMA, 1:
+ * s_nop 0 between them, 2: s_nop 1, 3: one unrelated vector instruction. */
+int wmmae_mfma_source_hazard_probe(int producer, int gap, float *d,
+                                   void *stream);
+
 /* Host only, no device access (no counterpart in the reference): where the
  * GEMM kernel that reads the fp32 operands itself begins a lane's 16-byte read
  * of k stage `stage` (32 floats a stage) of a row of k contiguous floats, in

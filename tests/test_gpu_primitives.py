@@ -269,3 +269,20 @@ def test_print_fragment_runs_and_prints_every_lane(dev):
     assert lines[1].split() == ["+0.000e+00", "+2.500e-01", "+5.000e-01", "+7.500e-01"]
     # lane 5 of the accumulator: 16 elements "(main)+(error / 2048)" = (1.5)+(5)
     assert lines[66 + 5].split() == ["(+1.500e+00)+(+5.000e+00)"] * 16
+
+
+@pytest.mark.parametrize("producer", [0, 1])
+def test_a_register_written_right_before_a_hand_placed_mfma_is_read_stale(tc, dev, producer):
+    """The hardware fact behind wmma_extension_amd/isa_check.py: a vector-ALU write (v_mov_b32, or
+    the v_accvgpr_read_b32 of a reload from an AGPR spill copy) of a source register directly in
+    front of an MFMA is not interlocked - the MFMA multiplies the old contents (32 = 32 x 1 x 1);
+    one wait state or any instruction in between, and it sees the new ones (40 = 24 + 8 x 2).
+    The compiler spaces its own MFMAs; inside an asm statement nobody does, hence the check of
+    the generated code.  (Should a later part interlock this, the first assertion fails and the
+    check can go.)"""
+    for _ in range(20):
+        stale = tc.mfma_source_hazard_probe(producer, 0, dev)
+        assert bool((stale == 32.0).all()), stale
+    for gap in (1, 2, 3):
+        fresh = tc.mfma_source_hazard_probe(producer, gap, dev)
+        assert bool((fresh == 40.0).all()), (gap, fresh)

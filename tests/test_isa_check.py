@@ -1,9 +1,10 @@
 """The check of the generated code around inline-asm MFMAs (wmma_extension_amd/isa_check.py).
 
 A vector-ALU write of a register directly in front of an MFMA that reads it is a hazard the
-hardware does not interlock (one-wave probe on gfx950: `v_mov_b32` or `v_accvgpr_read_b32` into a
-source register, then the MFMA: the MFMA multiplied the old contents in 51 200 of 51 200 results;
-with `s_nop 0` or any instruction in between, the new ones).  The compiler spaces its own MFMAs,
+hardware does not interlock (one-wave probe on gfx950, wmmae_mfma_source_hazard_probe, run by
+tests/test_gpu_primitives.py: `v_mov_b32` or `v_accvgpr_read_b32` into a source register, then
+the MFMA: the MFMA multiplies the old contents, every time; with `s_nop 0` or any instruction
+in between, the new ones).  The compiler spaces its own MFMAs,
 but it does not look into asm statements, and its register allocator may reload a fragment
 register from an AGPR copy right at the statement.  Snippets below are shaped like the compiler's
 output."""

@@ -67,6 +67,7 @@ EXPORTS = [
     "wmmae_tcec_sgemm_k_slices",
     "wmmae_tcec_force_k_slices",
     "wmmae_tcec_path_estimates",
+    "wmmae_mfma_source_hazard_probe",
 ]
 
 
@@ -172,6 +173,7 @@ _SIGNATURES = {
     "wmmae_tcec_sgemm_k_slices": (_i, [_i, _i, _i, _i, _i, _i, _c.POINTER(_i)]),
     "wmmae_tcec_force_k_slices": (_i, [_i]),
     "wmmae_tcec_path_estimates": (_i, [_i, _i, _i, _i, _i, _c.POINTER(_c.c_double)]),
+    "wmmae_mfma_source_hazard_probe": (_i, [_i, _i, _vp, _vp]),
 }
 
 

@@ -574,4 +574,29 @@ int wmmae_mfma_probe(const int type, const int m, const int n, const int k,
   return WMMAE_STATUS_NOT_SUPPORTED;
 }
 
+int wmmae_mfma_source_hazard_probe(const int producer, const int gap,
+                                   float *const d, void *const stream) {
+  if (!d)
+    return WMMAE_STATUS_NULL_POINTER;
+  if (producer < 0 || producer > 1 || gap < 0 || gap > 3)
+    return WMMAE_STATUS_INVALID_VALUE;
+  hipStream_t s = static_cast<hipStream_t>(stream);
+#define WMMAE_HAZARD(P_, G_)                                                   \
+  if (producer == P_ && gap == G_) {                                           \
+    hipLaunchKernelGGL((wmmae_harness::mfma_source_hazard_kernel<P_, G_>),     \
+                       dim3(1), dim3(64), 0, s, d);                            \
+    return launch_status();                                                    \
+  }
+  WMMAE_HAZARD(0, 0)
+  WMMAE_HAZARD(0, 1)
+  WMMAE_HAZARD(0, 2)
+  WMMAE_HAZARD(0, 3)
+  WMMAE_HAZARD(1, 0)
+  WMMAE_HAZARD(1, 1)
+  WMMAE_HAZARD(1, 2)
+  WMMAE_HAZARD(1, 3)
+#undef WMMAE_HAZARD
+  return WMMAE_STATUS_INVALID_VALUE;
+}
+
 } // extern "C"

@@ -22,6 +22,8 @@
 //   tcec_api_gemm_kernel    : a tiled GEMM written against the public tcec:: API only
 //                             (reference: test/tcec/batch_gemm.cu:196-386)
 //   mfma_probe_kernel       : one raw MFMA on caller-supplied bit patterns
+//   mfma_source_hazard_kernel: a vector-ALU write of an MFMA source register
+//                             directly in front of a hand-placed MFMA
 //   tcec_mma_complex_kernel : one-wave complex D = A*B (+C) through fragment_complex
 //                             (reference: test/tcec/mma_complex.cu:22-101)
 //   primitive_mma_kernel    : mma::load_matrix_sync -> mma_sync -> mma::store_matrix_sync
@@ -431,6 +433,54 @@ __global__ void __launch_bounds__(64)
   w::load_matrix_sync(fc, c, N, w::mem_row_major);
   w::mma_sync(fc, fa, fb, fc);
   w::store_matrix_sync(d, fc, N, w::mem_row_major);
+}
+
+// --------------------------------------------------------------------------
+// Probe of a pipeline hazard the compiler does not see when an MFMA is issued
+// from inline asm: one wave multiplies a 16x32 tile of ones by a 32x16 tile of
+// ones (bf16), after overwriting the last register of the A operand (two of a
+// lane's eight k) with twos by a vector-ALU instruction placed PRODUCER and GAP
+// wait states in front of the MFMA, all inside one asm statement.  Every
+// element of D is 40 when the matrix core saw the new register contents and 32
+// when it saw the old ones.  PRODUCER 0: v_mov_b32, 1: v_accvgpr_read_b32 (what
+// a reload from an AGPR spill copy is); GAP 0: nothing in between, 1: s_nop 0,
+// 2: s_nop 1, 3: one unrelated v_mov_b32.
+// --------------------------------------------------------------------------
+template <int PRODUCER, int GAP>
+__global__ void __launch_bounds__(64)
+    mfma_source_hazard_kernel(float *const d) {
+  typedef float f32x4 __attribute__((ext_vector_type(4)));
+  typedef unsigned u32x4 __attribute__((ext_vector_type(4)));
+  const unsigned one = 0x3F803F80u, two = 0x40004000u; // bf16 pairs
+  const u32x4 b = {one, one, one, one};
+  f32x4 acc = {0.f, 0.f, 0.f, 0.f};
+#define WMMAE_HAZARD_ASM(PRODUCER_TEXT, GAP_TEXT)                              \
+  asm volatile("v_mov_b32 v100, %2\n\tv_mov_b32 v101, %2\n\t"                  \
+               "v_mov_b32 v102, %2\n\tv_mov_b32 v103, %2\n\t"                  \
+               "v_accvgpr_write_b32 a200, %3\n\t"                              \
+               "s_nop 7\n\ts_nop 7\n\t" PRODUCER_TEXT "\n\t" GAP_TEXT          \
+               "v_mfma_f32_16x16x32_bf16 %0, v[100:103], %1, %0\n\t"           \
+               "s_nop 15\n\ts_nop 15"                                          \
+               : "+a"(acc)                                                     \
+               : "v"(b), "v"(one), "v"(two)                                    \
+               : "v100", "v101", "v102", "v103", "v104", "a200")
+#define WMMAE_HAZARD_GAP(PRODUCER_TEXT)                                        \
+  if constexpr (GAP == 0)                                                      \
+    WMMAE_HAZARD_ASM(PRODUCER_TEXT, "");                                       \
+  else if constexpr (GAP == 1)                                                 \
+    WMMAE_HAZARD_ASM(PRODUCER_TEXT, "s_nop 0\n\t");                            \
+  else if constexpr (GAP == 2)                                                 \
+    WMMAE_HAZARD_ASM(PRODUCER_TEXT, "s_nop 1\n\t");                            \
+  else                                                                         \
+    WMMAE_HAZARD_ASM(PRODUCER_TEXT, "v_mov_b32 v104, %2\n\t")
+  if constexpr (PRODUCER == 0) {
+    WMMAE_HAZARD_GAP("v_mov_b32 v103, %3");
+  } else {
+    WMMAE_HAZARD_GAP("v_accvgpr_read_b32 v103, a200");
+  }
+#undef WMMAE_HAZARD_GAP
+#undef WMMAE_HAZARD_ASM
+  reinterpret_cast<f32x4 *>(d)[threadIdx.x] = acc;
 }
 
 // --------------------------------------------------------------------------

@@ -374,6 +374,15 @@ def mfma_probe(type_, m, n, k, a_bits, b_bits, c):
     return d
 
 
+def mfma_source_hazard_probe(producer, gap, device):
+    """256 accumulator values of the hazard probe (40: the MFMA saw the register just written,
+    32: it saw the old contents); see include/wmmae_tcec_aux.h."""
+    d = torch.empty(256, dtype=torch.float32, device=device)
+    st = _lib.lib().wmmae_mfma_source_hazard_probe(producer, gap, _ptr(d), _stream())
+    _lib.check(st, "wmmae_mfma_source_hazard_probe")
+    return d
+
+
 def utils_cp_async(size, mode, src):
     """src: 256 elements of `size` bytes (any dtype, CUDA); returns the copy made through LDS."""
     _need_cuda(src)
