@@ -290,6 +290,43 @@ def test_k_slice_query_and_hook(h):
     assert h.wmmae_tcec_force_k_slices(0) == 0
 
 
+def test_path_query_is_the_smallest_estimate(h):
+    """wmmae_tcec_path_estimates exposes what the driver chooses with: the path reported by
+    wmmae_tcec_sgemm_path is the one with the smallest estimate (each estimate no smaller than
+    the time the host needs to issue that path's launches: 11, 14.3 and 11.5 us); a path the
+    product cannot take has infinity; estimates grow with the work."""
+    import math
+    import random
+    est = (ctypes.c_double * 3)()
+    out = ctypes.c_int(-1)
+    rnd = random.Random(7)
+    floors = (11.0e-6, 14.3e-6, 11.5e-6)
+    seen = set()
+    for _ in range(400):
+        m, n = int(2 ** rnd.uniform(3, 12.5)), int(2 ** rnd.uniform(3, 12.5))
+        k, batch, policy = int(2 ** rnd.uniform(2, 15)), rnd.choice([1, 1, 2, 8, 64, 256]), rnd.randrange(5)
+        assert h.wmmae_tcec_path_estimates(m, n, k, batch, policy, est) == 0
+        e = [max(x, f) for x, f in zip(est, floors)]
+        assert all(x > 0 for x in est)
+        terms = {0: 2, 1: 1, 2: 3, 3: 2, 4: 1}[policy]
+        assert math.isinf(est[2]) == (terms == 3 or k < 4)           # the direct kernel: at most two terms, k >= 4
+        assert math.isinf(est[0]) == (k % 4 != 0 and k > 96)          # the single kernel wants 16-byte requests
+        assert not math.isinf(est[1])
+        assert h.wmmae_tcec_sgemm_path(m, n, k, batch, policy, 0, ctypes.byref(out)) == 0
+        best = min(range(3), key=lambda i: (e[i], (1, 0, 2)[i]))      # ties go to packed, then fused
+        assert {0: 0, 1: 1, 2: 1, 3: 2, 4: 2}[out.value] == best, (m, n, k, batch, policy, list(est), out.value)
+        seen.add(best)
+        # four times the entries: the two GEMM-kernel paths do not get faster (the single kernel's
+        # estimate has a step where the products stop being cut into K slices)
+        more = (ctypes.c_double * 3)()
+        assert h.wmmae_tcec_path_estimates(m, n, k, 4 * batch, policy, more) == 0
+        assert all(b >= a * 0.999 or math.isinf(a) for a, b in list(zip(est, more))[1:]), (m, n, k, batch, policy)
+    assert seen == {0, 1, 2}
+    assert h.wmmae_tcec_path_estimates(0, 16, 16, 1, 0, est) == -1
+    assert h.wmmae_tcec_path_estimates(16, 16, 16, 1, 7, est) == -1
+    assert h.wmmae_tcec_path_estimates(16, 16, 16, 1, 0, None) == -2
+
+
 def test_direct_kernel_reads_stay_inside_their_rows(h):
     """The GEMM kernel that loads the fp32 operands itself reads 16 bytes per lane and stage.  For
     every k from 4 on, every stage and every lane, the four floats lie inside the row of k floats
