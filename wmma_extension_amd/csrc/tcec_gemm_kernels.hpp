@@ -1215,11 +1215,17 @@ __global__ void __launch_bounds__(WGM *WGN * 64)
     // writes whole 128-byte lines, first of the even columns, then of the odd.
     // Forced packed path, same box: 1024^2 x 128 x 256 entries 0.458 -> 0.434
     // ms, 2048^2 x 256 x 16 0.152 -> 0.145, one term 0.336 -> 0.314, 4096^3
-    // 0.322 -> 0.318.  Not in the kernel that splits the fp32 operands itself:
-    // the values the swap keeps live cost its K loop two more registers in
-    // scratch (c5b 1.45 -> 1.60 ms), nor in the round-to-nearest variants (their
-    // fragments then come back from AGPR copies right in front of the MFMAs
-    // that read them, see wmma_extension_amd/isa_check.py).
+    // 0.322 -> 0.318.  The kernel that splits the fp32 operands itself has no
+    // register to spare: with the choice made per pair of tiles, as here, the
+    // compiler keeps the accumulators' values in sight of three store paths
+    // at once, and two more of its K loop's values went to scratch (c5b 1.45
+    // -> 1.60 ms).  It decides once per item instead (below): the wave's whole
+    // piece inside C -> every pair by the swap, else the plain loop; that
+    // costs no scratch at all, and 1024 entries of 256^3 go from 0.175 to
+    // 0.166 ms, 1024^2 x 128 x 256 entries from 0.389 to 0.355.  Not in the
+    // round-to-nearest variants (their fragments then come back from AGPR
+    // copies right in front of the MFMAs that read them, see
+    // wmma_extension_amd/isa_check.py).
     constexpr bool WHOLE_LINES = !DIRECT && !RN_MAIN && MT_ % 2 == 0;
     const int odd = static_cast<int>(lane & 1u);
     const int blk_row0 = (to_tail ? 0 : it.tm * BM) + wm * Cfg::WM;
@@ -1248,6 +1254,18 @@ __global__ void __launch_bounds__(WGM *WGN * 64)
       *reinterpret_cast<gf32x4 *>(dst1) = d1;
       *reinterpret_cast<gf32x4 *>(dst2) = d2;
     };
+    if constexpr (DIRECT && !RN_MAIN && MT_ % 2 == 0) {
+      // the wave's whole piece inside C: every pair by the swap, no other
+      // path in sight of the accumulators (one decision per item)
+      if (vec_out && blk_row0 + Cfg::WM <= M && blk_col0 + Cfg::WN <= N) {
+#pragma unroll
+        for (int j = 0; j < NT_; j++)
+#pragma unroll
+          for (int i = 0; i < MT_; i += 2)
+            store_tile_pair(i, j);
+        return;
+      }
+    }
 #pragma unroll
     for (int j = 0; j < NT_; j++) {
       const bool cols_inside = blk_col0 + 16 * j + 16 <= N;
