@@ -494,6 +494,42 @@ PATHCHECK_SHAPES = [
 PATH_NAMES = {0: "chosen", 2: "packed", 4: "fused", 8: "direct"}
 
 
+def vendor_mfma_yardstick(torch, dev, names=("c3", "c4")):
+    """What ONE plain half-precision product of the vendor library (torch.matmul -> hipBLASLt) reaches
+    on the leading terms of the same operands, same box, same minute: how much of the nominal
+    matrix peak a tuned kernel sustains on this data under the power limit.  A yardstick beside the
+    roofline fractions of this library's kernels (which issue 3 or 6 such products per result and
+    accumulate the error terms apart); never part of `value`."""
+    out = {}
+    for name in names:
+        w = dict(WORKLOADS[name])
+        m, n, k = w["m"], w["n"], w["k"]
+        dt = torch.bfloat16 if "BF16" in w["policy"] else torch.float16
+        A, Bt = make_inputs(torch, w, dev, 0x5EED + 3)
+        a, b = A[0].to(dt), Bt[0].to(dt).t()                 # row-major A, column-major B, as the workload
+        del A, Bt
+        flops = 2.0 * m * n * k
+        steps = max(10, min(400, int(1.5e15 / flops)))       # about one second
+        c = torch.matmul(a, b)
+        for _ in range(max(3, steps // 10)):
+            torch.matmul(a, b, out=c)
+        torch.cuda.synchronize()
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        e0.record()
+        for _ in range(steps):
+            torch.matmul(a, b, out=c)
+        e1.record()
+        torch.cuda.synchronize()
+        ms = e0.elapsed_time(e1) / steps
+        tf = flops / (ms * 1e-3) / 1e12
+        out[name] = {"what": f"torch.matmul, {str(dt).split('.')[-1]} in and out, {m}x{n}x{k}, "
+                             f"{w['dist']} operands rounded to the type", "steps": steps,
+                     "ms": round(ms, 4), "tflops": round(tf, 1), "frac_of_mfma_peak": round(tf / PEAK_MFMA_TFLOPS, 4)}
+        del a, b, c
+        torch.cuda.empty_cache()
+    return out
+
+
 def random_path_shapes(count, seed):
     """Seeded random products for the path check: m, n = 45 .. 5000, k = 32 .. 32768, 1 .. 1024
     entries, 1e8 .. 4e11 flop, half of them with dimensions that are multiples of nothing, all
@@ -601,7 +637,8 @@ def main():
     ap.add_argument("--no-secondary", action="store_true",
                     help="with the default workload: skip the 4096^3 half of the metric (c3), the "
                          "API-level GEMM figure, the batched / K-heavy configurations (c5a, c5b), the "
-                         "primitive tile stream (c2) and the path check")
+                         "primitive tile stream (c2), the path check and the vendor library's "
+                         "half-precision yardstick")
     ap.add_argument("--flags", type=int, default=0)
     ap.add_argument("--dist", default=None, choices=["uniform", "normal", "exp", "zeros"],
                     help="override the workload's input distribution (zeros: what the kernel reaches "
@@ -714,6 +751,10 @@ def main():
                             "shapes": [{"shape": f"{r['m']}x{r['n']}x{r['k']} x{r['entries']} {r['policy']}",
                                         "chosen_path": r["chosen_path"], "chosen_over_best": r["chosen_over_best"],
                                         "ms": r["ms"]} for r in pc["shapes"]]}
+        # the vendor library's single half-precision product on the same data (a yardstick for the
+        # roofline fractions above: what the power limit leaves a tuned kernel of this part)
+        torch.cuda.empty_cache()
+        out["vendor_mfma_yardstick"] = vendor_mfma_yardstick(torch, dev)
     if not args.no_cpu:
         from oracle import oracle as orc
         out["cpu_baseline"] = cpu_baseline(orc, w)
