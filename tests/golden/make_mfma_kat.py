@@ -11,7 +11,9 @@ patterns, c, d: float32):
     small or tiny negative C, cancellation, carries across a power of two - the cases
     that tell the alignment grids, truncation directions and guard bits apart;
   * seeded random tiles with exponents spread far wider than a product's 24-bit window,
-    sparse tiles, tiles whose products cancel in pairs.
+    sparse tiles, tiles whose products cancel in pairs;
+  * bf16 tiles whose sums are fp32 subnormals (what is kept below the last bit of such a
+    result before it is rounded).
 Run on a GPU box:  python tests/golden/make_mfma_kat.py [output.npz]
 """
 import os
@@ -111,6 +113,47 @@ def random_tile(rng, name, M, N, K, mode):
     return a, b, c
 
 
+def subnormal_result_tiles(rng):
+    """bf16 16x16x32 tiles whose sums end below fp32's smallest normal number: operands with
+    biased exponent fields 0 .. 6 (subnormal and the smallest normal bf16 values) times operands
+    of 2^-30 .. 2^-8, so that the products reach far below 2^-149; C zero, subnormal or tiny.
+    (fp16 products cannot get there: the smallest is 2^-48.)  Tile 0 is hand made, one experiment
+    per diagonal element: the single products 21 * 2^-133 times 61 * 2^-25 = (2.5 + 2^-9) * 2^-149
+    and -9 * 2^-133 times 199 * 2^-25 = -(3.5 - 2^-9) * 2^-149, alone and on top of a subnormal C."""
+    def field(shape, elo, ehi, sparse=1.0):
+        e = rng.integers(elo, ehi + 1, shape).astype(np.uint16)
+        m = rng.integers(0, 1 << 7, shape).astype(np.uint16)
+        s = rng.integers(0, 2, shape).astype(np.uint16)
+        v = (s << 15) | (e << 7) | m
+        v[rng.random(shape) >= sparse] = 0
+        return v
+
+    def c_of(kind):
+        sign = rng.integers(0, 2, (16, 16)).astype(np.uint32) << 31
+        if kind == 0:
+            return np.zeros((16, 16), np.float32)
+        if kind == 1:
+            return (rng.integers(0, 1 << 23, (16, 16)).astype(np.uint32) | sign).view(np.float32)
+        return (rng.integers(1 << 23, 8 << 23, (16, 16)).astype(np.uint32) | sign).view(np.float32)
+    a0 = np.zeros((16, 32), np.uint16)
+    b0 = np.zeros((32, 16), np.uint16)
+    c0 = np.zeros((16, 16), np.float32)
+    u = np.float32(2.0 ** -149)
+    # diagonal element i: one product (subnormal a = bits * 2^-133) * b, plus C
+    for i, (a_bits, b_val, c_units) in enumerate(((21, 61 * 2.0 ** -25, 0), (0x8000 | 9, 199 * 2.0 ** -25, 0),
+                                                  (21, 61 * 2.0 ** -25, 4), (0x8000 | 9, 199 * 2.0 ** -25, -2))):
+        a0[i, 0] = a_bits
+        b0[0, i] = bf16bits(np.float32(b_val))[()]
+        c0[i, i] = c_units * u
+    tiles = [(a0, b0, c0)]
+    for (alo, ahi) in ((0, 0), (0, 3), (1, 6)):
+        for (blo, bhi) in ((127 - 22, 127 - 8), (127 - 30, 127 - 18)):
+            for ckind in (0, 1, 2):
+                for sparse in (1.0, 0.1):
+                    tiles.append((field((16, 32), alo, ahi, sparse), field((32, 16), blo, bhi), c_of(ckind)))
+    return tiles
+
+
 def main():
     out_path = sys.argv[1] if len(sys.argv) > 1 else os.path.join(ROOT, "tests", "golden", "mfma_kat.npz")
     out = {}
@@ -133,6 +176,11 @@ def main():
             key = f"{name}_{M}x{N}x{K}"
             out[key + "_a"], out[key + "_b"] = np.stack(A), np.stack(B)
             out[key + "_c"], out[key + "_d"] = np.stack(C), np.stack(D)
+    sub = subnormal_result_tiles(np.random.default_rng(0x53554221))
+    out["bf16_subnormal_results_16x16x32_a"] = np.stack([t[0] for t in sub])
+    out["bf16_subnormal_results_16x16x32_b"] = np.stack([t[1] for t in sub])
+    out["bf16_subnormal_results_16x16x32_c"] = np.stack([t[2] for t in sub])
+    out["bf16_subnormal_results_16x16x32_d"] = np.stack([run(1, 16, 16, 32, *t) for t in sub])
     np.savez_compressed(out_path, **out)
     print("wrote", out_path, sum(v.nbytes for v in out.values()), "bytes raw")
 

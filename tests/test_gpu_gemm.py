@@ -75,6 +75,58 @@ def test_sgemm_aligned_shapes(tc, orc, dev, policy, mnk):
     assert np.array_equal(D.view(np.uint32), emu.view(np.uint32)), np.abs(D - emu).max()
 
 
+def _random_patterns(rng, shape, emin, emax, zeros=0.02):
+    """fp32 values with uniformly drawn sign, exponent (emin .. emax) and mantissa bits."""
+    e = rng.integers(emin, emax + 1, shape)
+    bits = ((rng.integers(0, 2, shape).astype(np.uint32) << 31) | ((e + 127).astype(np.uint32) << 23)
+            | rng.integers(0, 1 << 23, shape).astype(np.uint32))
+    v = bits.view(np.float32).copy()
+    v[rng.random(shape) < zeros] = 0.0
+    return v
+
+
+@pytest.mark.parametrize("policy", [0, 1, 2, 3, 4])
+@pytest.mark.parametrize("regime", ["wide", "tiny_a", "subnormal_a"])
+def test_sgemm_wide_exponent_range_same_bits_as_the_model(tc, orc, dev, policy, regime):
+    """Operands far from [-1, 1]: exponents over the whole range a policy's 16-bit type holds
+    (and past it: fp16 terms of values above 65504 are infinities), operands whose terms are
+    subnormal in that type, and fp32 subnormals - where residual terms underflow and sums end
+    below 2^-126.  The packed, the single-kernel and the direct path give the bits of the oracle's
+    model of the matrix core there too, infinities and NaNs in the same places."""
+    from wmma_extension_amd._lib import WmmaeError
+    kind, ec = POL_KIND[policy]
+    f16 = kind == 0
+    for (m, n, k) in ((200, 136, 328), (64, 64, 32)):
+        rng = np.random.default_rng(1000 + 10 * policy + m + len(regime))
+        if regime == "wide":
+            lo, hi = (-40, 15) if f16 else (-60, 60)
+            A, B = _random_patterns(rng, (m, k), lo, hi), _random_patterns(rng, (k, n), lo, hi)
+        elif regime == "tiny_a":
+            lo, hi = (-30, -10) if f16 else (-126, -100)
+            A, B = _random_patterns(rng, (m, k), lo, hi), _random_patterns(rng, (k, n), -3, 3)
+        else:
+            A = (rng.integers(0, 1 << 24, (m, k)).astype(np.uint32)
+                 | (rng.integers(0, 2, (m, k)).astype(np.uint32) << 31)).view(np.float32)
+            B = _random_patterns(rng, (k, n), -3, 3)
+        emu = orc.tcec_matmul(A, B, kind=kind, ec=ec, fk=32, main_outside=False, hw_model=True)
+        ran = 0
+        for flag in (2, 4, 8):
+            try:
+                D = _gemm(tc, dev, A, B, policy, flags=flag)
+            except WmmaeError as e:
+                assert flag == 8 and e.status == -4 and policy == 2, (flag, e)   # direct: one or two terms
+                continue
+            ran += 1
+            fin = np.isfinite(emu)
+            assert np.array_equal(np.isnan(D), np.isnan(emu)) and np.array_equal(np.isinf(D), np.isinf(emu))
+            assert np.array_equal(np.signbit(D[~np.isnan(emu)]), np.signbit(emu[~np.isnan(emu)]))
+            assert np.array_equal(D[fin].view(np.uint32), emu[fin].view(np.uint32)), \
+                (policy, regime, (m, n, k), flag, int((D[fin].view(np.uint32) != emu[fin].view(np.uint32)).sum()))
+        assert ran >= 2
+        if regime == "subnormal_a" and not f16:
+            assert (np.abs(emu) < 2.0 ** -110).all() and (emu != 0).mean() > 0.9   # sums around 2^-126 and below
+
+
 @pytest.mark.parametrize("policy", [0, 2])
 @pytest.mark.parametrize("mnk", [(1, 1, 1), (17, 5, 3), (100, 37, 77), (129, 255, 33), (300, 200, 100),
                                  (16, 16, 1000), (1000, 3, 8), (700, 37, 77), (130, 1031, 45)])
