@@ -296,7 +296,10 @@ static inline float orc_mma_block_exact(const float *a, const float *b, int fk,
  *     from its leading one down (a subnormal result: to a multiple of 2^-157,
  *     eight bits below fp32's smallest step), and then rounded to nearest even
  *   - a zero result is +0.
- * Non-finite inputs are not modelled (plain double arithmetic).
+ * Non-finite inputs are not modelled (plain double arithmetic), nor are sums
+ * of finite products that leave fp32's range: the hardware then returns NaNs in
+ * places where this model returns an infinity (seen with bf16 operands of
+ * 2^56 .. 2^63 through the GEMM driver; the finite results still agree).
  * a, b: n values that are exactly representable in the 16-bit type. */
 static inline int64_t shr_floor(int64_t v, int sh) {
   if (sh <= 0)

@@ -401,6 +401,38 @@ def test_api_level_gemm_matches_driver(tc, orc, dev, type_ec):
     assert e.value.status == -4
 
 
+@pytest.mark.parametrize("type_ec", [(0, 1), (0, 0), (2, 1)])
+def test_api_level_gemm_wide_exponent_range(tc, orc, dev, type_ec):
+    """The kernel on the public API with operands over the whole exponent range of the policy's
+    16-bit type, operands whose terms are subnormal there and fp32 subnormals: the split at the
+    fragment load, the fp32 adds outside the matrix core and the store give the model's bits."""
+    type_, ec = type_ec
+    policy = {(0, 1): 0, (0, 0): 1, (2, 1): 2}[type_ec]
+    f16 = type_ == 0
+    m, n, k = 256, 384, 160
+    for regime in ("wide", "tiny_a", "subnormal_a"):
+        rng = np.random.default_rng(5 + policy + len(regime))
+        if regime == "wide":
+            lo, hi = (-40, 14) if f16 else (-60, 60)
+            A, Bt = _random_patterns(rng, (m, k), lo, hi), _random_patterns(rng, (n, k), lo, hi)
+        elif regime == "tiny_a":
+            lo, hi = (-30, -10) if f16 else (-126, -100)
+            A, Bt = _random_patterns(rng, (m, k), lo, hi), _random_patterns(rng, (n, k), -3, 3)
+        else:
+            A = (rng.integers(0, 1 << 24, (m, k)).astype(np.uint32)
+                 | (rng.integers(0, 2, (m, k)).astype(np.uint32) << 31)).view(np.float32)
+            Bt = _random_patterns(rng, (n, k), -3, 3)
+        dC = torch.zeros((n, m), dtype=torch.float32, device=dev)
+        tc.api_gemm(type_, ec, m, n, k, 1.0, torch.from_numpy(A).to(dev), k, torch.from_numpy(Bt).to(dev), k,
+                    0.0, dC, m)
+        torch.cuda.synchronize()
+        got = dC.cpu().numpy().T
+        emu = orc.tcec_matmul(A, Bt.T, kind=POL_KIND[policy][0], ec=bool(ec), fk=32, main_outside=bool(ec),
+                              hw_model=True)
+        assert np.isfinite(emu).all()
+        assert np.array_equal(got.view(np.uint32), emu.view(np.uint32)), (regime, np.abs(got - emu).max())
+
+
 def test_api_level_gemm_pointer_arrays(tc, orc, dev):
     """The API-level kernel on device arrays of matrix pointers (launch_bgemm's calling
     convention, batch_gemm.cu:433-443): every entry equals the single-matrix call bit for bit,

@@ -74,6 +74,55 @@ def test_mma_tile_all_layouts(tc, orc, dev, type_, ec, inst, shape, rounding):
             assert err < (TH_NOEC if type_ == 0 else 8 * TH_NOEC)   # bf16 has 3 fewer bits
 
 
+def _random_patterns(rng, shape, emin, emax, zeros=0.02):
+    """fp32 values with uniformly drawn sign, exponent (emin .. emax) and mantissa bits."""
+    e = rng.integers(emin, emax + 1, shape)
+    bits = ((rng.integers(0, 2, shape).astype(np.uint32) << 31) | ((e + 127).astype(np.uint32) << 23)
+            | rng.integers(0, 1 << 23, shape).astype(np.uint32))
+    v = bits.view(np.float32).copy()
+    v[rng.random(shape) < zeros] = 0.0
+    return v
+
+
+def _subnormal_patterns(rng, shape, bits):
+    return (rng.integers(0, 1 << bits, shape).astype(np.uint32)
+            | (rng.integers(0, 2, shape).astype(np.uint32) << 31)).view(np.float32)
+
+
+@pytest.mark.parametrize("type_", [0, 1, 2])
+@pytest.mark.parametrize("ec", [1, 0])
+def test_mma_tile_wide_exponent_range(tc, orc, dev, type_, ec):
+    """Operands far from [-1, 1] through the device API: the whole exponent range of the 16-bit
+    type, operands whose terms are subnormal there, and fp32 subnormals (residual terms
+    underflow, sums and the fp32 adds outside the matrix core end below 2^-126), with and
+    without C, all three roundings and instruction shapes: the oracle's model, bit for bit."""
+    kind = KIND_OF_TYPE[type_]
+    f16 = kind == 0
+    for inst, rounding, regime in itertools.product((0, 1, 2), (0, 1, 2), ("wide", "tiny_a", "subnormal_a")):
+        m, n, k = _dims(0, inst)
+        main_outside = bool(ec) if rounding == 0 else rounding == 1
+        rng = np.random.default_rng(type_ * 1000 + ec * 100 + inst * 10 + rounding + len(regime))
+        if regime == "wide":
+            lo, hi = (-40, 14) if f16 else (-60, 60)
+            A, B = _random_patterns(rng, (m, k), lo, hi), _random_patterns(rng, (k, n), lo, hi)
+            C = _random_patterns(rng, (m, n), 2 * lo, 28 if f16 else 2 * hi)
+        elif regime == "tiny_a":
+            lo, hi = (-30, -10) if f16 else (-126, -100)
+            A, B = _random_patterns(rng, (m, k), lo, hi), _random_patterns(rng, (k, n), -3, 3)
+            C = _random_patterns(rng, (m, n), lo, hi)
+        else:
+            A, B = _subnormal_patterns(rng, (m, k), 24), _random_patterns(rng, (k, n), -3, 3)
+            C = _subnormal_patterns(rng, (m, n), 25)
+        for Cc in (None, C):
+            D = _run(tc, dev, 0, type_, ec, inst, A, B, Cc, 0, 1, 1, 1, rounding)
+            emu = orc.tcec_matmul(A, B, Cc, kind=kind, ec=bool(ec), fk=INST_K[inst],
+                                  main_outside=main_outside, hw_model=True)
+            fin = np.isfinite(emu)
+            assert np.array_equal(np.isfinite(D), fin), (inst, rounding, regime)
+            assert np.array_equal(D[fin].view(np.uint32), emu[fin].view(np.uint32)), \
+                (inst, rounding, regime, Cc is not None)
+
+
 @pytest.mark.parametrize("type_", [0, 1, 2])
 @pytest.mark.parametrize("ec", [1, 0])
 def test_mma_tile_exact_cases(tc, orc, dev, type_, ec):
