@@ -13,7 +13,9 @@ patterns, c, d: float32):
   * seeded random tiles with exponents spread far wider than a product's 24-bit window,
     sparse tiles, tiles whose products cancel in pairs;
   * bf16 tiles whose sums are fp32 subnormals (what is kept below the last bit of such a
-    result before it is rounded).
+    result before it is rounded);
+  * bf16 tiles whose products and sums leave fp32's range (where infinities and NaNs appear);
+  * tiles with infinities and NaNs among the operands.
 Run on a GPU box:  python tests/golden/make_mfma_kat.py [output.npz]
 """
 import os
@@ -154,6 +156,84 @@ def subnormal_result_tiles(rng):
     return tiles
 
 
+def overflow_tiles(rng):
+    """bf16 16x16x32 tiles whose products and sums leave fp32's range (operands of 2^58 .. 2^64),
+    C zero, large or infinite.  Tile 0 is hand made, one experiment per diagonal element
+    (OVERFLOW_EXPERIMENTS: k -> (a, b), and C)."""
+    def field(shape, elo, ehi, sparse=1.0):
+        e = rng.integers(elo, ehi + 1, shape).astype(np.uint16)
+        m = rng.integers(0, 1 << 7, shape).astype(np.uint16)
+        s = rng.integers(0, 2, shape).astype(np.uint16)
+        v = (s << 15) | (e << 7) | m
+        v[rng.random(shape) >= sparse] = 0
+        return v
+    a0 = np.zeros((16, 32), np.float32)
+    b0 = np.zeros((32, 16), np.float32)
+    c0 = np.zeros((16, 16), np.float32)
+    for i, (prods, cv) in enumerate(OVERFLOW_EXPERIMENTS):
+        for k, (x, y) in prods.items():
+            a0[i, k] = x
+            b0[k, i] = y
+        c0[i, i] = cv
+    tiles = [(bf16bits(a0), bf16bits(b0), c0)]
+    for (lo, hi) in ((58, 63), (61, 63), (62, 64)):
+        for sparse in (1.0, 0.2):
+            for ckind in range(3):
+                a = field((16, 32), 127 + lo, 127 + hi, sparse)
+                b = field((32, 16), 127 + lo, 127 + min(hi, 63))
+                if ckind == 0:
+                    c = np.zeros((16, 16), np.float32)
+                elif ckind == 1:
+                    c = (rng.choice([-1.0, 1.0], (16, 16)) * (1 + rng.random((16, 16)))
+                         * 2.0 ** rng.integers(120, 128, (16, 16))).astype(np.float32)
+                else:
+                    c = np.where(rng.random((16, 16)) < 0.5, np.inf, -np.inf).astype(np.float32)
+                tiles.append((a, b, c))
+    return tiles
+
+
+def nonfinite_operand_tiles(rng, mant_bits, bias, emax):
+    """16x16x32 tiles of moderate values with infinities, NaNs and zeros strewn over A and B
+    (1, 5 and 30 % of the elements non-finite), C zero, finite, or infinite with a row of NaNs."""
+    tiles = []
+    for frac in (0.01, 0.05, 0.3):
+        for ckind in range(3):
+            def field(shape):
+                e = rng.integers(bias - 4, bias + 4, shape).astype(np.uint16)
+                m = rng.integers(0, 1 << mant_bits, shape).astype(np.uint16)
+                s = rng.integers(0, 2, shape).astype(np.uint16)
+                v = (s << 15) | (e << mant_bits) | m
+                r = rng.random(shape)
+                v[r < frac] = (s[r < frac] << 15) | (emax << mant_bits)                               # +-inf
+                v[(r >= frac) & (r < 1.5 * frac)] = (emax << mant_bits) | (1 << (mant_bits - 1)) | 1  # NaN
+                v[(r >= 1.5 * frac) & (r < 1.5 * frac + 0.1)] = 0
+                return v
+            a, b = field((16, 32)), field((32, 16))
+            if ckind == 0:
+                c = np.zeros((16, 16), np.float32)
+            elif ckind == 1:
+                c = rng.standard_normal((16, 16)).astype(np.float32)
+            else:
+                c = np.where(rng.random((16, 16)) < 0.5, np.inf, -np.inf).astype(np.float32)
+                c[0, :] = np.nan
+            tiles.append((a, b, c))
+    return tiles
+
+
+_H = 1.5 * 2.0 ** 63
+_B = 2.0 ** 64
+OVERFLOW_EXPERIMENTS = (
+    ({0: (_B, _B)}, 0.0),                                           # one product of 2^128
+    ({0: (_B, _B), 1: (-_B, _B)}, 0.0),                             # two of them, opposite signs
+    ({0: (_H, _B), 1: (_H, _B)}, 0.0),                              # finite products, sum 3 * 2^127
+    ({0: (_H, _B), 1: (_H, _B), 8: (-_H, _B), 9: (-_H, _B)}, 0.0),  # ... taken back in the next group
+    ({0: (_H, _B), 1: (_H, _B), 2: (-_H, _B), 3: (-_H, _B)}, 0.0),  # ... taken back in the same group
+    ({0: (-_B, _B)}, np.inf),                                       # infinite C against an infinite product
+    ({0: (-_H, _B)}, np.inf),                                       # infinite C against a finite one
+    ({0: (2.0 ** 63, _B)}, 1.5 * 2.0 ** 127),                       # C + product = 2.5 * 2^127
+)
+
+
 def main():
     out_path = sys.argv[1] if len(sys.argv) > 1 else os.path.join(ROOT, "tests", "golden", "mfma_kat.npz")
     out = {}
@@ -181,6 +261,18 @@ def main():
     out["bf16_subnormal_results_16x16x32_b"] = np.stack([t[1] for t in sub])
     out["bf16_subnormal_results_16x16x32_c"] = np.stack([t[2] for t in sub])
     out["bf16_subnormal_results_16x16x32_d"] = np.stack([run(1, 16, 16, 32, *t) for t in sub])
+    ovf = overflow_tiles(np.random.default_rng(0x4F564621))
+    out["bf16_overflow_16x16x32_a"] = np.stack([t[0] for t in ovf])
+    out["bf16_overflow_16x16x32_b"] = np.stack([t[1] for t in ovf])
+    out["bf16_overflow_16x16x32_c"] = np.stack([t[2] for t in ovf])
+    out["bf16_overflow_16x16x32_d"] = np.stack([run(1, 16, 16, 32, *t) for t in ovf])
+    for type_, name, mant_bits, bias, emax in ((0, "f16", 10, 15, 31), (1, "bf16", 7, 127, 255)):
+        nf = nonfinite_operand_tiles(np.random.default_rng(0x4E414E21 + type_), mant_bits, bias, emax)
+        key = f"{name}_nonfinite_operands_16x16x32"
+        out[key + "_a"] = np.stack([t[0] for t in nf])
+        out[key + "_b"] = np.stack([t[1] for t in nf])
+        out[key + "_c"] = np.stack([t[2] for t in nf])
+        out[key + "_d"] = np.stack([run(type_, 16, 16, 32, *t) for t in nf])
     np.savez_compressed(out_path, **out)
     print("wrote", out_path, sum(v.nbytes for v in out.values()), "bytes raw")
 

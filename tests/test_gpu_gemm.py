@@ -86,19 +86,26 @@ def _random_patterns(rng, shape, emin, emax, zeros=0.02):
 
 
 @pytest.mark.parametrize("policy", [0, 1, 2, 3, 4])
-@pytest.mark.parametrize("regime", ["wide", "tiny_a", "subnormal_a"])
+@pytest.mark.parametrize("regime", ["wide", "tiny_a", "subnormal_a", "huge"])
 def test_sgemm_wide_exponent_range_same_bits_as_the_model(tc, orc, dev, policy, regime):
     """Operands far from [-1, 1]: exponents over the whole range a policy's 16-bit type holds
     (and past it: fp16 terms of values above 65504 are infinities), operands whose terms are
     subnormal in that type, and fp32 subnormals - where residual terms underflow and sums end
-    below 2^-126.  The packed, the single-kernel and the direct path give the bits of the oracle's
-    model of the matrix core there too, infinities and NaNs in the same places."""
+    below 2^-126 - and bf16 operands of 2^56 .. 2^63, whose sums leave fp32's range.  The packed,
+    the single-kernel and the direct path give the bits of the oracle's model of the matrix core
+    there too, infinities and NaNs in the same places."""
     from wmma_extension_amd._lib import WmmaeError
     kind, ec = POL_KIND[policy]
     f16 = kind == 0
+    if regime == "huge" and f16:
+        pytest.skip("fp16 terms of such operands are infinities: tests/test_gpu_gemm_nonfinite.py")
     for (m, n, k) in ((200, 136, 328), (64, 64, 32)):
         rng = np.random.default_rng(1000 + 10 * policy + m + len(regime))
-        if regime == "wide":
+        if regime == "huge":
+            # products up to 2^127 and sums beyond fp32's range: infinities and NaNs where the
+            # model has them
+            A, B = _random_patterns(rng, (m, k), 56, 63), _random_patterns(rng, (k, n), 56, 63)
+        elif regime == "wide":
             lo, hi = (-40, 15) if f16 else (-60, 60)
             A, B = _random_patterns(rng, (m, k), lo, hi), _random_patterns(rng, (k, n), lo, hi)
         elif regime == "tiny_a":
