@@ -51,3 +51,34 @@ def test_split_of_every_fp32_pattern(tc, orc, dev, policy, kind_name, terms):
                 raise AssertionError(
                     f"policy {policy} term {t}: fp32 pattern {base + i:#010x} -> device {int(got[t][i]):#06x}, "
                     f"oracle {int(want[t][i]):#06x} ({int(differ.sum())} patterns of this pass differ)")
+
+
+def test_cast_of_every_fp32_pattern(tc, orc, dev):
+    """utils `cast` to half, bfloat16 and tf32 (the reference's detail/common.hpp:22-61 and its
+    cvt.rna, :73-91) for every fp32 bit pattern.  half / bfloat16: against torch's own conversions
+    (round to nearest even; NaNs by class).  tf32: against the oracle's rule in integer arithmetic
+    (add half a step of the 13 dropped bits to the magnitude, clear them: ties away from zero;
+    infinities and NaNs pass through) - on the device for all patterns, and the oracle's own
+    function on a strided sample of each pass."""
+    log_chunk = 27
+    count = 1 << log_chunk
+    for chunk in range((1 << 32) >> log_chunk):
+        base = chunk << log_chunk
+        bits = torch.arange(base, base + count, dtype=torch.int64, device=dev)
+        x = bits.to(torch.int32).view(torch.float32)
+        for dst, tdt, exp_mask, man_mask in ((0, torch.float16, 0x7C00, 0x03FF), (1, torch.bfloat16, 0x7F80, 0x007F)):
+            got = tc.utils_cast(dst, x).to(torch.int32) & 0xFFFF
+            want = x.to(tdt).view(torch.int16).to(torch.int32) & 0xFFFF
+            nan = ((got & exp_mask) == exp_mask) & ((got & man_mask) != 0)
+            nan_w = ((want & exp_mask) == exp_mask) & ((want & man_mask) != 0)
+            assert torch.equal(nan, nan_w), (chunk, dst)
+            assert torch.equal(got[~nan], want[~nan]), (chunk, dst)
+        t = tc.utils_cast(2, x).view(torch.int32).to(torch.int64) & 0xFFFFFFFF
+        nonfinite = (bits & 0x7F800000) == 0x7F800000
+        rule = torch.where(nonfinite, bits, (bits + 0x1000) & 0xFFFFE000)
+        assert torch.equal(t, rule), chunk
+        sample = x[::65537].cpu().numpy()
+        fin = np.isfinite(sample)
+        want = np.array([orc.to_tf32(e) for e in sample[fin]], dtype=np.float32)
+        got = tc.utils_cast(2, x[::65537].contiguous()).cpu().numpy()[fin]
+        assert np.array_equal(got.view(np.uint32), want.view(np.uint32)), chunk
