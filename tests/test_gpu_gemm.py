@@ -440,6 +440,37 @@ def test_api_level_gemm_wide_exponent_range(tc, orc, dev, type_ec):
         assert np.array_equal(got.view(np.uint32), emu.view(np.uint32)), (regime, np.abs(got - emu).max())
 
 
+@pytest.mark.parametrize("flag", [2, 8])
+def test_fold_of_k_slices_is_the_same_with_any_layout_of_c(tc, dev, flag):
+    """The kernel that adds the K slices takes 16 bytes per access where C allows it and single
+    elements elsewhere (a padded leading dimension, a base that is no multiple of 16 bytes, a
+    pointer array): same sums in the same order, same bits, with alpha and beta."""
+    m, n, k, policy = 512, 384, 20000, 0
+    assert tc.sgemm_k_slices(m, n, k, 1, policy, flag) > 1
+    g = torch.Generator(device=dev).manual_seed(31)
+    A = torch.rand((m, k), generator=g, device=dev) * 2 - 1
+    B = torch.rand((n, k), generator=g, device=dev) * 2 - 1
+    C0 = torch.rand((n, m), generator=g, device=dev) * 2 - 1
+    ws = torch.empty(tc.workspace_bytes(m, n, k, 1, policy), dtype=torch.uint8, device=dev)
+    for alpha, beta in ((1.0, 0.0), (-0.75, 1.5)):
+        outs = []
+        for pad, shift in ((0, 0), (1, 0), (4, 0), (0, 1), (4, 3)):
+            buf = torch.full((n * (m + pad) + 8,), 7.0, device=dev)
+            C = buf[shift:shift + n * (m + pad)].view(n, m + pad)
+            C[:, :m] = C0
+            tc.sgemm("T", "N", m, n, k, alpha, A, k, B, k, beta, C, m + pad, policy, flag, ws)
+            torch.cuda.synchronize()
+            assert (C[:, m:] == 7.0).all() and (buf[:shift] == 7.0).all()
+            outs.append(C[:, :m].clone())
+        # ... and through an array of pointers
+        C = C0.clone()
+        ptr = lambda t: torch.tensor([t.data_ptr()], dtype=torch.int64, device=dev)   # noqa: E731
+        tc.sgemm_batched("T", "N", m, n, k, alpha, ptr(A), k, ptr(B), k, beta, ptr(C), m, 1, policy, flag, ws)
+        torch.cuda.synchronize()
+        outs.append(C)
+        assert all(torch.equal(outs[0], o) for o in outs[1:]), (alpha, beta)
+
+
 def test_api_level_gemm_pointer_arrays(tc, orc, dev):
     """The API-level kernel on device arrays of matrix pointers (launch_bgemm's calling
     convention, batch_gemm.cu:433-443): every entry equals the single-matrix call bit for bit,

@@ -588,15 +588,30 @@ int launch_gemm(const GemmArgs &g) {
     st = launch_status();
   }
   if (st == WMMAE_STATUS_SUCCESS && zdim > 1) {
-    const long long blocks = ceil_div(static_cast<long long>(g.m) * g.n, 256);
-    for (int e0 = 0; e0 < g.batch; e0 += kMaxGridY)
-      hipLaunchKernelGGL(wmmae_gemm::reduce_splits_kernel,
-                         dim3(static_cast<unsigned>(blocks),
-                              std::min(g.batch - e0, kMaxGridY)),
-                         dim3(256), 0, g.stream, g.partial, zdim, g.c, g.m, g.n,
-                         g.ldc, g.stride_c, g.c_ptrs, g.alpha, g.beta,
-                         static_cast<long long>(g.batch),
-                         static_cast<unsigned>(e0));
+    // 16 bytes per access where every slice column and every column of C starts
+    // on a 16-byte boundary (entries of a pointer array: not known here)
+    const bool vec = g.m % 4 == 0 && g.ldc % 4 == 0 && g.c_ptrs == nullptr &&
+                     reinterpret_cast<uintptr_t>(g.c) % 16 == 0 &&
+                     g.stride_c % 4 == 0 &&
+                     reinterpret_cast<uintptr_t>(g.partial) % 16 == 0;
+    const long long blocks =
+        ceil_div(static_cast<long long>(g.m) * g.n, vec ? 1024 : 256);
+    for (int e0 = 0; e0 < g.batch; e0 += kMaxGridY) {
+      const dim3 grid(static_cast<unsigned>(blocks),
+                      std::min(g.batch - e0, kMaxGridY));
+      if (vec)
+        hipLaunchKernelGGL(wmmae_gemm::reduce_splits_kernel<4>, grid, dim3(256),
+                           0, g.stream, g.partial, zdim, g.c, g.m, g.n, g.ldc,
+                           g.stride_c, g.c_ptrs, g.alpha, g.beta,
+                           static_cast<long long>(g.batch),
+                           static_cast<unsigned>(e0));
+      else
+        hipLaunchKernelGGL(wmmae_gemm::reduce_splits_kernel<1>, grid, dim3(256),
+                           0, g.stream, g.partial, zdim, g.c, g.m, g.n, g.ldc,
+                           g.stride_c, g.c_ptrs, g.alpha, g.beta,
+                           static_cast<long long>(g.batch),
+                           static_cast<unsigned>(e0));
+    }
     st = launch_status();
   }
   return st;

@@ -285,8 +285,11 @@ __global__ void __launch_bounds__(256)
 // reduce_splits_kernel: C = alpha * sum_z partial[z] + beta * C for split-K.
 // partial[z][batch] are dense column-major M x N slices; the sum runs over z
 // in ascending order in double precision, so the result does not depend on
-// the launch geometry.
+// the launch geometry.  A thread owns VEC consecutive elements of a slice
+// (VEC == 4: M, ldc and the entries' bases are multiples of four floats, so
+// the four are rows of one column and every access is one 16-byte piece).
 // --------------------------------------------------------------------------
+template <int VEC>
 __global__ void __launch_bounds__(256)
     reduce_splits_kernel(const float *__restrict__ partial, const int splits,
                          float *__restrict__ C, const int M, const int N,
@@ -294,19 +297,46 @@ __global__ void __launch_bounds__(256)
                          float *const *__restrict__ c_ptrs, const float alpha,
                          const float beta, const long long batches,
                          const unsigned entry0) {
-  const long long e = static_cast<long long>(blockIdx.x) * 256 + threadIdx.x;
+  static_assert(VEC == 1 || VEC == 4, "one element or one 16-byte piece");
+  const long long e =
+      (static_cast<long long>(blockIdx.x) * 256 + threadIdx.x) * VEC;
   const long long mn = static_cast<long long>(M) * N;
   if (e >= mn)
     return;
   const long long entry = entry0 + blockIdx.y;
-  double s = 0.;
-  for (int z = 0; z < splits; z++)
-    s += static_cast<double>(partial[(z * batches + entry) * mn + e]);
+  double s[VEC];
+#pragma unroll
+  for (int x = 0; x < VEC; x++)
+    s[x] = 0.;
+  for (int z = 0; z < splits; z++) {
+    const float *const src = partial + (z * batches + entry) * mn + e;
+    if constexpr (VEC == 4) {
+      const f32x4 v = *reinterpret_cast<const f32x4 *>(src);
+#pragma unroll
+      for (int x = 0; x < 4; x++)
+        s[x] += static_cast<double>(v[x]);
+    } else {
+      s[0] += static_cast<double>(*src);
+    }
+  }
   float *const cb =
       c_ptrs != nullptr ? c_ptrs[entry] : C + entry * batch_stride_c;
   float *const p = cb + (e % M) + (e / M) * ldc;
-  const float v = alpha * static_cast<float>(s);
-  *p = beta == 0.f ? v : v + beta * *p;
+  if constexpr (VEC == 4) {
+    f32x4 out;
+    f32x4 old = {0.f, 0.f, 0.f, 0.f};
+    if (beta != 0.f)
+      old = *reinterpret_cast<const f32x4 *>(p);
+#pragma unroll
+    for (int x = 0; x < 4; x++) {
+      const float v = alpha * static_cast<float>(s[x]);
+      out[x] = beta == 0.f ? v : v + beta * old[x];
+    }
+    *reinterpret_cast<f32x4 *>(p) = out;
+  } else {
+    const float v = alpha * static_cast<float>(s[0]);
+    *p = beta == 0.f ? v : v + beta * *p;
+  }
 }
 
 // --------------------------------------------------------------------------
