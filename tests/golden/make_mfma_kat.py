@@ -15,7 +15,8 @@ patterns, c, d: float32):
   * bf16 tiles whose sums are fp32 subnormals (what is kept below the last bit of such a
     result before it is rounded);
   * bf16 tiles whose products and sums leave fp32's range (where infinities and NaNs appear);
-  * tiles with infinities and NaNs among the operands.
+  * tiles with infinities and NaNs among the operands;
+  * fp32 operands through the fp32 policy of the device API (fp32_policy_*: a, b fp32 values).
 Run on a GPU box:  python tests/golden/make_mfma_kat.py [output.npz]
 """
 import os
@@ -273,6 +274,26 @@ def main():
         out[key + "_b"] = np.stack([t[1] for t in nf])
         out[key + "_c"] = np.stack([t[2] for t in nf])
         out[key + "_d"] = np.stack([run(type_, 16, 16, 32, *t) for t in nf])
+    # the fp32 policy through the device API (tcec::mma_sync on float fragments, 32x32x32 and
+    # 16x48x64 problems, with C): operands and results as fp32
+    rng = np.random.default_rng(0x46503332)
+    A, B, C, D = [], [], [], []
+    for wide in (0, 1):
+        m, n, k = 32, 32, 32
+        a = rng.uniform(-1, 1, (m, k)) * (np.exp2(rng.integers(-20, 20, (m, k))) if wide else 1.0)
+        b = rng.uniform(-1, 1, (k, n)) * (np.exp2(rng.integers(-20, 20, (k, n))) if wide else 1.0)
+        c = rng.uniform(-1, 1, (m, n)) * (np.exp2(rng.integers(-20, 20, (m, n))) if wide else 1.0)
+        a, b, c = a.astype(np.float32), b.astype(np.float32), c.astype(np.float32)
+        d = torch.full((m * n,), float("nan"), dtype=torch.float32, device=dev)
+        tc.mma_tile(0, 3, 0, 1, torch.from_numpy(a.reshape(-1)).to(dev), torch.from_numpy(b.reshape(-1)).to(dev),
+                    torch.from_numpy(c.reshape(-1)).to(dev), 0, 0, 0, 0, 0, d)
+        torch.cuda.synchronize()
+        A.append(a)
+        B.append(b)
+        C.append(c)
+        D.append(d.cpu().numpy().reshape(m, n))
+    out["fp32_policy_32x32x32_a"], out["fp32_policy_32x32x32_b"] = np.stack(A), np.stack(B)
+    out["fp32_policy_32x32x32_c"], out["fp32_policy_32x32x32_d"] = np.stack(C), np.stack(D)
     np.savez_compressed(out_path, **out)
     print("wrote", out_path, sum(v.nbytes for v in out.values()), "bytes raw")
 

@@ -520,6 +520,9 @@ def test_api_level_gemm_fp32_policy(tc, orc, dev):
     e_cpu = orc.max_rel_err(orc.gemm_f32(A, Bt.T), ref)
     # two fp32 summations in different orders: same error scale, neither exact
     assert e_gpu <= 4 * e_cpu and e_gpu > 0
+    # the order of the matrix core's fused multiply-adds is known: the oracle's model, bit for bit
+    emu = orc.fp32_policy_matmul(A, Bt.T)
+    assert np.array_equal(got.view(np.uint32), emu.view(np.uint32)), np.abs(got - emu).max()
     # and TCEC with error correction on the same inputs is no worse than 2x either of them
     e_tcec = orc.max_rel_err(_gemm(tc, dev, A, Bt.T, 0), ref)
     assert e_tcec <= 2 * min(e_gpu, e_cpu)
