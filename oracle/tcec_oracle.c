@@ -651,17 +651,23 @@ void orc_gemm_f32(int m, int n, int k, const float *A, long long lda_r,
  * k must be a multiple of 16; C may be NULL (zeros). */
 void orc_fp32_policy_matmul(int m, int n, int k, const float *A, long long lda_r,
                             long long lda_c, const float *B, long long ldb_r,
-                            long long ldb_c, const float *C, float *D) {
+                            long long ldb_c, const float *C, float *D,
+                            int main_outside) {
 #pragma omp parallel for collapse(2)
   for (int i = 0; i < m; i++) {
     for (int j = 0; j < n; j++) {
       float acc = C ? C[(size_t)i * n + j] : 0.f;
-      for (int f0 = 0; f0 + 16 <= k; f0 += 16)
+      for (int f0 = 0; f0 + 16 <= k; f0 += 16) {
+        /* main_outside (mma_rn_sync, no_cor.hpp:750-855): every 16 of k starts
+           from zero on the matrix core and is added with an fp32 add */
+        float blk = main_outside ? 0.f : acc;
         for (int x = 0; x < 4; x++)
           for (int g = 0; g < 4; g++) {
             const int l = f0 + 4 * g + x;
-            acc = fmaf(A[i * lda_r + l * lda_c], B[l * ldb_r + j * ldb_c], acc);
+            blk = fmaf(A[i * lda_r + l * lda_c], B[l * ldb_r + j * ldb_c], blk);
           }
+        acc = main_outside ? acc + blk : blk;
+      }
       D[(size_t)i * n + j] = acc;
     }
   }

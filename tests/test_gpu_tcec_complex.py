@@ -76,6 +76,38 @@ def test_complex_mma_matches_composed_real_products(tc, orc, dev, type_):
     assert np.abs(D.real - re).max() <= scale and np.abs(D.imag - im).max() <= scale
 
 
+@pytest.mark.parametrize("type_ec", [(0, 1), (0, 0), (1, 1), (1, 0), (2, 1), (2, 0), (3, 0)])
+def test_complex_mma_bits_of_the_chained_real_products(tc, orc, dev, type_ec):
+    """The four real products of a complex one run in pairs on one accumulator fragment each
+    (complex.hpp:609-646: re = Ar Br + Cr, then - Ai Bi on top; im = Ai Br + Ci, then Ar Bi), the
+    error part carried from the first product of a pair into the second and folded once at the
+    store.  That is one real TCEC product over the joined operands [Ar | Ai] [Br ; -Bi] and
+    [Ai | Ar] [Br ; Bi]: the oracle's model of the matrix core gives the same bits, for every
+    rounding variant, with and without C, and for the fp32 policy."""
+    type_, ec = type_ec
+
+    def f(x):
+        return np.ascontiguousarray(x, dtype=np.float32)
+    for rounding, with_c in itertools.product((0, 1, 2), (0, 1)):
+        rng = np.random.default_rng(type_ * 100 + ec * 10 + rounding + with_c)
+        A, B = _rand(rng), _rand(rng)
+        C = _rand(rng) if with_c else None
+        D = _run(tc, dev, type_, ec, A, B, C, 0, 1, 1, 1, rounding)
+        main_outside = bool(ec) if rounding == 0 else rounding == 1
+
+        def mm(a1, a2, b1, b2, c):
+            a, b = f(np.concatenate([a1, a2], axis=1)), f(np.concatenate([b1, b2], axis=0))
+            c = None if c is None else f(c)
+            if type_ == 3:
+                return orc.fp32_policy_matmul(a, b, c, main_outside=rounding == 1)
+            return orc.tcec_matmul(a, b, c, kind=KIND_OF_TYPE[type_], ec=bool(ec), fk=32,
+                                   main_outside=main_outside, hw_model=True)
+        re = mm(A.real, A.imag, B.real, -B.imag, C.real if with_c else None)
+        im = mm(A.imag, A.real, B.real, B.imag, C.imag if with_c else None)
+        assert np.array_equal(f(D.real).view(np.uint32), re.view(np.uint32)), (rounding, with_c)
+        assert np.array_equal(f(D.imag).view(np.uint32), im.view(np.uint32)), (rounding, with_c)
+
+
 @pytest.mark.parametrize("type_", [0, 2, 3])
 def test_complex_exact_cases_roundings_and_scaled_io(tc, orc, dev, type_):
     rng = np.random.default_rng(11)

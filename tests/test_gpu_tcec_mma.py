@@ -302,6 +302,13 @@ def test_fp32_policy_mma_tile(tc, orc, dev):
             # the oracle's model of it, bit for bit
             emu = orc.fp32_policy_matmul(A, B, C)
             assert np.array_equal(D.view(np.uint32), emu.view(np.uint32)), (shape, a_col, b_col, c_col, d_col, with_c)
+            if a_col == b_col:
+                # mma_rz_sync chains through the matrix core like the default; mma_rn_sync starts
+                # every 16 of k from zero there and adds outside
+                for rounding in (1, 2):
+                    D2 = _run(tc, dev, shape, 3, 0, 1, A, B, C, a_col, b_col, c_col, d_col, rounding)
+                    emu2 = orc.fp32_policy_matmul(A, B, C, main_outside=rounding == 1)
+                    assert np.array_equal(D2.view(np.uint32), emu2.view(np.uint32)), (shape, rounding, with_c)
     # error correction does not exist for fp32 operands
     from wmma_extension_amd._lib import WmmaeError
     with pytest.raises(WmmaeError) as e:
