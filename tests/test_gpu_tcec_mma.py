@@ -196,6 +196,18 @@ def test_matvec(tc, orc, dev, type_, ec):
             assert err < 1e-3
         else:
             assert err < (TH_NOEC if type_ == 0 else 8 * TH_NOEC)
+        # the vector is the first column (row) of an otherwise empty operand fragment: the same
+        # matrix product in the oracle's model of the matrix core, bit for bit
+        X = np.zeros((32, 32), np.float32)
+        if left:
+            X[0, :] = x
+            emu = orc.tcec_matmul(X, A, kind=KIND_OF_TYPE[type_], ec=bool(ec), fk=32, main_outside=bool(ec),
+                                  hw_model=True)[0, :]
+        else:
+            X[:, 0] = x
+            emu = orc.tcec_matmul(A, X, kind=KIND_OF_TYPE[type_], ec=bool(ec), fk=32, main_outside=bool(ec),
+                                  hw_model=True)[:, 0]
+        assert np.array_equal(y.view(np.uint32), emu.view(np.uint32)), (a_col, left)
 
 
 @pytest.mark.parametrize("type_", [0, 1, 2])
@@ -341,6 +353,14 @@ def test_fp32_policy_matvec(tc, orc, dev):
         ref = (x.astype(np.float64) @ A.astype(np.float64)) if left else \
             (A.astype(np.float64) @ x.astype(np.float64))
         assert np.abs(y - ref).max() < TH_EC
+        X = np.zeros((32, 32), np.float32)
+        if left:
+            X[0, :] = x
+            emu = orc.fp32_policy_matmul(X, A)[0, :]
+        else:
+            X[:, 0] = x
+            emu = orc.fp32_policy_matmul(A, X)[:, 0]
+        assert np.array_equal(y.view(np.uint32), emu.view(np.uint32)), (a_col, left)
 
 
 def test_fp32_policy_elementwise(tc, orc, dev):
