@@ -80,6 +80,8 @@ def lib():
         h.orc_gemm_f64.argtypes = [_i, _i, _i, _fp, _ll, _ll, _fp, _ll, _ll, _dp, _ll, _ll]
         h.orc_gemm_f32.restype = None
         h.orc_gemm_f32.argtypes = [_i, _i, _i, _fp, _ll, _ll, _fp, _ll, _ll, _fp, _ll, _ll]
+        h.orc_epilogue.restype = None
+        h.orc_epilogue.argtypes = [_ll, _fp, _c.c_float, _c.c_float, _fp, _fp, _i]
         h.orc_fp32_policy_matmul.restype = None
         h.orc_fp32_policy_matmul.argtypes = [_i, _i, _i, _fp, _ll, _ll, _fp, _ll, _ll, _c.c_void_p, _fp, _i]
         h.orc_gemm_f32_tn.restype = None
@@ -229,6 +231,18 @@ def gemm_f32(A, B):
     D = np.zeros((m, n), dtype=np.float32)
     lib().orc_gemm_f32(m, n, k, a, ar, ac, b, br, bc, D.reshape(-1), n, 1)
     return D
+
+
+def epilogue(t, alpha, beta, C=None, api_form=False):
+    """alpha * t + beta * C as the driver's kernels round it: t * alpha, then one fused
+    multiply-add of beta * C (beta == 0: C is not read).  api_form: as the GEMM written on the
+    public API rounds it (beta * C first, then one fused multiply-add of alpha * t)."""
+    t = np.ascontiguousarray(t, dtype=np.float32)
+    c = np.ascontiguousarray(C if C is not None else np.zeros_like(t), dtype=np.float32)
+    assert c.shape == t.shape
+    out = np.empty_like(t)
+    lib().orc_epilogue(t.size, t.reshape(-1), float(alpha), float(beta), c.reshape(-1), out.reshape(-1), int(api_form))
+    return out
 
 
 def fp32_policy_matmul(A, B, C=None, main_outside=False):

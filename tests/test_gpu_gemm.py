@@ -398,6 +398,8 @@ def test_api_level_gemm_matches_driver(tc, orc, dev, type_ec):
         else:
             expect = alpha * emu.astype(np.float64) + beta * C0
             assert (np.abs(got - expect) <= 2 * 2.0**-24 * (np.abs(alpha * emu) + np.abs(beta * C0))).all()
+            # ... and exactly: beta * C rounded, then one fused multiply-add of alpha * (hi + lo / 2048)
+            assert np.array_equal(got.view(np.uint32), orc.epilogue(emu, alpha, beta, C0, api_form=True).view(np.uint32))
         # the driver chains the leading product through the matrix core instead: two roundings
         # of the same sums
         drv = _gemm(tc, dev, A, Bt.T, policy, alpha=alpha, beta=beta, C=C0)
@@ -584,12 +586,14 @@ def test_sgemm_randomised_sweep(tc, orc, dev):
         D = _gemm(tc, dev, A, B, policy, alpha=alpha, beta=beta, C=C, ta=ta, tb=tb, ld_pad=ld_pad)
         kind, ec = POL_KIND[policy]
         emu = orc.tcec_matmul(A, B, kind=kind, ec=ec, fk=32, main_outside=False, hw_model=True)
-        expect = alpha * emu.astype(np.float64) + beta * C
         if tc.sgemm_path(m, n, k, 1, policy) == tc.PATH_PACKED_SPLIT_K:
             # K slices round their partial sums
+            expect = alpha * emu.astype(np.float64) + beta * C
             tol = 32 * 2.0**-24 * max(1.0, np.abs(expect).max())
+            assert (np.abs(D - expect) <= tol).all(), (case, m, n, k, policy, ta, tb, alpha, beta, ld_pad)
         else:
-            # same sums as the emulator; alpha and beta are applied in fp32
-            tol = 2 * 2.0**-24 * (np.abs(alpha * emu) + np.abs(beta * C)) + 2.0**-140
-        assert (np.abs(D - expect) <= tol).all(), (case, m, n, k, policy, ta, tb, alpha, beta, ld_pad)
+            # same sums as the emulator, and the same epilogue: one multiplication by alpha, one
+            # fused multiply-add of beta * C - the same bits
+            assert np.array_equal(D.view(np.uint32), orc.epilogue(emu, alpha, beta, C).view(np.uint32)), \
+                (case, m, n, k, policy, ta, tb, alpha, beta, ld_pad)
         _check(orc, D, A, B, policy, C=C, alpha=alpha, beta=beta)

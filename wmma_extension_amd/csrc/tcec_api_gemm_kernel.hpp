@@ -185,8 +185,8 @@ __global__ void __launch_bounds__(ApiGemmShape::THREADS, WAVES_PER_SIMD)
     tcec::load_matrix_sync(fin, cw, ldc, w::mem_col_major);
     fc.integrate();
 #pragma unroll
-    for (unsigned i = 0; i < fc.num_elements; i++)
-      fc.x(i) = alpha * fc.x(i) + beta * fin.x(i);
+    for (unsigned i = 0; i < fc.num_elements; i++) // (the roundings written out)
+      fc.x(i) = __builtin_fmaf(alpha, fc.x(i), beta * fin.x(i));
     tcec::store_matrix_sync(cw, fc, ldc, w::mem_col_major);
   }
 }
