@@ -442,6 +442,39 @@ def test_api_level_gemm_wide_exponent_range(tc, orc, dev, type_ec):
         assert np.array_equal(got.view(np.uint32), emu.view(np.uint32)), (regime, np.abs(got - emu).max())
 
 
+@pytest.mark.parametrize("case", [(0, (128, 128, 20000), 0, (1.0, 0.0)), (0, (128, 96, 20000), 2, (-0.75, 1.5)),
+                                  (0, (256, 128, 9999), 8, (1.0, 0.0)), (2, (200, 136, 8000), 2, (2.5, -1.0)),
+                                  (3, (192, 128, 20000), 8, (1.0, 0.0)), (1, (96, 80, 30000), 0, (1.0, 1.0)),
+                                  (0, (256, 256, 8192), 0, (1.0, 0.0))])
+def test_k_slices_same_bits_as_the_model(tc, orc, dev, case):
+    """A product cut into K slices: every slice is the product over its share of k (whole stages
+    of 32, ceil(stages / slices) each) in the oracle's model of the matrix core, folded to
+    main + err / scale in fp32; the slices are added in ascending order in double precision,
+    rounded to fp32, and alpha and beta applied as by the other paths.  Same bits, on the packed
+    path, the direct path and the library's choice."""
+    policy, (m, n, k), flag, (alpha, beta) = case
+    kind, ec = POL_KIND[policy]
+    rng = np.random.default_rng(m + k)
+    A = rng.uniform(-1, 1, (m, k)).astype(np.float32)
+    B = rng.uniform(-1, 1, (k, n)).astype(np.float32)
+    C = rng.uniform(-1, 1, (m, n)).astype(np.float32)
+    slices = tc.sgemm_k_slices(m, n, k, 1, policy, flag)
+    assert slices > 1
+    ws = torch.empty(tc.workspace_bytes(m, n, k, 1, policy), dtype=torch.uint8, device=dev)
+    D = _gemm(tc, dev, A, B, policy, alpha=alpha, beta=beta, C=C, flags=flag, workspace=ws)
+    stages = (k + 31) // 32
+    per = -(-stages // slices)
+    total = np.zeros((m, n), np.float64)
+    for s0 in range(0, stages, per):
+        ka, kb = 32 * s0, min(k, 32 * (s0 + per))
+        Ap = np.zeros((m, 32 * (-(-(kb - ka) // 32))), np.float32)          # the last stage padded with zeros
+        Bp = np.zeros((Ap.shape[1], n), np.float32)
+        Ap[:, :kb - ka], Bp[:kb - ka, :] = A[:, ka:kb], B[ka:kb, :]
+        total += orc.tcec_matmul(Ap, Bp, kind=kind, ec=ec, fk=32, main_outside=False, hw_model=True).astype(np.float64)
+    emu = orc.epilogue(total.astype(np.float32), alpha, beta, C)
+    assert np.array_equal(D.view(np.uint32), emu.view(np.uint32)), int((D.view(np.uint32) != emu.view(np.uint32)).sum())
+
+
 @pytest.mark.parametrize("flag", [2, 8])
 def test_fold_of_k_slices_is_the_same_with_any_layout_of_c(tc, dev, flag):
     """The kernel that adds the K slices takes 16 bytes per access where C allows it and single
