@@ -34,6 +34,28 @@ def _check_rows(orc, A, Bt, Ct, rows, seed=7):
     return orc.max_rel_err(c, ref), orc.max_rel_err(c32, ref), orc.frobenius_residual(c, ref)
 
 
+def _same_bits_as_the_model(orc, A, Bt, Ct, rows, cols, kind, slices=1):
+    """Rows `rows` and columns `cols` of the result against the oracle's model of the matrix core
+    (every instruction in its measured arithmetic, K slices folded in double precision as the
+    library folds them): the same bits at full size as in the small tests."""
+    r = torch.as_tensor(rows, device=A.device)
+    c = torch.as_tensor(cols, device=A.device)
+    a, bt = A[r].cpu().numpy(), Bt[c].cpu().numpy()
+    got = np.ascontiguousarray(Ct[c][:, r].cpu().numpy().T)
+    k = a.shape[1]
+    stages = (k + 31) // 32
+    per = -(-stages // slices)
+    total = np.zeros(got.shape, np.float64)
+    for s0 in range(0, stages, per):
+        ka, kb = 32 * s0, min(k, 32 * (s0 + per))
+        part = orc.tcec_matmul(np.ascontiguousarray(a[:, ka:kb]), np.ascontiguousarray(bt[:, ka:kb].T), kind=kind,
+                               ec=True, fk=32, main_outside=False, hw_model=True)
+        if slices == 1:
+            return bool(np.array_equal(got.view(np.uint32), part.view(np.uint32)))
+        total += part.astype(np.float64)
+    return bool(np.array_equal(got.view(np.uint32), total.astype(np.float32).view(np.uint32)))
+
+
 def test_config3_4096_fp16_ec(tc, orc, dev):
     """M=N=K=4096, A row-major, B col-major, uniform[-1,1], alpha=1, beta=0."""
     n = 4096
@@ -44,6 +66,7 @@ def test_config3_4096_fp16_ec(tc, orc, dev):
     err, e32, fro = _check_rows(orc, A, Bt, Ct, 128)
     assert err <= 2 * e32, (err, e32)
     assert fro < 5e-7
+    assert _same_bits_as_the_model(orc, A, Bt, Ct, [0, 1777, 4095], list(range(0, n, 3)), orc.SPLIT_F16)
     # without error correction the same product is ~1000x less accurate (the gate has teeth)
     C0 = tc.matmul_tn(A, Bt, tc.Policy.F16_NOEC)
     err0, _, _ = _check_rows(orc, A, Bt, C0, 16)
@@ -64,6 +87,7 @@ def test_config4_16384_bf16_three_terms(tc, orc, dev):
     err, e32, fro = _check_rows(orc, A, Bt, Ct, 48)
     assert err <= 2 * e32, (err, e32)
     assert fro < 1e-6
+    assert _same_bits_as_the_model(orc, A, Bt, Ct, [5, 16383], list(range(1, n, 17)), orc.SPLIT_BF16X3)
     # linearity in a power of two: (2A) B == 2 (A B) bit for bit (bf16 terms scale exactly)
     C2 = tc.matmul_tn(A * 2, Bt, tc.Policy.BF16X3_EC, workspace=ws)
     assert torch.equal(C2, Ct * 2)
@@ -88,6 +112,8 @@ def test_config5a_strided_batched_256(tc, orc, dev):
         c = np.ascontiguousarray(Ct[b].cpu().numpy().T)
         c32 = orc.gemm_f32(A[b].cpu().numpy(), Bt[b].cpu().numpy().T)
         assert orc.max_rel_err(c, ref) <= 2 * orc.max_rel_err(c32, ref)
+    for b in (2, 1022):
+        assert _same_bits_as_the_model(orc, A[b], Bt[b], Ct[b], list(range(n)), list(range(n)), orc.SPLIT_F16)
     # every batch entry equals the same product done alone
     for b in (3, 700):
         assert torch.equal(Ct[b], tc.matmul_tn(A[b].contiguous(), Bt[b].contiguous(), tc.Policy.F16_EC))
@@ -104,6 +130,9 @@ def test_config5b_k_heavy(tc, orc, dev):
     assert err <= 2 * e32, (err, e32)
     # the sequential fp32 loop loses ~sqrt(K) ulps here; TCEC stays well below it
     assert err < e32
+    slices = tc.sgemm_k_slices(m, m, k, 1, tc.Policy.F16_EC, 0)
+    assert slices > 1
+    assert _same_bits_as_the_model(orc, A, Bt, Ct, [0, 1023], list(range(0, m, 8)), orc.SPLIT_F16, slices)
 
 
 def test_reference_harness_command_prints_the_reference_csv(tc, orc, dev):
