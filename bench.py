@@ -252,7 +252,38 @@ def bench_primitives(args, torch, tcec, dev, w, steps=None, warmup=None, cpu=Non
     return res
 
 
-def accuracy_block(torch, tcec, orc, A, Bt, Ct, rows):
+POLICY_MODEL = {"F16_EC": (0, True), "F16_NOEC": (0, False), "BF16X3_EC": (2, True), "BF16X2_EC": (1, True),
+                "BF16_NOEC": (1, False)}
+
+
+def model_bits_block(orc, a, bt, c, policy_name, slices):
+    """Two of the sampled rows, every 16th column: the result against the oracle's model of the
+    matrix core (each MFMA in its measured arithmetic, in the driver's order; K slices folded in
+    double precision as the library folds them).  The model gives the library's bits, so this
+    reads true or names the number of differing elements."""
+    import numpy as np
+    kind, ec = POLICY_MODEL[policy_name]
+    a2, bt2 = np.ascontiguousarray(a[:2]), np.ascontiguousarray(bt[::16])
+    got = np.ascontiguousarray(c[:2, ::16])
+    k = a2.shape[1]
+    stages = (k + 31) // 32
+    per = -(-stages // max(slices, 1))
+    total = np.zeros(got.shape, np.float64)
+    for s0 in range(0, stages, per):
+        ka, kb = 32 * s0, min(k, 32 * (s0 + per))
+        ap = np.zeros((2, 32 * (-(-(kb - ka) // 32))), np.float32)
+        bp = np.zeros((ap.shape[1], bt2.shape[0]), np.float32)
+        ap[:, :kb - ka], bp[:kb - ka, :] = a2[:, ka:kb], bt2[:, ka:kb].T
+        part = orc.tcec_matmul(ap, bp, kind=kind, ec=ec, fk=32, main_outside=False, hw_model=True)
+        total = part if slices <= 1 else total + part.astype(np.float64)
+    want = np.ascontiguousarray(total.astype(np.float32))
+    differing = int((got.view(np.uint32) != want.view(np.uint32)).sum())
+    return {"equal": differing == 0, "differing": differing, "elements": int(got.size), "k_slices": int(slices),
+            "what": "2 sampled rows x every 16th column of C against the oracle's bit-level model of the "
+                    "gfx950 matrix core in the driver's instruction order"}
+
+
+def accuracy_block(torch, tcec, orc, A, Bt, Ct, rows, model=None):
     """max|C - C64| / max|C64| on `rows` seeded full rows of batch 0 for the TCEC result and for
     three plain fp32 products of the same rows: the oracle's sequential CPU loop, the vendor's
     fp32 GEMM on the GPU and this library's fp32 policy (the API-level GEMM on the matrix core's
@@ -283,7 +314,11 @@ def accuracy_block(torch, tcec, orc, A, Bt, Ct, rows):
         tcec.api_gemm(3, 0, rows, n, k, 1.0, a_rows, k, Bt[0], k, 0.0, out, rows)
         torch.cuda.synchronize()
         plain["fp32_policy_api_gemm_gpu"] = orc.max_rel_err(np.ascontiguousarray(out.cpu().numpy().T), ref)
+    extra = {}
+    if model is not None:
+        extra["same_bits_as_matrix_core_model"] = model_bits_block(orc, a, bt, np.ascontiguousarray(c), *model)
     return {
+        **extra,
         "max_rel_err_vs_fp64": float(f"{err:.4e}"),
         "plain_fp32_max_rel_err_vs_fp64": float(f"{plain['cpu_loop']:.4e}"),
         "plain_fp32_comparators": {k_: float(f"{v:.4e}") for k_, v in plain.items()},
@@ -451,7 +486,11 @@ def run_gemm_workload(args, torch, tcec, dev, name, steps, warmup):
                     "100 MHz counter; the timed region is delimited by two stamps on the work stream"}
     if not args.no_accuracy:
         from oracle import oracle as orc
-        out.update(accuracy_block(torch, tcec, orc, A, Bt, Ct, 128 if k >= 8192 else 256))
+        slices = tcec.sgemm_k_slices(m, n, k, batch, policy, flags & 14)
+        # (the tiles of a partly empty last round may be cut into K slices of their own: not modelled here)
+        tail = packed and slices == 1 and ws_bytes > 0
+        out.update(accuracy_block(torch, tcec, orc, A, Bt, Ct, 128 if k >= 8192 else 256,
+                                  model=None if tail or (flags & 1) else (w["policy"], slices)))
     return out, w
 
 
