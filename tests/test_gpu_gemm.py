@@ -135,6 +135,33 @@ def test_sgemm_wide_exponent_range_same_bits_as_the_model(tc, orc, dev, policy, 
 
 
 @pytest.mark.parametrize("policy", [0, 2])
+@pytest.mark.parametrize("mnk", [(200, 136, 328), (512, 256, 160), (520, 392, 1000), (64, 64, 32)])
+def test_sgemm_rn_main_flag_same_bits_as_the_model(tc, orc, dev, policy, mnk):
+    """WMMAE_FLAG_RN_MAIN: the leading product of every 32 of k starts from zero on the matrix
+    core and is added with an fp32 add outside it (the reference's mma_rn_sync,
+    tcec/tcec.hpp:673-694); the error products stay chained.  The oracle's model in that order
+    gives the bits, on the packed path, the single kernel and the library's choice, with alpha
+    and beta too."""
+    m, n, k = mnk
+    kind, ec = POL_KIND[policy]
+    rng = np.random.default_rng(m + 3 * n + k + policy)
+    A = rng.uniform(-1, 1, (m, k)).astype(np.float32)
+    B = rng.uniform(-1, 1, (k, n)).astype(np.float32)
+    C = rng.uniform(-1, 1, (m, n)).astype(np.float32)
+    emu = orc.tcec_matmul(A, B, kind=kind, ec=ec, fk=32, main_outside=True, hw_model=True)
+    chained = orc.tcec_matmul(A, B, kind=kind, ec=ec, fk=32, main_outside=False, hw_model=True)
+    if k > 32:
+        assert not np.array_equal(emu, chained)                  # the flag does change the bits
+    for path_flag in (0, 2, 4):
+        if tc.sgemm_k_slices(m, n, k, 1, policy, 1 | path_flag) > 1:
+            continue
+        D = _gemm(tc, dev, A, B, policy, flags=1 | path_flag)
+        assert np.array_equal(D.view(np.uint32), emu.view(np.uint32)), (path_flag, int((D != emu).sum()))
+        D = _gemm(tc, dev, A, B, policy, alpha=-0.75, beta=1.5, C=C, flags=1 | path_flag)
+        assert np.array_equal(D.view(np.uint32), orc.epilogue(emu, -0.75, 1.5, C).view(np.uint32)), path_flag
+
+
+@pytest.mark.parametrize("policy", [0, 2])
 @pytest.mark.parametrize("mnk", [(1, 1, 1), (17, 5, 3), (100, 37, 77), (129, 255, 33), (300, 200, 100),
                                  (16, 16, 1000), (1000, 3, 8), (700, 37, 77), (130, 1031, 45)])
 def test_sgemm_ragged_shapes(tc, orc, dev, policy, mnk):
