@@ -88,7 +88,7 @@ def test_random_products_on_every_path(tc, dev, seed):
             assert torch.equal(res[DIRECT], res[PACKED]), c
 
 
-def test_tail_slices_are_the_only_difference_on_a_large_single_product(tc, dev):
+def test_tail_slices_are_the_only_difference_on_a_large_single_product(tc, orc, dev):
     """2293 x 1802 x 5518: the packed path, given room for them, cuts K for the tiles of its partly
     empty last round, and those tiles come out with other last bits; with a workspace that only
     holds the packed operands it gives the bits of the direct and of the single kernel, with
@@ -115,3 +115,42 @@ def test_tail_slices_are_the_only_difference_on_a_large_single_product(tc, dev):
         assert 0 < differing < m * n // 4
         scale = out["packed"].abs().max().item()
         assert (out["tail"] - out["packed"]).abs().max().item() < 1e-5 * scale
+        if (alpha, beta) == (1.0, 0.0):
+            _tail_tiles_follow_the_model(orc, A, B, out["packed"], out["tail"], k)
+
+
+def _tail_tiles_follow_the_model(orc, A, B, whole, cut, k):
+    """Sampled rows of the two results above against the oracle's model of the matrix core: the
+    uncut run is the model over all of k; an element of the cut run is either that or the model
+    over K slices of equal whole stages (2 .. 16 of them, one count for the whole product), the
+    slices added in double precision - and both kinds occur (the cut tiles are the last of the
+    walk through the tile grid: the bottom rows of C)."""
+    import numpy as np
+    m = A.shape[0]
+    rows = [0, 777, m - 300, m - 130, m - 2, m - 1]
+    a = A[rows].cpu().numpy()
+    bt = B.cpu().numpy()
+    got_whole = np.ascontiguousarray(whole[:, rows].cpu().numpy().T)
+    got_cut = np.ascontiguousarray(cut[:, rows].cpu().numpy().T)
+
+    def model(ka, kb):
+        ap = np.zeros((len(rows), 32 * (-(-(kb - ka) // 32))), np.float32)
+        bp = np.zeros((ap.shape[1], bt.shape[0]), np.float32)
+        ap[:, :kb - ka], bp[:kb - ka, :] = a[:, ka:kb], bt[:, ka:kb].T
+        return orc.tcec_matmul(ap, bp, kind=orc.SPLIT_F16, ec=True, fk=32, main_outside=False, hw_model=True)
+    full = model(0, k)
+    assert np.array_equal(got_whole.view(np.uint32), full.view(np.uint32))
+    other = got_cut.view(np.uint32) != full.view(np.uint32)
+    assert other.any() and not other.all()
+    stages = (k + 31) // 32
+    explained = []
+    for count in range(2, 17):
+        per = -(-stages // count)
+        if -(-stages // per) != count:
+            continue
+        total = np.zeros(full.shape, np.float64)
+        for s0 in range(0, stages, per):
+            total += model(32 * s0, min(k, 32 * (s0 + per))).astype(np.float64)
+        if np.array_equal(got_cut.view(np.uint32)[other], total.astype(np.float32).view(np.uint32)[other]):
+            explained.append(count)
+    assert len(explained) >= 1, "no slice count explains the cut tiles"
