@@ -312,6 +312,16 @@ int wmmae_tcec_api_gemm(int type, int ec, int m, int n, int k,
                         const float *alpha, const float *A, int lda,
                         const float *B, int ldb, const float *beta, float *C,
                         int ldc, void *stream);
+/* The same kernel with the product of every k step issued by tcec::mma_sync
+ * (rounding 0, as above), mma_rn_sync (1) or mma_rz_sync (2)
+ * (tcec/tcec.hpp:640-706, 773-831, 896-927).  On gfx950 the matrix core
+ * accumulates with round-to-nearest-even, so the chained variant is as accurate
+ * as the reference's default and faster. */
+int wmmae_tcec_api_gemm_rounding(int type, int ec, int rounding, int m, int n,
+                                 int k, const float *alpha, const float *A,
+                                 int lda, const float *B, int ldb,
+                                 const float *beta, float *C, int ldc,
+                                 void *stream);
 /* The same kernel on device arrays of `batch` matrix pointers (each 16-byte
  * aligned), the calling convention of the reference's launch_bgemm
  * (test/tcec/batch_gemm.cu:433-443). */

@@ -431,6 +431,17 @@ def test_api_level_gemm_matches_driver(tc, orc, dev, type_ec):
         # of the same sums
         drv = _gemm(tc, dev, A, Bt.T, policy, alpha=alpha, beta=beta, C=C0)
         assert np.abs(got - drv).max() <= 16 * 2.0**-24 * max(1.0, np.abs(ref).max())
+        # the kernel with mma_rn_sync / mma_rz_sync in place of mma_sync: the model in that order
+        if (alpha, beta) == (1.0, 0.0):
+            for rounding in (1, 2):
+                dC = torch.zeros((n, m), dtype=torch.float32, device=dev)
+                tc.api_gemm(type_, ec, m, n, k, 1.0, dA, k, dB, k, 0.0, dC, m, rounding=rounding)
+                torch.cuda.synchronize()
+                emu_r = orc.tcec_matmul(A, Bt.T, kind=POL_KIND[policy][0], ec=bool(ec), fk=32,
+                                        main_outside=rounding == 1, hw_model=True)
+                assert np.array_equal(dC.cpu().numpy().T.view(np.uint32), emu_r.view(np.uint32)), rounding
+            # (chained, it gives the driver's bits)
+            assert np.array_equal(dC.cpu().numpy().T, drv)
     from wmma_extension_amd._lib import WmmaeError
     with pytest.raises(WmmaeError) as e:
         tc.api_gemm(type_, ec, 100, n, k, 1.0, dA, k, dB, k, 0.0, dC, 100)

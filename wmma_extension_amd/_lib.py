@@ -49,6 +49,7 @@ EXPORTS = [
     "wmmae_tcec_frag_dump",
     "wmmae_tcec_elementwise",
     "wmmae_tcec_api_gemm",
+    "wmmae_tcec_api_gemm_rounding",
     "wmmae_tcec_api_gemm_batched",
     "wmmae_tcec_mma_complex",
     "wmmae_primitive_mma",
@@ -155,6 +156,7 @@ _SIGNATURES = {
     "wmmae_tcec_frag_dump": (_i, [_i, _i, _i, _i, _vp, _vp, _i, _i, _vp]),
     "wmmae_tcec_elementwise": (_i, [_i, _i, _i, _vp, _c.c_float, _i, _i, _vp]),
     "wmmae_tcec_api_gemm": (_i, [_i, _i, _i, _i, _i, _fp, _vp, _i, _vp, _i, _fp, _vp, _i, _vp]),
+    "wmmae_tcec_api_gemm_rounding": (_i, [_i, _i, _i, _i, _i, _i, _fp, _vp, _i, _vp, _i, _fp, _vp, _i, _vp]),
     "wmmae_tcec_api_gemm_batched": (_i, [_i, _i, _i, _i, _i, _fp, _vp, _i, _vp, _i, _fp, _vp, _i, _i, _vp]),
     "wmmae_tcec_mma_complex": (_i, [_i, _i, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _c.c_float, _vp]),
     "wmmae_primitive_mma": (_i, [_i, _i, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _vp]),

@@ -15,11 +15,11 @@ int api_gemm_impl(const int type, const int ec, const int m, const int n,
                   const long long stride_b, const float *const beta,
                   float *const C, float *const *const c_ptrs, const int ldc,
                   const long long stride_c, const int batch,
-                  void *const stream) {
+                  void *const stream, const int rounding = 0) {
   using S = wmmae_harness::ApiGemmShape;
   if (!alpha || !beta || (!A && !a_ptrs) || (!B && !b_ptrs) || (!C && !c_ptrs))
     return WMMAE_STATUS_NULL_POINTER;
-  if (m <= 0 || n <= 0 || k <= 0 || batch < 0)
+  if (m <= 0 || n <= 0 || k <= 0 || batch < 0 || rounding < 0 || rounding > 2)
     return WMMAE_STATUS_INVALID_VALUE;
   if (lda < k || ldb < k || ldc < m)
     return WMMAE_STATUS_BAD_LEADING_DIM;
@@ -47,15 +47,26 @@ int api_gemm_impl(const int type, const int ec, const int m, const int n,
     return with_ec(ec, [&](auto te) -> int {
       using EC = typename decltype(te)::type;
       using P = typename harness_policy<T, EC, 16, 16, 32>::type;
-      auto kernel = wmmae_harness::tcec_api_gemm_kernel<T, P, 2>;
-      static std::atomic<unsigned long long> lds_allowed{0};
-      WMMAE_HIP_TRY(allow_dynamic_lds(reinterpret_cast<const void *>(kernel),
-                                      S::LDS_BYTES, lds_allowed));
-      hipLaunchKernelGGL(kernel, dim3(static_cast<unsigned>(blocks)),
-                         dim3(S::THREADS), S::LDS_BYTES, s, m, n, k, al, A,
-                         a_ptrs, lda, stride_a, B, b_ptrs, ldb, stride_b, be, C,
-                         c_ptrs, ldc, stride_c);
-      return launch_status();
+      const auto launch = [&](auto rr) -> int {
+        auto kernel =
+            wmmae_harness::tcec_api_gemm_kernel<T, P, 2, decltype(rr)::value>;
+        static std::atomic<unsigned long long> lds_allowed{0};
+        WMMAE_HIP_TRY(allow_dynamic_lds(reinterpret_cast<const void *>(kernel),
+                                        S::LDS_BYTES, lds_allowed));
+        hipLaunchKernelGGL(kernel, dim3(static_cast<unsigned>(blocks)),
+                           dim3(S::THREADS), S::LDS_BYTES, s, m, n, k, al, A,
+                           a_ptrs, lda, stride_a, B, b_ptrs, ldb, stride_b, be,
+                           C, c_ptrs, ldc, stride_c);
+        return launch_status();
+      };
+      switch (rounding) {
+      case 1:
+        return launch(std::integral_constant<int, 1>{});
+      case 2:
+        return launch(std::integral_constant<int, 2>{});
+      default:
+        return launch(std::integral_constant<int, 0>{});
+      }
     });
   });
 }
@@ -71,6 +82,17 @@ int wmmae_tcec_api_gemm(const int type, const int ec, const int m, const int n,
                         void *const stream) {
   return api_gemm_impl(type, ec, m, n, k, alpha, A, nullptr, lda, 0, B, nullptr,
                        ldb, 0, beta, C, nullptr, ldc, 0, 1, stream);
+}
+
+int wmmae_tcec_api_gemm_rounding(const int type, const int ec,
+                                 const int rounding, const int m, const int n,
+                                 const int k, const float *const alpha,
+                                 const float *const A, const int lda,
+                                 const float *const B, const int ldb,
+                                 const float *const beta, float *const C,
+                                 const int ldc, void *const stream) {
+  return api_gemm_impl(type, ec, m, n, k, alpha, A, nullptr, lda, 0, B, nullptr,
+                       ldb, 0, beta, C, nullptr, ldc, 0, 1, stream, rounding);
 }
 
 int wmmae_tcec_api_gemm_batched(const int type, const int ec, const int m,

@@ -82,7 +82,9 @@ __device__ __forceinline__ void stage_tile(float *const dst,
 // one batch entry.  A: m x k row-major (lda), B: k x n column-major (ldb), C:
 // m x n column-major (ldc); m, n multiples of 128, k of 32; batch entry y at
 // base + y*stride or, when the pointer arrays are set, at ptrs[y].
-template <class T, class Policy, int WAVES_PER_SIMD>
+// ROUNDING: 0 tcec::mma_sync (the reference's default for the policy), 1
+// mma_rn_sync, 2 mma_rz_sync.
+template <class T, class Policy, int WAVES_PER_SIMD, int ROUNDING = 0>
 __global__ void __launch_bounds__(ApiGemmShape::THREADS, WAVES_PER_SIMD)
     tcec_api_gemm_kernel(const int m, const int n, const int k,
                          const float alpha, const float *const A,
@@ -128,6 +130,14 @@ __global__ void __launch_bounds__(ApiGemmShape::THREADS, WAVES_PER_SIMD)
       tcec::fragment<w::accumulator, S::WM, S::WN, S::WK, T, void, Policy>;
   FragC fc;
   tcec::fill_zero(fc);
+  const auto mma = [](FragC &d, const FragA &a, const FragB &b) {
+    if constexpr (ROUNDING == 1)
+      tcec::mma_rn_sync(d, a, b, d);
+    else if constexpr (ROUNDING == 2)
+      tcec::mma_rz_sync(d, a, b, d);
+    else
+      tcec::mma_sync(d, a, b, d);
+  };
 
   auto stage_in = [&](const int stage, const int k0) {
     float *const sa = smem + stage * S::STAGE_FLOATS;
@@ -165,10 +175,10 @@ __global__ void __launch_bounds__(ApiGemmShape::THREADS, WAVES_PER_SIMD)
                                                        false);
       tcec::load_matrix_sync<tcec::col_major_swizzled>(fb[cur], sb + kk, S::LD,
                                                        false);
-      tcec::mma_sync(fc, fa[1 - cur], fb[1 - cur], fc);
+      mma(fc, fa[1 - cur], fb[1 - cur]);
     }
     constexpr int last = ((S::SK / S::WK) - 1) & 1;
-    tcec::mma_sync(fc, fa[last], fb[last], fc);
+    mma(fc, fa[last], fb[last]);
 
     cpa::wait_all();
     __syncthreads();

@@ -343,13 +343,19 @@ def elementwise(type_, ec, inst, base, do_neg, do_integrate, device="cuda"):
     return out
 
 
-def api_gemm(type_, ec, m, n, k, alpha, A, lda, B, ldb, beta, C, ldc):
-    """Tiled GEMM written against the public device API only."""
+def api_gemm(type_, ec, m, n, k, alpha, A, lda, B, ldb, beta, C, ldc, rounding=0):
+    """Tiled GEMM written against the public device API only (rounding: 0 tcec::mma_sync,
+    1 mma_rn_sync, 2 mma_rz_sync)."""
     _need_cuda(A, B, C)
     _check_gemm_operands("T", "N", m, n, k, A, lda, B, ldb, C, ldc)
-    st = _lib.lib().wmmae_tcec_api_gemm(type_, int(ec), m, n, k, _f(alpha), _ptr(A), lda, _ptr(B), ldb,
-                                        _f(beta), _ptr(C), ldc, _stream())
-    _lib.check(st, "wmmae_tcec_api_gemm")
+    if rounding == 0:
+        st = _lib.lib().wmmae_tcec_api_gemm(type_, int(ec), m, n, k, _f(alpha), _ptr(A), lda, _ptr(B), ldb,
+                                            _f(beta), _ptr(C), ldc, _stream())
+        _lib.check(st, "wmmae_tcec_api_gemm")
+        return
+    st = _lib.lib().wmmae_tcec_api_gemm_rounding(type_, int(ec), int(rounding), m, n, k, _f(alpha), _ptr(A), lda,
+                                                 _ptr(B), ldb, _f(beta), _ptr(C), ldc, _stream())
+    _lib.check(st, "wmmae_tcec_api_gemm_rounding")
 
 
 def api_gemm_batched(type_, ec, m, n, k, alpha, A_array, lda, B_array, ldb, beta, C_array, ldc, batch):
