@@ -13,8 +13,8 @@ ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
 INCLUDE = os.path.join(ROOT, "include")
 HIPCC = os.environ.get("HIPCC", "/opt/rocm/bin/hipcc")
 
-# the reference's headers for this path (its per-architecture NVIDIA tables sm_*.hpp, m16n8k*.hpp
-# and the simt/ emulation directory have no counterpart: one layout model serves gfx950)
+# the reference's headers for this path (its per-architecture NVIDIA tables sm_*.hpp and
+# m16n8k*.hpp have no counterpart: one layout model serves gfx950)
 HEADERS = [
     "wmma_extension/wmma_extension.hpp",
     "wmma_extension/wmma_mma.hpp",
@@ -34,7 +34,45 @@ HEADERS = [
     "wmma_extension/tcec/detail/notc.hpp",
     "wmma_extension/tcec/detail/print.hpp",
     "wmma_extension/tcec/detail/wmma_extension_include.hpp",
+    "wmma_extension/tcec/detail/wmma_extension_simt_include.hpp",
+    "wmma_extension/tcec/detail/simt/mma_simt.hpp",
+    "wmma_extension/tcec/detail/simt/detail/common.hpp",
+    "wmma_extension/tcec/detail/simt/detail/fma.hpp",
+    "wmma_extension/tcec/detail/simt/detail/m16n16k16.hpp",
 ]
+
+# the fragment namespace behind the reference's op_simt policy, used directly
+# (reference: tcec/detail/simt/mma_simt.hpp:9-262, simt/detail/fma.hpp:10-24)
+MMA_SIMT = r"""
+#include <hip/hip_runtime.h>
+#include <wmma_extension/tcec/detail/wmma_extension_simt_include.hpp>
+#include <type_traits>
+namespace w = mtk::wmma;
+namespace s = mtk::wmma::mma_simt;
+using frag_a = s::fragment<w::matrix_a, 16, 16, 16, float, w::row_major>;
+using frag_b = s::fragment<w::matrix_b, 16, 16, 16, float, w::col_major>;
+using frag_c = s::fragment<w::accumulator, 16, 16, 16, float>;
+static_assert(std::is_same<frag_a, w::fragment<w::matrix_a, 16, 16, 16, float, w::row_major>>::value, "");
+__global__ void k(float *d, const float *a, const float *b, const float *c, float *v) {
+  frag_a fa;
+  frag_b fb;
+  frag_c fc, fd;
+  s::load_matrix_sync(fa, a, 16);
+  s::load_matrix_sync(fb, b, 16);
+  s::load_matrix_sync(fc, c, 16, w::mem_col_major);
+  s::mma_sync(fd, fa, fb, fc);
+  s::foreach_ij<frag_c>(w::mem_col_major, [&](const unsigned *list, const unsigned n, const unsigned i,
+                                              const unsigned j) {
+    for (unsigned x = 0; x < n; x++)
+      fd.x[list[x]] += s::detail::fma<float, float, float>{}(float(i), float(j), 1.f);
+  });
+  s::store_matrix_sync(d, fd, 16, w::mem_col_major);
+  s::fill_zero(fa);
+  s::load_vector(fa, v);
+  s::store_vector(v, fd, w::mem_col_major);
+  v[20] = float(s::detail::fma<double, double, double>{}(1.0, 2.0, 3.0));
+}
+"""
 
 DETAIL_NAMES = r"""
 #include <hip/hip_runtime.h>
@@ -101,6 +139,11 @@ def test_every_reference_include_path_compiles_alone():
         results = list(pool.map(_syntax_only, sources))
     bad = [(h, out[-2000:]) for h, (rc, out) in zip(HEADERS, results) if rc != 0]
     assert not bad, bad
+
+
+def test_mma_simt_namespace_compiles_against_the_reference_spelling():
+    rc, out = _syntax_only(MMA_SIMT)
+    assert rc == 0, out[-4000:]
 
 
 def test_detail_names_of_the_reference_are_there():
