@@ -1,7 +1,7 @@
 """Seeded random products through every path of the driver against the oracle's model of the
 matrix core, bit for bit: shapes that are no multiples of anything (k from 1 on), every policy,
-alpha / beta, padded leading dimensions, the round-to-nearest flag, K slices where the driver
-cuts K.  Expected = every slice in the model (k padded with zeros to whole stages of 32, as the
+alpha / beta, all four transpose combinations, padded leading dimensions, the round-to-nearest
+flag, K slices where the driver cuts K.  Expected = every slice in the model (k padded with zeros to whole stages of 32, as the
 kernels pad), slices added in double precision in ascending order, then the epilogue
 (alpha, one fused multiply-add of beta * C)."""
 import random
@@ -48,14 +48,18 @@ def test_random_products_have_the_bits_of_the_model(tc, orc, dev, seed):
         alpha, beta = rnd.choice([(1.0, 0.0), (1.0, 0.0), (-0.75, 1.5), (2.5, -1.0)])
         pad = rnd.choice([0, 0, 1, 4])
         rn = rnd.random() < 0.2 and policy in (0, 2)
+        ta, tb = rnd.choice([("T", "N")] * 3 + [("N", "N"), ("N", "T"), ("T", "T")])
         kind, ec = POL_KIND[policy]
         A = rng.uniform(-1, 1, (m, k)).astype(np.float32)
         B = rng.uniform(-1, 1, (k, n)).astype(np.float32)
         C = rng.uniform(-1, 1, (m, n)).astype(np.float32)
-        dA = torch.zeros((m, k + pad), device=dev)
-        dB = torch.zeros((n, k + pad), device=dev)
-        dA[:, :k] = torch.from_numpy(A).to(dev)
-        dB[:, :k] = torch.from_numpy(np.ascontiguousarray(B.T)).to(dev)
+        # column-major BLAS storage: op(A) = 'T' keeps A as m rows of k floats, 'N' as k rows of m
+        a_store = A if ta == "T" else np.ascontiguousarray(A.T)
+        b_store = np.ascontiguousarray(B.T) if tb == "N" else B
+        dA = torch.zeros((a_store.shape[0], a_store.shape[1] + pad), device=dev)
+        dB = torch.zeros((b_store.shape[0], b_store.shape[1] + pad), device=dev)
+        dA[:, :a_store.shape[1]] = torch.from_numpy(a_store).to(dev)
+        dB[:, :b_store.shape[1]] = torch.from_numpy(b_store).to(dev)
         models = {}
         for path in (0, PACKED, FUSED, DIRECT):
             flags = path | (1 if rn else 0)
@@ -64,20 +68,21 @@ def test_random_products_have_the_bits_of_the_model(tc, orc, dev, seed):
             ws = torch.empty(max(16, tc.workspace_bytes(m, n, k, 1, policy)), dtype=torch.uint8, device=dev)
             try:
                 slices = tc.sgemm_k_slices(m, n, k, 1, policy, flags)
-                tc.sgemm("T", "N", m, n, k, alpha, dA, k + pad, dB, k + pad, beta, dC, m + pad, policy, flags, ws)
+                tc.sgemm(ta, tb, m, n, k, alpha, dA, dA.shape[1], dB, dB.shape[1], beta, dC, m + pad, policy,
+                         flags, ws)
             except WmmaeError as e:
                 assert e.status == -4 and path in (FUSED, DIRECT), (case, path, e)
                 continue
             torch.cuda.synchronize()
             got = dC.cpu().numpy()
             assert (got[:, m:] == 7.0).all(), (case, path)
-            if path == 0 and pad % 4 != 0:
-                continue            # (the count the query reports holds for tight leading dimensions)
+            if path == 0 and (pad % 4 != 0 or (ta, tb) != ("T", "N")):
+                continue            # (the count the query reports holds for 'T', 'N' and tight leading dimensions)
             if slices not in models:
                 models[slices] = orc.epilogue(_model(orc, A, B, kind, ec, slices, rn), alpha, beta, C)
             want = models[slices]
             D = np.ascontiguousarray(got[:, :m].T)
             assert np.array_equal(D.view(np.uint32), want.view(np.uint32)), \
-                (case, (m, n, k), policy, path, slices, alpha, beta, pad, rn, int((D != want).sum()))
+                (case, (m, n, k), policy, path, slices, alpha, beta, pad, rn, ta, tb, int((D != want).sum()))
             checked += 1
     assert checked >= 80
