@@ -26,7 +26,9 @@
  *   orc_gemm_f64 / _f32        numpy float64 / float32 matmul
  *   orc_fp32_policy_matmul     results recorded from an MI355X (same fixture)
  *                              and an independent restatement in exact
- *                              rational arithmetic
+ *                              rational arithmetic (both variants)
+ *   orc_epilogue               exact rational arithmetic rounded by hand, both
+ *                              forms; beta == 0 never reads C
  *   orc_to_tf32                tie cases written out as literals and a float64
  *                              restatement (scale, floor(x + 1/2), scale back)
  *   orc_mfma_dot / _tile       results recorded from an MI355X for structured
