@@ -35,10 +35,13 @@
  *                              and random bit patterns (tests/golden/
  *                              mfma_kat.npz), the probes 1 + k*2^-24, 2^24 + 3
  *                              and a product 2^25 below the largest as
- *                              literals, sums below 2^-126 (recorded tiles
- *                              and four hand-made products as literals); on
- *                              the GPU, bit equality with fresh raw MFMAs of
- *                              every shape and type
+ *                              literals, sums below 2^-126, sums and products
+ *                              beyond fp32's range, infinite and NaN operands
+ *                              (recorded tiles, hand-made cases as literals);
+ *                              on the GPU, bit equality with fresh raw MFMAs
+ *                              of every shape and type
+ *   orc_max_rel_err / _abs_err / orc_frobenius_residual
+ *                              values written out as literals
  * PARITY UNPINNED: the bit-level result of the reference's hardware MMA
  * (CUDA <mma.h> / PTX mma.sync; summation order and rounding inside the tensor
  * core are not specified and not reproducible on MFMA).  orc_mma_block with
