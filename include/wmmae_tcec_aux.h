@@ -71,6 +71,16 @@ int wmmae_tcec_sgemm_k_slices(int m, int n, int k, int batch, int policy,
 int wmmae_tcec_path_estimates(int m, int n, int k, int batch, int policy,
                               double *seconds);
 
+/* Measurement hook (no counterpart in the reference): the calling thread's
+ * next wmmae_tcec_sgemm* / wmmae_tcec_gemm_packed calls record `begin_event`
+ * on their stream right before the MFMA GEMM kernel of the packed or the direct
+ * path and `end_event` right after it (after the fold of its K slices, where
+ * there is one), so that a caller can time that kernel inside a whole call
+ * (hipEventElapsedTime after the events have completed).  Both hipEvent_t, or
+ * both NULL to switch the hook off.  The single-kernel ("fused") path records
+ * nothing.  The events stay the caller's. */
+int wmmae_tcec_time_gemm_kernel(void *begin_event, void *end_event);
+
 /* Test hook (no counterpart in the reference): the calling thread's next
  * wmmae_tcec_sgemm* / wmmae_tcec_gemm_packed calls and workspace queries cut K
  * into `slices` slices (at most 32, at least six k stages of 32 each: smaller

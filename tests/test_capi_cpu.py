@@ -25,7 +25,7 @@ def test_header_and_library_agree(h):
     declared_aux = set(re.findall(r"\b(wmmae_[a-z0-9_]+)\s*\(", aux))
     # the measurement aids live in their own header, outside the product ABI
     assert declared_aux == {"wmmae_clock_samples", "wmmae_mfma_probe", "wmmae_direct_read_first",
-                            "wmmae_tcec_sgemm_k_slices", "wmmae_tcec_force_k_slices",
+                            "wmmae_tcec_sgemm_k_slices", "wmmae_tcec_force_k_slices", "wmmae_tcec_time_gemm_kernel",
                             "wmmae_tcec_path_estimates", "wmmae_mfma_source_hazard_probe"} and not (declared & declared_aux)
     declared |= declared_aux
     assert declared == set(_lib.EXPORTS)

@@ -513,6 +513,42 @@ def test_k_slices_same_bits_as_the_model(tc, orc, dev, case):
     assert np.array_equal(D.view(np.uint32), emu.view(np.uint32)), int((D.view(np.uint32) != emu.view(np.uint32)).sum())
 
 
+def test_gemm_kernel_events_inside_a_call(tc, dev):
+    """wmmae_tcec_time_gemm_kernel: a call on the packed or the direct path records the caller's
+    two events right around its MFMA GEMM kernel (and the fold of its K slices): the time between
+    them is positive and shorter than the whole call's, which also runs the split pass; the
+    result is the call's usual one; after the block nothing is recorded any more."""
+    m = n = k = 2048
+    g = torch.Generator(device=dev).manual_seed(3)
+    A = torch.rand((m, k), generator=g, device=dev) * 2 - 1
+    B = torch.rand((n, k), generator=g, device=dev) * 2 - 1
+    ws = torch.empty(tc.workspace_bytes(m, n, k, 1, 0), dtype=torch.uint8, device=dev)
+    for flag in (2, 8):
+        C0 = torch.empty((n, m), device=dev)
+        tc.sgemm("T", "N", m, n, k, 1.0, A, k, B, k, 0.0, C0, m, 0, flag, ws)
+        torch.cuda.synchronize()
+        C = torch.empty((n, m), device=dev)
+        e0, e1, w0, w1 = (torch.cuda.Event(enable_timing=True) for _ in range(4))
+        inner, whole = [], []
+        for _ in range(5):
+            w0.record()
+            with tc.timed_gemm_kernel(e0, e1):
+                tc.sgemm("T", "N", m, n, k, 1.0, A, k, B, k, 0.0, C, m, 0, flag, ws)
+            w1.record()
+            torch.cuda.synchronize()
+            inner.append(e0.elapsed_time(e1))
+            whole.append(w0.elapsed_time(w1))
+        assert torch.equal(C, C0)
+        assert 0.0 < min(inner) <= min(whole)
+        if flag == 2:
+            assert min(inner) < 0.95 * min(whole)          # the split pass is outside the two events
+        # outside the block: the events keep their last times
+        before = e0.elapsed_time(e1)
+        tc.sgemm("T", "N", m, n, k, 1.0, A, k, B, k, 0.0, C, m, 0, flag, ws)
+        torch.cuda.synchronize()
+        assert e0.elapsed_time(e1) == before
+
+
 @pytest.mark.parametrize("flag", [2, 8])
 def test_fold_of_k_slices_is_the_same_with_any_layout_of_c(tc, dev, flag):
     """The kernel that adds the K slices takes 16 bytes per access where C allows it and single

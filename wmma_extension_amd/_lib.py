@@ -67,6 +67,7 @@ EXPORTS = [
     "wmmae_direct_read_first",
     "wmmae_tcec_sgemm_k_slices",
     "wmmae_tcec_force_k_slices",
+    "wmmae_tcec_time_gemm_kernel",
     "wmmae_tcec_path_estimates",
     "wmmae_mfma_source_hazard_probe",
 ]
@@ -174,6 +175,7 @@ _SIGNATURES = {
     "wmmae_direct_read_first": (_i, [_i, _i, _i, _i, _c.POINTER(_ll)]),
     "wmmae_tcec_sgemm_k_slices": (_i, [_i, _i, _i, _i, _i, _i, _c.POINTER(_i)]),
     "wmmae_tcec_force_k_slices": (_i, [_i]),
+    "wmmae_tcec_time_gemm_kernel": (_i, [_vp, _vp]),
     "wmmae_tcec_path_estimates": (_i, [_i, _i, _i, _i, _i, _c.POINTER(_c.c_double)]),
     "wmmae_mfma_source_hazard_probe": (_i, [_i, _i, _vp, _vp]),
 }

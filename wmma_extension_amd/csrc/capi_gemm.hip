@@ -365,6 +365,10 @@ inline double split_time(const int terms, const int m, const int n,
 // next calls instead of the estimates' choice, so that two kernels can be run on
 // the same cut of K and compared bit by bit.  0: the estimates choose.
 thread_local int t_forced_k_slices = 0;
+// Measurement hook (wmmae_tcec_time_gemm_kernel): events this thread's calls
+// record on their stream right before the MFMA GEMM kernel and right after it
+// (after the fold of its K slices where there is one).
+thread_local hipEvent_t t_gemm_begin = nullptr, t_gemm_end = nullptr;
 constexpr int kMaxSplits = 32, kMinStagesPerSplit = 6;
 inline int choose_splits(const int terms, const int m, const int n, const int k,
                          const int batch, const bool direct = false) {
@@ -568,6 +572,8 @@ int launch_gemm(const GemmArgs &g) {
       }
     }
   }
+  if (t_gemm_begin != nullptr)
+    WMMAE_HIP_TRY(hipEventRecord(t_gemm_begin, g.stream));
   hipLaunchKernelGGL(kernel, dim3(grid), dim3(Cfg::NTHREADS), Cfg::LDS_BYTES,
                      g.stream, g.a, g.b,
                      g.c, g.m, g.n, KT, rb_a, rb_b, g.ldc, g.alpha, g.beta,
@@ -614,6 +620,8 @@ int launch_gemm(const GemmArgs &g) {
     }
     st = launch_status();
   }
+  if (st == WMMAE_STATUS_SUCCESS && t_gemm_end != nullptr)
+    WMMAE_HIP_TRY(hipEventRecord(t_gemm_end, g.stream));
   return st;
 }
 
@@ -1451,6 +1459,15 @@ int wmmae_tcec_path_estimates(const int m, const int n, const int k,
   seconds[0] = e.fused;
   seconds[1] = e.packed;
   seconds[2] = e.direct;
+  return WMMAE_STATUS_SUCCESS;
+}
+
+int wmmae_tcec_time_gemm_kernel(void *const begin_event,
+                                void *const end_event) {
+  if ((begin_event == nullptr) != (end_event == nullptr))
+    return WMMAE_STATUS_NULL_POINTER;
+  t_gemm_begin = static_cast<hipEvent_t>(begin_event);
+  t_gemm_end = static_cast<hipEvent_t>(end_event);
   return WMMAE_STATUS_SUCCESS;
 }
 

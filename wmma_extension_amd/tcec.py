@@ -135,6 +135,29 @@ def path_estimates(m, n, k, batch=1, policy=Policy.F16_EC):
     return tuple(out)
 
 
+class timed_gemm_kernel:
+    """Within the block, this thread's packed- and direct-path calls record `begin` / `end`
+    (torch.cuda.Event with timing) right before and after their MFMA GEMM kernel:
+    begin.elapsed_time(end) after a synchronisation is that kernel's time inside the whole call."""
+
+    def __init__(self, begin, end):
+        self.begin, self.end = begin, end
+
+    def __enter__(self):
+        # (a torch event gets its handle at its first record)
+        for e in (self.begin, self.end):
+            if not e.cuda_event:
+                e.record()
+        _lib.check(_lib.lib().wmmae_tcec_time_gemm_kernel(ctypes.c_void_p(self.begin.cuda_event),
+                                                          ctypes.c_void_p(self.end.cuda_event)),
+                   "wmmae_tcec_time_gemm_kernel")
+        return self
+
+    def __exit__(self, *exc):
+        _lib.lib().wmmae_tcec_time_gemm_kernel(None, None)
+        return False
+
+
 class forced_k_slices:
     """Test aid: within the block, this thread's GEMM calls cut K into `slices` slices."""
 
