@@ -2,11 +2,12 @@
 """Benchmark of the TCEC SGEMM hot path on one MI355X.
 
 One "step" = one full product C = A*B on synthetic seeded fp32 inputs that are
-already resident in HBM, run on the path the library's time estimates choose
-for the shape: split+pack of A, split+pack of B and the MFMA GEMM on the packed
-path (large single products, the headline workload), or the one kernel that
-splits the fp32 operands itself (batches of medium-sized matrices, K-heavy
-products).  The workspace is allocated once, outside the timed region.
+already resident in HBM: one call of the library's SGEMM entry point, on the
+path its time estimates choose for the shape - the split+pack of both operands
+and the MFMA GEMM on the packed path (large single products, the headline
+workload), or the one kernel that splits the fp32 operands itself (batches of
+medium-sized matrices, K-heavy products).  The workspace is allocated once,
+outside the timed region.
 
 Prints ONE JSON line: effective fp32 TFLOPS (2*M*N*K*batch / t), the MFMA
 roofline of the GEMM kernel measured with HIP events inside the timed region,
